@@ -1,0 +1,49 @@
+// dsx_device.h — device-side helpers shared by the kernels of libdsx_hip.so (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+#include "dsx.h"
+
+namespace dsx {
+
+constexpr int kWave = 64;
+
+// Activation functions of engine/kActivation.cu:46-153, applied in the epilogue of the producing kernel.
+template <int ACT>
+__device__ __forceinline__ float activate(float x, float slope, float alpha, float lambda)
+{
+    if constexpr (ACT == DSX_ACT_SIGMOID) {
+        return 1.0f / (1.0f + __expf(-x));
+    } else if constexpr (ACT == DSX_ACT_TANH) {
+        return tanhf(x);
+    } else if constexpr (ACT == DSX_ACT_RELU) {
+        return fmaxf(0.0f, x);
+    } else if constexpr (ACT == DSX_ACT_LRELU) {
+        return fmaxf(x, x * slope);
+    } else if constexpr (ACT == DSX_ACT_ELU) {
+        return (x > 0.0f) ? x : alpha * (__expf(x) - 1.0f);
+    } else if constexpr (ACT == DSX_ACT_SELU) {
+        return (x > 0.0f) ? lambda * x : lambda * alpha * (__expf(x) - 1.0f);
+    } else {
+        return x;
+    }
+}
+
+__device__ __forceinline__ float activate_rt(float x, uint32_t act, float slope, float alpha, float lambda)
+{
+    switch (act) {
+    case DSX_ACT_SIGMOID: return activate<DSX_ACT_SIGMOID>(x, slope, alpha, lambda);
+    case DSX_ACT_TANH: return activate<DSX_ACT_TANH>(x, slope, alpha, lambda);
+    case DSX_ACT_RELU: return activate<DSX_ACT_RELU>(x, slope, alpha, lambda);
+    case DSX_ACT_LRELU: return activate<DSX_ACT_LRELU>(x, slope, alpha, lambda);
+    case DSX_ACT_ELU: return activate<DSX_ACT_ELU>(x, slope, alpha, lambda);
+    case DSX_ACT_SELU: return activate<DSX_ACT_SELU>(x, slope, alpha, lambda);
+    default: return x;
+    }
+}
+
+// CalculateActivation (engine/NNLayer.cpp:1646-1683) runs a kernel only for sigmoid, tanh, ReLU, leaky ReLU, ELU, SELU and
+// softmax; every other ordinal leaves the unit buffer as it is.  Softmax is a row operation with its own kernel.
+inline bool is_elementwise_activation(uint32_t act) { return act != DSX_ACT_SOFTMAX; }
+
+}  // namespace dsx

@@ -1,0 +1,410 @@
+// dsx_fc.hip — dense forward of a fully connected layer: fp32 MFMA GEMM with bias, accumulate and activation fused in the
+// epilogue, plus the stand-alone activation kernels.
+//
+// GEMM: Z[B x n] = act(acc? Z : 0 + bias + X[B x k] . W[k x n]).  A 256-lane workgroup (2 x 2 wavefronts) owns a
+// (64*MI) x (64*NI) tile of Z; each wavefront keeps MI x NI accumulators of v_mfma_f32_32x32x2_f32 (32 x 32 fp32 each) in
+// registers.  X and W tiles of 16 k-steps are staged k-major in LDS (double buffered, one barrier per step) so that the
+// 64 lanes of an MFMA operand read 2 x 32 consecutive floats.  Workgroup ids are remapped so that the workgroups that land
+// on one XCD (id mod 8) sweep all row tiles of a few column tiles: a W tile is then fetched by one L2 only.
+#include "dsx_device.h"
+#include "dsx_internal.h"
+
+namespace dsx {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kFcThreads = 256;
+constexpr int kFcBK = 16;
+constexpr int kXcds = 8;
+
+struct FcArgs {
+    const float* X;
+    const float* W;
+    const float* bias;
+    float* Z;
+    uint32_t ldx, ldw, ldz;
+    uint32_t batch, k, n;
+    uint32_t tiles_m, tiles_n;
+    int accumulate;
+    uint32_t act;
+    float slope, alpha, lambda;
+};
+
+// MI, NI: 32x32 MFMA blocks per wavefront in M and N.  XV / WV: vector width (floats) of the global loads of X / W.
+// TRANS: W is stored [n][k].
+template <int MI, int NI, int XV, int WV, bool TRANS, int ACT>
+__global__ __launch_bounds__(kFcThreads) void fc_gemm_kernel(FcArgs a)
+{
+    constexpr int BM = 64 * MI, BN = 64 * NI, BK = kFcBK;
+    constexpr int LDA = BM + 4, LDB = BN + 4;
+    constexpr int A_ELEMS = BM * BK / kFcThreads;   // floats of the X tile per lane
+    constexpr int B_ELEMS = BN * BK / kFcThreads;
+    __shared__ float sA[2][BK][LDA];
+    __shared__ float sB[2][BK][LDB];
+
+    // XCD-aware tile order
+    const uint32_t total = a.tiles_m * a.tiles_n;
+    uint32_t wg = blockIdx.x;
+    {
+        const uint32_t per_xcd = (total + kXcds - 1) / kXcds;
+        const uint32_t xcd = wg % kXcds, local = wg / kXcds;
+        wg = xcd * per_xcd + local;
+        if (local >= per_xcd || wg >= total) return;
+    }
+    const uint32_t tm = wg % a.tiles_m, tn = wg / a.tiles_m;
+    const uint32_t row0 = tm * BM, col0 = tn * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    floatx16 acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < NI; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    float ra[A_ELEMS], rb[B_ELEMS];
+
+    // X tile: element (i, kk) of the tile is X[row0 + i][k0 + kk]; lanes walk k fastest.
+    auto load_a = [&](uint32_t k0) {
+        if constexpr (XV == 4) {
+#pragma unroll
+            for (int p = 0; p < A_ELEMS / 4; p++) {
+                const int idx = tid + p * kFcThreads;
+                const int i = idx / (BK / 4), k4 = (idx % (BK / 4)) * 4;
+                const uint32_t r = row0 + i, kk = k0 + k4;
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (r < a.batch) {
+                    const float* src = a.X + (uint64_t)r * a.ldx + kk;
+                    if (kk + 4 <= a.k) {
+                        v = *reinterpret_cast<const float4*>(src);
+                    } else {
+                        if (kk < a.k) v.x = src[0];
+                        if (kk + 1 < a.k) v.y = src[1];
+                        if (kk + 2 < a.k) v.z = src[2];
+                    }
+                }
+                ra[p * 4 + 0] = v.x; ra[p * 4 + 1] = v.y; ra[p * 4 + 2] = v.z; ra[p * 4 + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < A_ELEMS; p++) {
+                const int idx = tid + p * kFcThreads;
+                const int i = idx / BK, kk = idx % BK;
+                const uint32_t r = row0 + i;
+                ra[p] = (r < a.batch && k0 + kk < a.k) ? a.X[(uint64_t)r * a.ldx + k0 + kk] : 0.0f;
+            }
+        }
+    };
+    auto store_a = [&](int buf) {
+        if constexpr (XV == 4) {
+#pragma unroll
+            for (int p = 0; p < A_ELEMS / 4; p++) {
+                const int idx = tid + p * kFcThreads;
+                const int i = idx / (BK / 4), k4 = (idx % (BK / 4)) * 4;
+#pragma unroll
+                for (int c = 0; c < 4; c++) sA[buf][k4 + c][i] = ra[p * 4 + c];
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < A_ELEMS; p++) {
+                const int idx = tid + p * kFcThreads;
+                sA[buf][idx % BK][idx / BK] = ra[p];
+            }
+        }
+    };
+    // W tile: element (kk, j) is W[k0 + kk][col0 + j] (or W[col0 + j][k0 + kk] when TRANS).
+    auto load_b = [&](uint32_t k0) {
+        if constexpr (TRANS) {
+            if constexpr (WV == 4) {
+#pragma unroll
+                for (int p = 0; p < B_ELEMS / 4; p++) {
+                    const int idx = tid + p * kFcThreads;
+                    const int j = idx / (BK / 4), k4 = (idx % (BK / 4)) * 4;
+                    const uint32_t c = col0 + j, kk = k0 + k4;
+                    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                    if (c < a.n) {
+                        const float* src = a.W + (uint64_t)c * a.ldw + kk;
+                        if (kk + 4 <= a.k) {
+                            v = *reinterpret_cast<const float4*>(src);
+                        } else {
+                            if (kk < a.k) v.x = src[0];
+                            if (kk + 1 < a.k) v.y = src[1];
+                            if (kk + 2 < a.k) v.z = src[2];
+                        }
+                    }
+                    rb[p * 4 + 0] = v.x; rb[p * 4 + 1] = v.y; rb[p * 4 + 2] = v.z; rb[p * 4 + 3] = v.w;
+                }
+            } else {
+#pragma unroll
+                for (int p = 0; p < B_ELEMS; p++) {
+                    const int idx = tid + p * kFcThreads;
+                    const int j = idx / BK, kk = idx % BK;
+                    const uint32_t c = col0 + j;
+                    rb[p] = (c < a.n && k0 + kk < a.k) ? a.W[(uint64_t)c * a.ldw + k0 + kk] : 0.0f;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < B_ELEMS / WV; p++) {
+                const int idx = tid + p * kFcThreads;
+                const int kk = idx / (BN / WV), j = (idx % (BN / WV)) * WV;
+                const uint32_t c = col0 + j, kr = k0 + kk;
+                float v[WV];
+#pragma unroll
+                for (int e = 0; e < WV; e++) v[e] = 0.0f;
+                if (kr < a.k) {
+                    const float* src = a.W + (uint64_t)kr * a.ldw + c;
+                    if (c + WV <= a.n) {
+                        if constexpr (WV == 4) {
+                            const float4 t = *reinterpret_cast<const float4*>(src);
+                            v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+                        } else if constexpr (WV == 2) {
+                            const float2 t = *reinterpret_cast<const float2*>(src);
+                            v[0] = t.x; v[1] = t.y;
+                        } else {
+                            v[0] = src[0];
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < WV; e++)
+                            if (c + e < a.n) v[e] = src[e];
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < WV; e++) rb[p * WV + e] = v[e];
+            }
+        }
+    };
+    auto store_b = [&](int buf) {
+        if constexpr (TRANS) {
+            if constexpr (WV == 4) {
+#pragma unroll
+                for (int p = 0; p < B_ELEMS / 4; p++) {
+                    const int idx = tid + p * kFcThreads;
+                    const int j = idx / (BK / 4), k4 = (idx % (BK / 4)) * 4;
+#pragma unroll
+                    for (int c = 0; c < 4; c++) sB[buf][k4 + c][j] = rb[p * 4 + c];
+                }
+            } else {
+#pragma unroll
+                for (int p = 0; p < B_ELEMS; p++) {
+                    const int idx = tid + p * kFcThreads;
+                    sB[buf][idx % BK][idx / BK] = rb[p];
+                }
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < B_ELEMS / WV; p++) {
+                const int idx = tid + p * kFcThreads;
+                const int kk = idx / (BN / WV), j = (idx % (BN / WV)) * WV;
+#pragma unroll
+                for (int e = 0; e < WV; e++) sB[buf][kk][j + e] = rb[p * WV + e];
+            }
+        }
+    };
+
+    const uint32_t nk = (a.k + BK - 1) / BK;
+    load_a(0);
+    load_b(0);
+    store_a(0);
+    store_b(0);
+    __syncthreads();
+    for (uint32_t kt = 0; kt < nk; kt++) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) {
+            load_a((kt + 1) * BK);
+            load_b((kt + 1) * BK);
+        }
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 2) {
+            float av[MI], bv[NI];
+#pragma unroll
+            for (int i = 0; i < MI; i++) av[i] = sA[buf][kk + lhi][wm * 32 * MI + i * 32 + l32];
+#pragma unroll
+            for (int j = 0; j < NI; j++) bv[j] = sB[buf][kk + lhi][wn * 32 * NI + j * 32 + l32];
+#pragma unroll
+            for (int i = 0; i < MI; i++)
+#pragma unroll
+                for (int j = 0; j < NI; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nk) {
+            store_a(buf ^ 1);
+            store_b(buf ^ 1);
+        }
+        __syncthreads();
+    }
+
+    // Epilogue: accumulator register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 block.
+#pragma unroll
+    for (int j = 0; j < NI; j++) {
+        const uint32_t c = col0 + wn * 32 * NI + j * 32 + l32;
+        if (c >= a.n) continue;
+        const float bias = a.bias ? a.bias[c] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < MI; i++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const uint32_t r = row0 + wm * 32 * MI + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
+                if (r < a.batch) {
+                    float* dst = a.Z + (uint64_t)r * a.ldz + c;
+                    float x = acc[i][j][v] + bias;
+                    if (a.accumulate) x += *dst;
+                    *dst = activate<ACT>(x, a.slope, a.alpha, a.lambda);
+                }
+            }
+        }
+    }
+}
+
+template <int MI, int NI, int XV, int WV, bool TRANS>
+static void launch_fc_act(const FcArgs& a, uint32_t grid)
+{
+    hipStream_t s = ctx().stream;
+#define DSX_ACT_CASE(A) \
+    case A: hipLaunchKernelGGL((fc_gemm_kernel<MI, NI, XV, WV, TRANS, A>), dim3(grid), dim3(kFcThreads), 0, s, a); break;
+    switch (a.act) {
+        DSX_ACT_CASE(DSX_ACT_SIGMOID)
+        DSX_ACT_CASE(DSX_ACT_TANH)
+        DSX_ACT_CASE(DSX_ACT_RELU)
+        DSX_ACT_CASE(DSX_ACT_LRELU)
+        DSX_ACT_CASE(DSX_ACT_ELU)
+        DSX_ACT_CASE(DSX_ACT_SELU)
+    default: hipLaunchKernelGGL((fc_gemm_kernel<MI, NI, XV, WV, TRANS, DSX_ACT_LINEAR>), dim3(grid), dim3(kFcThreads), 0, s, a); break;
+    }
+#undef DSX_ACT_CASE
+}
+
+template <int MI, int NI> static void launch_fc_shape(FcArgs& a, int xv, int wv, bool trans)
+{
+    constexpr int BM = 64 * MI, BN = 64 * NI;
+    a.tiles_m = (a.batch + BM - 1) / BM;
+    a.tiles_n = (a.n + BN - 1) / BN;
+    const uint32_t total = a.tiles_m * a.tiles_n;
+    const uint32_t grid = ((total + kXcds - 1) / kXcds) * kXcds;
+    if (trans) {
+        if (xv == 4 && wv == 4) launch_fc_act<MI, NI, 4, 4, true>(a, grid);
+        else if (xv == 4) launch_fc_act<MI, NI, 4, 1, true>(a, grid);
+        else if (wv == 4) launch_fc_act<MI, NI, 1, 4, true>(a, grid);
+        else launch_fc_act<MI, NI, 1, 1, true>(a, grid);
+    } else if (xv == 4) {
+        if (wv == 4) launch_fc_act<MI, NI, 4, 4, false>(a, grid);
+        else if (wv == 2) launch_fc_act<MI, NI, 4, 2, false>(a, grid);
+        else launch_fc_act<MI, NI, 4, 1, false>(a, grid);
+    } else {
+        if (wv == 4) launch_fc_act<MI, NI, 1, 4, false>(a, grid);
+        else if (wv == 2) launch_fc_act<MI, NI, 1, 2, false>(a, grid);
+        else launch_fc_act<MI, NI, 1, 1, false>(a, grid);
+    }
+}
+
+int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int transposed, const float* bias, float* Z, uint32_t ldz,
+           uint32_t batch, uint32_t k, uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params)
+{
+    FcArgs a{};
+    a.X = X; a.W = W; a.bias = bias; a.Z = Z;
+    a.ldx = ldx; a.ldw = ldw; a.ldz = ldz;
+    a.batch = batch; a.k = k; a.n = n;
+    a.accumulate = accumulate;
+    a.act = activation;
+    a.slope = params ? params->slope : 0.01f;
+    a.alpha = params ? params->alpha : 1.0f;
+    a.lambda = params ? params->lambda : 1.0f;
+    const int xv = (((uintptr_t)X % 16) == 0 && (ldx % 4) == 0) ? 4 : 1;
+    int wv = 1;
+    if (((uintptr_t)W % 16) == 0 && (ldw % 4) == 0) wv = 4;
+    else if (!transposed && ((uintptr_t)W % 8) == 0 && (ldw % 2) == 0) wv = 2;
+    // Large tiles when they still give every CU a few workgroups, small tiles otherwise.
+    const uint64_t big_tiles = (uint64_t)((batch + 127) / 128) * ((n + 127) / 128);
+    if (big_tiles >= (uint64_t)ctx().num_cus * 2)
+        launch_fc_shape<2, 2>(a, xv, wv, transposed != 0);
+    else
+        launch_fc_shape<1, 1>(a, xv, wv, transposed != 0);
+    DSX_LAUNCH_CHECK("fc_gemm_kernel");
+    return DSX_OK;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// Stand-alone activations (used when a layer has several sources, so the GEMM epilogue cannot apply them).
+
+__global__ __launch_bounds__(256) void activation_kernel(float* z, uint64_t size, uint32_t act, float slope, float alpha, float lambda)
+{
+    uint64_t pos = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const uint64_t step = (uint64_t)gridDim.x * blockDim.x;
+    for (; pos < size; pos += step) z[pos] = activate_rt(z[pos], act, slope, alpha, lambda);
+}
+
+// Row softmax (engine/kActivation.cu:155-236): a = min(1, exp(x - max) / sum exp(x - max)); one workgroup per row.
+__global__ __launch_bounds__(256) void softmax_kernel(float* z, uint32_t stride)
+{
+    __shared__ float sRed[256 / kWave];
+    float* row = z + (uint64_t)blockIdx.x * stride;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float m = -__builtin_inff();
+    for (uint32_t j = threadIdx.x; j < stride; j += 256) m = fmaxf(m, row[j]);
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, kWave));
+    if (lane == 0) sRed[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(sRed[0], sRed[1]), fmaxf(sRed[2], sRed[3]));
+    __syncthreads();
+    float s = 0.0f;
+    for (uint32_t j = threadIdx.x; j < stride; j += 256) s += __expf(row[j] - m);
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, kWave);
+    if (lane == 0) sRed[wave] = s;
+    __syncthreads();
+    s = (sRed[0] + sRed[1]) + (sRed[2] + sRed[3]);
+    const float inv = 1.0f / s;
+    for (uint32_t j = threadIdx.x; j < stride; j += 256) row[j] = fminf(1.0f, __expf(row[j] - m) * inv);
+}
+
+}  // namespace dsx
+
+using namespace dsx;
+
+extern "C" {
+
+int dsx_fc_forward(const float* X, uint32_t ldx, const float* W, int transposed, const float* bias, float* Z, uint32_t ldz,
+                   uint32_t batch, uint32_t k, uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(X && W && Z, "dsx_fc_forward: null device pointer");
+    DSX_CHECK_ARG(k > 0 && n > 0, "dsx_fc_forward: k = %u, n = %u", k, n);
+    DSX_CHECK_ARG(ldx >= k && ldz >= n, "dsx_fc_forward: row pitch smaller than the row (ldx %u < k %u or ldz %u < n %u)", ldx, k, ldz, n);
+    DSX_CHECK_ARG(is_elementwise_activation(activation), "dsx_fc_forward: activation %u is a row operation; pass DSX_ACT_LINEAR and call dsx_activation", activation);
+    if (batch == 0) return DSX_OK;
+    return fc_run(X, ldx, W, transposed ? k : n, transposed, bias, Z, ldz, batch, k, n, accumulate, activation, params);
+}
+
+int dsx_activation(float* unit, uint32_t batch, uint32_t stride, uint32_t activation, const dsx_act_params* params)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(unit && stride > 0, "dsx_activation: null unit or zero stride");
+    if (batch == 0) return DSX_OK;
+    if (activation == DSX_ACT_SOFTMAX) {
+        hipLaunchKernelGGL(softmax_kernel, dim3(batch), dim3(256), 0, ctx().stream, unit, stride);
+        DSX_LAUNCH_CHECK("softmax_kernel");
+        return DSX_OK;
+    }
+    switch (activation) {
+    case DSX_ACT_SIGMOID:
+    case DSX_ACT_TANH:
+    case DSX_ACT_RELU:
+    case DSX_ACT_LRELU:
+    case DSX_ACT_ELU:
+    case DSX_ACT_SELU: break;
+    default: return DSX_OK;   // CalculateActivation (engine/NNLayer.cpp:1646-1683) does nothing for the other kinds
+    }
+    const uint64_t size = (uint64_t)batch * stride;
+    uint64_t blocks = (size + 1023) / 1024;
+    const uint64_t cap = (uint64_t)ctx().num_cus * 32;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(activation_kernel, dim3((uint32_t)blocks), dim3(256), 0, ctx().stream, unit, size, activation,
+                       params ? params->slope : 0.01f, params ? params->alpha : 1.0f, params ? params->lambda : 1.0f);
+    DSX_LAUNCH_CHECK("activation_kernel");
+    return DSX_OK;
+}
+
+}  // extern "C"

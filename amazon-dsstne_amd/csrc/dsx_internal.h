@@ -1,0 +1,64 @@
+// dsx_internal.h — shared state and helpers of libdsx_hip.so (not part of the public ABI).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include "dsx.h"
+
+namespace dsx {
+
+struct Context {
+    bool initialized = false;
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    int num_cus = 0;
+    size_t gpu_bytes = 0;   // bytes currently held through dsx_malloc / dsx_malloc_managed
+    size_t cpu_bytes = 0;   // bytes currently held through dsx_malloc_host
+};
+
+Context& ctx();
+int set_error(int code, const char* fmt, ...);
+
+// engine/NNTypes.h:49
+constexpr float kMaxValue = 999999999999999.0f;
+
+}  // namespace dsx
+
+#define DSX_REQUIRE_INIT()                                                                     \
+    do {                                                                                       \
+        if (!dsx::ctx().initialized) return dsx::set_error(DSX_ENOTINIT, "%s: dsx_init has not been called", __func__); \
+    } while (0)
+
+#define DSX_HIP(call)                                                                                          \
+    do {                                                                                                       \
+        hipError_t e_ = (call);                                                                                \
+        if (e_ != hipSuccess) return dsx::set_error(DSX_EHIP, "%s: %s failed: %s", __func__, #call, hipGetErrorString(e_)); \
+    } while (0)
+
+#define DSX_CHECK_ARG(cond, ...)                                  \
+    do {                                                          \
+        if (!(cond)) return dsx::set_error(DSX_EINVAL, __VA_ARGS__); \
+    } while (0)
+
+// After a kernel launch: pick up launch-configuration errors (the analogue of LAUNCHERROR, engine/GpuTypes.h:215-223).
+#define DSX_LAUNCH_CHECK(name)                                                                                     \
+    do {                                                                                                           \
+        hipError_t e_ = hipGetLastError();                                                                         \
+        if (e_ != hipSuccess) return dsx::set_error(DSX_EHIP, "%s: launch of %s failed: %s", __func__, name, hipGetErrorString(e_)); \
+    } while (0)
+
+namespace dsx {
+// Top-K building blocks shared with the KNN search (dsx_topk.hip).
+// topk_run: per-row top-k of in[batch][pitch] over the first `width` columns.  With partial != NULL the packed lists go to
+// partial[b][partial_slot0 + segment][k] (forced_segments workgroups per row) instead of keys/values.
+int topk_run(const float* in, uint32_t pitch, uint32_t width, uint32_t batch, uint32_t k, float* keys, uint32_t* values,
+             uint32_t position, const uint32_t* index, const uint64_t* fstart, const uint64_t* fend, const uint32_t* fidx,
+             const float* fmul, uint32_t col_offset, uint64_t* partial, uint32_t partial_slots, uint32_t partial_slot0,
+             uint32_t forced_segments);
+int topk_merge(const uint64_t* partial, uint32_t slots, uint32_t k, float* keys, uint32_t* values, uint32_t batch);
+// GEMM building block shared with the KNN search (dsx_fc.hip): Z = X.W (+bias, activation), see dsx_fc_forward.
+int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int transposed, const float* bias, float* Z, uint32_t ldz,
+           uint32_t batch, uint32_t k, uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params);
+}  // namespace dsx

@@ -1,0 +1,249 @@
+// dsx_runtime.hip — context, memory and timing entry points of libdsx_hip.so.
+#include <cstring>
+#include <map>
+#include <mutex>
+#include "dsx_internal.h"
+
+namespace dsx {
+
+Context& ctx()
+{
+    static Context c;
+    return c;
+}
+
+static thread_local char g_error[1024] = "";
+
+int set_error(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+static std::mutex g_alloc_mutex;
+static std::map<void*, size_t> g_device_allocs;
+static std::map<void*, size_t> g_host_allocs;
+
+}  // namespace dsx
+
+using namespace dsx;
+
+extern "C" {
+
+const char* dsx_last_error(void) { return g_error; }
+
+int dsx_is_initialized(void) { return ctx().initialized ? 1 : 0; }
+
+int dsx_init(int device)
+{
+    Context& c = ctx();
+    if (c.initialized) {
+        if (c.device == device) return DSX_OK;
+        return set_error(DSX_EINVAL, "dsx_init: already initialised on device %d (one context per process)", c.device);
+    }
+    int count = 0;
+    DSX_HIP(hipGetDeviceCount(&count));
+    if (count < 1) return set_error(DSX_EHIP, "dsx_init: no HIP device is visible");
+    DSX_CHECK_ARG(device >= 0 && device < count, "dsx_init: device %d out of range (%d visible)", device, count);
+    DSX_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    DSX_HIP(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return set_error(DSX_EUNSUPPORTED, "dsx_init: device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
+    DSX_HIP(hipStreamCreateWithFlags(&c.stream, hipStreamNonBlocking));
+    DSX_HIP(hipEventCreate(&c.ev_start));
+    DSX_HIP(hipEventCreate(&c.ev_stop));
+    c.device = device;
+    c.num_cus = prop.multiProcessorCount;
+    c.initialized = true;
+    return DSX_OK;
+}
+
+int dsx_shutdown(void)
+{
+    Context& c = ctx();
+    if (!c.initialized) return DSX_OK;
+    hipStreamSynchronize(c.stream);
+    {
+        std::lock_guard<std::mutex> lock(g_alloc_mutex);
+        for (auto& kv : g_device_allocs) hipFree(kv.first);
+        for (auto& kv : g_host_allocs) hipHostFree(kv.first);
+        g_device_allocs.clear();
+        g_host_allocs.clear();
+        c.gpu_bytes = c.cpu_bytes = 0;
+    }
+    hipEventDestroy(c.ev_start);
+    hipEventDestroy(c.ev_stop);
+    hipStreamDestroy(c.stream);
+    c = Context();
+    return DSX_OK;
+}
+
+int dsx_get_device_info(dsx_device_info* info)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(info, "dsx_get_device_info: null info");
+    hipDeviceProp_t prop;
+    DSX_HIP(hipGetDeviceProperties(&prop, ctx().device));
+    memset(info, 0, sizeof(*info));
+    strncpy(info->name, prop.name, sizeof(info->name) - 1);
+    strncpy(info->arch, prop.gcnArchName, sizeof(info->arch) - 1);
+    info->compute_units = prop.multiProcessorCount;
+    info->wavefront_size = prop.warpSize;
+    info->lds_bytes_per_cu = (int)prop.sharedMemPerBlock;
+    info->hbm_bytes = prop.totalGlobalMem;
+    size_t free_b = 0, total_b = 0;
+    DSX_HIP(hipMemGetInfo(&free_b, &total_b));
+    info->hbm_free_bytes = free_b;
+    info->clock_khz = prop.clockRate;
+    info->memory_clock_khz = prop.memoryClockRate;
+    return DSX_OK;
+}
+
+int dsx_get_memory_usage(int* gpu_kib, int* cpu_kib)
+{
+    if (gpu_kib) *gpu_kib = (int)(ctx().gpu_bytes / 1024);
+    if (cpu_kib) *cpu_kib = (int)(ctx().cpu_bytes / 1024);
+    return DSX_OK;
+}
+
+void* dsx_stream(void) { return (void*)ctx().stream; }
+
+int dsx_malloc(void** p, size_t bytes)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(p, "dsx_malloc: null result pointer");
+    *p = nullptr;
+    if (bytes == 0) bytes = 4;
+    hipError_t e = hipMalloc(p, bytes);
+    if (e != hipSuccess) return set_error(DSX_ENOMEM, "dsx_malloc: hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+    DSX_HIP(hipMemsetAsync(*p, 0, bytes, ctx().stream));
+    std::lock_guard<std::mutex> lock(g_alloc_mutex);
+    g_device_allocs[*p] = bytes;
+    ctx().gpu_bytes += bytes;
+    return DSX_OK;
+}
+
+int dsx_malloc_managed(void** p, size_t bytes)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(p, "dsx_malloc_managed: null result pointer");
+    *p = nullptr;
+    if (bytes == 0) bytes = 4;
+    // Fine-grained pinned host memory mapped into the device: host-dereferenceable without page migration.
+    hipError_t e = hipHostMalloc(p, bytes, hipHostMallocMapped | hipHostMallocPortable);
+    if (e != hipSuccess) return set_error(DSX_ENOMEM, "dsx_malloc_managed: hipHostMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+    memset(*p, 0, bytes);
+    std::lock_guard<std::mutex> lock(g_alloc_mutex);
+    g_host_allocs[*p] = bytes;
+    ctx().cpu_bytes += bytes;
+    return DSX_OK;
+}
+
+int dsx_malloc_host(void** p, size_t bytes)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(p, "dsx_malloc_host: null result pointer");
+    *p = nullptr;
+    if (bytes == 0) bytes = 4;
+    hipError_t e = hipHostMalloc(p, bytes, hipHostMallocDefault);
+    if (e != hipSuccess) return set_error(DSX_ENOMEM, "dsx_malloc_host: hipHostMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+    std::lock_guard<std::mutex> lock(g_alloc_mutex);
+    g_host_allocs[*p] = bytes;
+    ctx().cpu_bytes += bytes;
+    return DSX_OK;
+}
+
+int dsx_free(void* p)
+{
+    if (!p) return DSX_OK;
+    DSX_REQUIRE_INIT();
+    {
+        std::lock_guard<std::mutex> lock(g_alloc_mutex);
+        auto it = g_device_allocs.find(p);
+        if (it == g_device_allocs.end()) {
+            auto ih = g_host_allocs.find(p);
+            if (ih == g_host_allocs.end()) return set_error(DSX_EINVAL, "dsx_free: %p was not allocated by this library", p);
+            ctx().cpu_bytes -= ih->second;
+            g_host_allocs.erase(ih);
+            DSX_HIP(hipStreamSynchronize(ctx().stream));
+            DSX_HIP(hipHostFree(p));
+            return DSX_OK;
+        }
+        ctx().gpu_bytes -= it->second;
+        g_device_allocs.erase(it);
+    }
+    DSX_HIP(hipStreamSynchronize(ctx().stream));
+    DSX_HIP(hipFree(p));
+    return DSX_OK;
+}
+
+int dsx_free_host(void* p) { return dsx_free(p); }
+
+int dsx_memset(void* p, int value, size_t bytes)
+{
+    DSX_REQUIRE_INIT();
+    if (bytes == 0) return DSX_OK;
+    DSX_CHECK_ARG(p, "dsx_memset: null pointer");
+    DSX_HIP(hipMemsetAsync(p, value, bytes, ctx().stream));
+    return DSX_OK;
+}
+
+int dsx_memcpy_h2d(void* dst, const void* src, size_t bytes)
+{
+    DSX_REQUIRE_INIT();
+    if (bytes == 0) return DSX_OK;
+    DSX_CHECK_ARG(dst && src, "dsx_memcpy_h2d: null pointer");
+    DSX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx().stream));
+    DSX_HIP(hipStreamSynchronize(ctx().stream));   // blocking like cudaMemcpy in GpuBuffer::Upload: src may be pageable
+    return DSX_OK;
+}
+
+int dsx_memcpy_d2h(void* dst, const void* src, size_t bytes)
+{
+    DSX_REQUIRE_INIT();
+    if (bytes == 0) return DSX_OK;
+    DSX_CHECK_ARG(dst && src, "dsx_memcpy_d2h: null pointer");
+    DSX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx().stream));
+    DSX_HIP(hipStreamSynchronize(ctx().stream));
+    return DSX_OK;
+}
+
+int dsx_memcpy_d2d(void* dst, const void* src, size_t bytes)
+{
+    DSX_REQUIRE_INIT();
+    if (bytes == 0) return DSX_OK;
+    DSX_CHECK_ARG(dst && src, "dsx_memcpy_d2d: null pointer");
+    DSX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx().stream));
+    return DSX_OK;
+}
+
+int dsx_sync(void)
+{
+    DSX_REQUIRE_INIT();
+    DSX_HIP(hipStreamSynchronize(ctx().stream));
+    return DSX_OK;
+}
+
+int dsx_timer_start(void)
+{
+    DSX_REQUIRE_INIT();
+    DSX_HIP(hipEventRecord(ctx().ev_start, ctx().stream));
+    return DSX_OK;
+}
+
+int dsx_timer_stop(float* elapsed_ms)
+{
+    DSX_REQUIRE_INIT();
+    DSX_HIP(hipEventRecord(ctx().ev_stop, ctx().stream));
+    DSX_HIP(hipEventSynchronize(ctx().ev_stop));
+    float ms = 0.0f;
+    DSX_HIP(hipEventElapsedTime(&ms, ctx().ev_start, ctx().ev_stop));
+    if (elapsed_ms) *elapsed_ms = ms;
+    return DSX_OK;
+}
+
+}  // extern "C"

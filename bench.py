@@ -1,0 +1,198 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse-recommendation inference path on one MI355X.
+
+A step = one pass of the hot path over one batch of synthetic input already resident in HBM:
+sparse input layer (SpMM + bias + ReLU) -> hidden FC layers -> output FC (sigmoid) -> filtered top-K.
+Default workload: the 27,278-item recommender autoencoder at batch 1024 (configs[1] of the benchmark definition).
+
+Prints ONE JSON line: whole-job predicted samples/s, the roofline figure of the dominant kernel (timed live with HIP
+events on the library's stream), every kernel's own figure, and a CPU baseline (the scalar OpenMP oracle) on a bounded
+sample of the same workload.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import numpy as np  # noqa: E402
+
+import __graft_entry__ as entry  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+FP32_MFMA_PEAK_TF = 157.3    # MI355X dense fp32 matrix, published
+
+
+def time_launches(pkg, lib, fn, reps):
+    """Average milliseconds of one call of fn(), measured with HIP events on the library stream over `reps` launches."""
+    fn()
+    pkg.check(lib.dsx_sync())
+    pkg.check(lib.dsx_timer_start())
+    for _ in range(reps):
+        fn()
+    ms = C.c_float()
+    pkg.check(lib.dsx_timer_stop(C.byref(ms)))
+    return ms.value / reps
+
+
+def network_bench(args, pkg, lib):
+    from amazon_dsstne_amd import ATTR_BOOLEAN, ATTR_INDEXED, synth
+    from amazon_dsstne_amd.pipeline import DevicePipeline
+
+    p = synth.config(args.config)
+    pipe = DevicePipeline(p, lib)
+    B, H, N, K = p.batch, p.widths[1], p.widths[-1], p.k
+    nnzB = p.batch_nnz()
+
+    for _ in range(args.warmup):
+        pipe.step()
+    pkg.check(lib.dsx_sync())
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        pipe.step()
+    pkg.check(lib.dsx_sync())
+    t1 = time.perf_counter()
+    ms_step = (t1 - t0) * 1e3 / args.steps
+
+    # per-kernel figures (HIP events around back-to-back launches of one kernel)
+    reps = max(10, min(100, args.steps))
+    params = C.byref(pipe.params)
+    ptr = pkg.ptr
+    kernels = {}
+
+    def k_sparse():
+        pkg.check(lib.dsx_sparse_layer_forward(p.attributes, p.data_type, 0, B, H, ptr(pipe.W[0]), ptr(pipe.index), ptr(pipe.start),
+                                               ptr(pipe.end), ptr(pipe.sidx), ptr(pipe.dw), ptr(pipe.sdata), ptr(pipe.b[0]),
+                                               p.acts[0], params, ptr(pipe.units[0])))
+    val_bytes = 0 if (p.attributes & ATTR_BOOLEAN) else p.sparse_data.dtype.itemsize
+    spmm_bytes = nnzB * (4 * H + 4 + val_bytes) + B * (16 + (4 if (p.attributes & ATTR_INDEXED) else 0)) + 4 * H + 4 * B * H
+    ms = time_launches(pkg, lib, k_sparse, reps)
+    kernels["sparse_z_kernel"] = {"bound": "hbm", "ms": ms, "achieved": spmm_bytes / ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                  "algorithmic_bytes": spmm_bytes}
+
+    for l in range(1, len(pipe.W)):
+        kk, n = p.widths[l], p.widths[l + 1]
+
+        def k_fc(l=l, kk=kk, n=n):
+            pkg.check(lib.dsx_fc_forward(ptr(pipe.units[l - 1]), kk, ptr(pipe.W[l]), 0, ptr(pipe.b[l]), ptr(pipe.units[l]), n, B, kk, n, 0,
+                                         p.acts[l], params))
+        flops = 2.0 * B * kk * n
+        ms = time_launches(pkg, lib, k_fc, reps)
+        name = "fc_gemm_kernel[%dx%dx%d]" % (B, kk, n)
+        kernels[name] = {"bound": "mfma", "ms": ms, "achieved": flops / ms / 1e9, "peak": FP32_MFMA_PEAK_TF, "unit": "TFLOP/s",
+                         "algorithmic_flops": flops}
+
+    def k_topk():
+        pipe.topk()
+    topk_bytes = 4 * B * N + 4 * nnzB + 8 * B * K
+    ms = time_launches(pkg, lib, k_topk, reps)
+    kernels["topk_scan_kernel"] = {"bound": "hbm", "ms": ms, "achieved": topk_bytes / ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                   "algorithmic_bytes": topk_bytes}
+    for v in kernels.values():
+        v["frac"] = v["achieved"] / v["peak"]
+
+    dominant = max(kernels, key=lambda n: kernels[n]["ms"])
+    d = kernels[dominant]
+    roofline = {"kernel": dominant, "bound": d["bound"], "achieved": round(d["achieved"], 3), "peak": d["peak"], "unit": d["unit"],
+                "frac": round(d["frac"], 4), "traffic": None, "avg_launch_ms": round(d["ms"], 5)}
+
+    # CPU baseline: the oracle (scalar C++ restatement of the reference kernels, OpenMP over rows) on whole batches of the
+    # same workload, bounded to about 10-20 s.
+    orc = entry.load_oracle()
+    cores = orc.lib().orc_num_threads()
+    secs, nb = 0.0, 0
+    budget = args.cpu_seconds
+    while nb < 1 or (secs < budget and nb < 64):
+        s, _, _, _ = orc.forward(p, 0, B, K, filtered=True)
+        secs += s
+        nb += 1
+    cpu = {"value": round(B * nb / secs, 1), "unit": "samples/s", "cores": cores, "kind": "port",
+           "sample": "%d full batches of %d rows of the same workload (%s), %.1f s" % (nb, B, p.name, secs)}
+
+    out = {
+        "metric": "predicted samples/sec (sparse-in -> filtered top-K) at batch %d" % B,
+        "value": round(B / (ms_step / 1e3), 1),
+        "unit": "samples/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": p.name, "batch": B, "input_width": p.widths[0], "layers": p.widths[1:], "top_k": K, "filtered": True,
+                   "batch_nnz": nnzB},
+        "roofline": roofline,
+        "kernels": {n: {k: (round(v, 5) if isinstance(v, float) else v) for k, v in kv.items()} for n, kv in kernels.items()},
+        "cpu_baseline": cpu,
+    }
+    return out
+
+
+def knn_bench(args, pkg, lib):
+    from amazon_dsstne_amd import synth
+
+    p = synth.knn_config(items=args.knn_items)
+    cm, rows, pad = p.column_major_padded()
+    Q, D, K = p.queries.shape[0], p.queries.shape[1], p.k
+    dI = pkg.DeviceArray.from_numpy(cm, lib)
+    dQ = pkg.DeviceArray.from_numpy(p.queries, lib)
+    scores = pkg.DeviceArray((Q, K), np.float32, lib)
+    idx = pkg.DeviceArray((Q, K), np.uint32, lib)
+    el = (C.c_float * 2)()
+
+    def step(timing=None):
+        pkg.check(lib.dsx_knn_search(dI.ptr, rows, pad, D, dQ.ptr, Q, K, scores.ptr, idx.ptr, None, 0, timing))
+    for _ in range(args.warmup):
+        step()
+    pkg.check(lib.dsx_sync())
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    pkg.check(lib.dsx_sync())
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    step(el)
+    flops = 2.0 * Q * D * (rows - pad)
+    roofline = {"kernel": "fc_gemm_kernel (knn scores)", "bound": "mfma", "achieved": round(flops / el[0] / 1e9, 3), "peak": FP32_MFMA_PEAK_TF,
+                "unit": "TFLOP/s", "frac": round(flops / el[0] / 1e9 / FP32_MFMA_PEAK_TF, 4), "traffic": None, "avg_launch_ms": round(el[0], 4),
+                "topk_ms": round(el[1], 4)}
+    orc = entry.load_oracle()
+    nq = 8
+    t0 = time.perf_counter()
+    orc.knn_search(cm, rows, pad, D, p.queries[:nq], K)
+    secs = time.perf_counter() - t0
+    cpu = {"value": round(nq / secs, 2), "unit": "queries/s", "cores": orc.lib().orc_num_threads(), "kind": "port",
+           "sample": "%d of the %d queries against the full item table, %.1f s" % (nq, Q, secs)}
+    return {"metric": "KNN queries/sec (exact top-%d over %d items)" % (K, rows - pad), "value": round(Q / (ms_step / 1e3), 1),
+            "unit": "queries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": p.name, "queries": Q, "dim": D, "items": rows - pad, "top_k": K}, "roofline": roofline,
+            "cpu_baseline": cpu}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", type=int, default=2, help="1..4 = networks of the benchmark definition, 5 = KNN")
+    ap.add_argument("--knn-items", type=int, default=2000000)
+    ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (the whole model lives in one MI355X's HBM); --gpus %d is not supported"
+                 % args.gpus)
+    pkg = entry.load_package()
+    lib = pkg.init(0)
+    out = knn_bench(args, pkg, lib) if args.config == 5 else network_bench(args, pkg, lib)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

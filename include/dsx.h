@@ -1,0 +1,217 @@
+/*
+ * dsx.h — C ABI of libdsx_hip.so: the MI355X (gfx950) device layer under the DSSTNE inference classes.
+ *
+ * Plain pointers and sizes only.  Every pointer named "device" is an address in HBM obtained from dsx_malloc (or any
+ * other HIP allocation of the same process).  All functions return 0 on success and a negative DSX_E* code on failure;
+ * dsx_last_error() then returns a message for the calling thread.  Kernels are enqueued on one library-owned HIP
+ * stream and return without waiting; dsx_sync() (or any dsx_memcpy_d2h) waits for them.
+ *
+ * Each entry point cites the function of the reference (paths relative to the reference root,
+ * engine/ = src/amazon/dsstne/engine/, knn/ = src/amazon/dsstne/knn/, utils/ = src/amazon/dsstne/utils/)
+ * whose device work it replaces.
+ */
+#ifndef DSX_H
+#define DSX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    DSX_OK = 0,
+    DSX_EINVAL = -1,     /* bad argument (null pointer, k out of range, unsupported type, ...) */
+    DSX_EHIP = -2,       /* a HIP runtime call failed */
+    DSX_ENOTINIT = -3,   /* dsx_init has not been called */
+    DSX_ENOMEM = -4,
+    DSX_EUNSUPPORTED = -5
+};
+
+/* NNDataSetEnums::Attributes bits, engine/NNEnum.h:9-19 */
+enum {
+    DSX_ATTR_SPARSE = 1,
+    DSX_ATTR_BOOLEAN = 2,
+    DSX_ATTR_INDEXED = 64,
+    DSX_ATTR_WEIGHTED = 128
+};
+
+/* NNDataSetEnums::DataType ordinals, engine/NNEnum.h:35-47 */
+enum {
+    DSX_T_UINT = 0,
+    DSX_T_INT = 1,
+    DSX_T_LLINT = 2,
+    DSX_T_ULLINT = 3,
+    DSX_T_FLOAT = 4,
+    DSX_T_DOUBLE = 5,
+    DSX_T_RGB8 = 6,
+    DSX_T_RGB16 = 7,
+    DSX_T_UCHAR = 8,
+    DSX_T_CHAR = 9
+};
+
+/* Activation ordinals, engine/NNTypes.h:91-105 */
+enum {
+    DSX_ACT_SIGMOID = 0,
+    DSX_ACT_TANH = 1,
+    DSX_ACT_RELU = 2,
+    DSX_ACT_LINEAR = 3,
+    DSX_ACT_PRELU = 4,
+    DSX_ACT_SOFTPLUS = 5,
+    DSX_ACT_SOFTSIGN = 6,
+    DSX_ACT_SOFTMAX = 7,
+    DSX_ACT_RELUMAX = 8,
+    DSX_ACT_LINEARMAX = 9,
+    DSX_ACT_ELU = 10,
+    DSX_ACT_LRELU = 11,
+    DSX_ACT_SELU = 12
+};
+
+/* Parameters of the parametric activations (NNLayer::_RELUSlope, _ELUAlpha, _SELULambda, engine/NNLayer.h:157-159). */
+typedef struct dsx_act_params {
+    float slope;
+    float alpha;
+    float lambda;
+} dsx_act_params;
+
+typedef struct dsx_device_info {
+    char name[256];
+    char arch[64];
+    int compute_units;
+    int wavefront_size;
+    int lds_bytes_per_cu;
+    size_t hbm_bytes;
+    size_t hbm_free_bytes;
+    int clock_khz;
+    int memory_clock_khz;
+} dsx_device_info;
+
+/* ---- context: GpuContext::Startup / Shutdown (engine/GpuTypes.cpp:62-406, 434-472) ------------------------------ */
+int dsx_init(int device);
+int dsx_shutdown(void);
+int dsx_is_initialized(void);
+const char* dsx_last_error(void);
+int dsx_get_device_info(dsx_device_info* info);
+/* GpuContext::GetMemoryUsage (engine/GpuTypes.cpp:520-525): KiB held through dsx_malloc* by this process. */
+int dsx_get_memory_usage(int* gpu_kib, int* cpu_kib);
+/* The HIP stream (hipStream_t) every kernel of this library is enqueued on, as an opaque pointer. */
+void* dsx_stream(void);
+
+/* ---- GpuBuffer<T> storage (engine/GpuTypes.h:392-625) ------------------------------------------------------------ */
+/* Device allocation, zero-filled like the GpuBuffer constructor (engine/GpuTypes.h:523). */
+int dsx_malloc(void** device_ptr, size_t bytes);
+/* Managed allocation (GpuBuffer bManaged = true): host-dereferenceable, zero-filled. */
+int dsx_malloc_managed(void** ptr, size_t bytes);
+/* Pinned host allocation for staging. */
+int dsx_malloc_host(void** host_ptr, size_t bytes);
+int dsx_free(void* device_ptr);
+int dsx_free_host(void* host_ptr);
+int dsx_memset(void* device_ptr, int value, size_t bytes);
+int dsx_memcpy_h2d(void* device_dst, const void* host_src, size_t bytes);   /* GpuBuffer::Upload   */
+int dsx_memcpy_d2h(void* host_dst, const void* device_src, size_t bytes);   /* GpuBuffer::Download */
+int dsx_memcpy_d2d(void* device_dst, const void* device_src, size_t bytes); /* GpuBuffer::Copy     */
+int dsx_sync(void);
+
+/* Event timing on the library stream (the reference keeps cudaEvent timings for KNN, knn/KnnExactGpu.cu:130-148). */
+int dsx_timer_start(void);
+int dsx_timer_stop(float* elapsed_ms); /* records the stop event, waits for it, returns the elapsed milliseconds */
+
+/* ---- layer input --------------------------------------------------------------------------------------------------- */
+/* kClearUnit / kClearDualSourceUnit / kClearTripleSourceUnit / kClearQuadSourceUnit (engine/kernels.cu:61-145):
+ * unit[b][j] = sum of the nbias (0..4) bias vectors; nbias == 0 zero-fills (engine/NNLayer.cpp:1002-1039). */
+int dsx_clear_unit(float* unit, const float* bias0, const float* bias1, const float* bias2, const float* bias3, uint32_t nbias,
+                   uint32_t stride, uint32_t batch);
+
+/* kLoadInputUnit<T> / kLoadIndexedInputUnit<T> (engine/kernels.cu:439-562): dense rows -> fp32 unit buffer.
+ * index == NULL for un-indexed data. */
+int dsx_load_input_unit(uint32_t data_type, uint32_t position, uint32_t batch, uint32_t stride, float* unit, const uint32_t* index,
+                        const void* data);
+
+/* kLoadSparseInputUnit / kLoadIndexedSparseInputUnit / kLoadSparseAnalogInputUnit<T> / kLoadIndexedSparseAnalogInputUnit<T>
+ * (engine/kernels.cu:147-286): zero-fill then scatter; used when the dataset is too dense for the sparse-Z path. */
+int dsx_load_sparse_input_unit(uint32_t attributes, uint32_t data_type, uint32_t position, uint32_t batch, uint32_t stride,
+                               float* unit, const uint32_t* index, const uint64_t* sparse_start, const uint64_t* sparse_end,
+                               const uint32_t* sparse_index, const float* data_weight, const void* sparse_data);
+
+/* kCalculateSparseZ / kCalculateIndexedSparseZ / kCalculateSparseAnalogZ<T> / kCalculateIndexedSparseAnalogZ<T>
+ * (engine/kernels.cu:662-1299; dispatch NNDataSet<T>::CalculateSparseZ, engine/NNTypes.h:527-545):
+ *   unit[b][:] = beta * unit[b][:] + sum over the non-zeros t of row r of (w_r * value_t) * weight[sparse_index[t]][:]
+ * with r = position + b, or index[position + b] when DSX_ATTR_INDEXED is set; value_t = 1 when DSX_ATTR_BOOLEAN is set;
+ * w_r = data_weight[r] when DSX_ATTR_WEIGHTED is set, else 1.  weight is [input width][stride] row-major.
+ * A row without non-zeros leaves unit[b] untouched. */
+int dsx_sparse_z(uint32_t attributes, uint32_t data_type, uint32_t position, uint32_t batch, uint32_t stride, const float* weight,
+                 const uint32_t* index, const uint64_t* sparse_start, const uint64_t* sparse_end, const uint32_t* sparse_index,
+                 const float* data_weight, const void* sparse_data, float* unit, float beta);
+
+/* Fused first layer for a layer whose only incoming source is a fast-sparse input:
+ * kClearUnit + kCalculate*SparseZ(beta = 1) + CalculateActivation of NNLayer::ForwardPropagateFullyConnected
+ * (engine/NNLayer.cpp:994-1167) in one kernel: unit[b][:] = act(bias[:] + sum ...).  bias may be NULL (zero). */
+int dsx_sparse_layer_forward(uint32_t attributes, uint32_t data_type, uint32_t position, uint32_t batch, uint32_t stride,
+                             const float* weight, const uint32_t* index, const uint64_t* sparse_start, const uint64_t* sparse_end,
+                             const uint32_t* sparse_index, const float* data_weight, const void* sparse_data, const float* bias,
+                             uint32_t activation, const dsx_act_params* params, float* unit);
+
+/* ---- fully connected layers ------------------------------------------------------------------------------------------ */
+/* Forward GEMM of NNLayer::ForwardPropagateFullyConnected (cublasSgemm call, engine/NNLayer.cpp:1056-1096), with the
+ * bias initialisation (kClearUnit, :1002-1039) and CalculateActivation (:1157, :1646-1683) optionally fused:
+ *   Z[b][j] = act( (accumulate ? Z[b][j] : 0) + bias[j] + sum_k X[b][k] * W[k][j] )
+ * X is [batch x k] row-major with row pitch ldx, Z is [batch x n] with row pitch ldz, W is [k x n] row-major
+ * (or [n x k] when transposed != 0: shared transposed weights, engine/NNLayer.cpp:1065-1072).
+ * bias may be NULL.  activation = DSX_ACT_LINEAR leaves the pre-activation in Z (for layers with several sources). */
+int dsx_fc_forward(const float* X, uint32_t ldx, const float* W, int transposed, const float* bias, float* Z, uint32_t ldz,
+                   uint32_t batch, uint32_t k, uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params);
+
+/* kCalculateSigmoidActivation ... kCalculateSELUActivation (engine/kActivation.cu:46-153) and
+ * kCalculateSoftMaxActivation (engine/kActivation.cu:155-236), in place on a [batch x stride] buffer. */
+int dsx_activation(float* unit, uint32_t batch, uint32_t stride, uint32_t activation, const dsx_act_params* params);
+
+/* kAddBuffers (engine/kernels.cu:4763-4781): dst += src (skip connections, engine/NNLayer.cpp:1099-1103). */
+int dsx_add_buffers(float* dst, const float* src, uint64_t size);
+
+/* ---- top-K ----------------------------------------------------------------------------------------------------------- */
+/* kCalculateTopK(pOutput, pKey, pValue, batch, width, k) (engine/kernels.cu:3202-3989): per row of `in`
+ * ([batch x width], pitch = width) the k largest values, descending, with their column numbers.
+ * Order is total: value descending, then column ascending.  1 <= k <= 256.  Slots beyond `width` candidates hold
+ * key -999999999999999.0f and index 0 (engine/NNTypes.h:49, engine/kernels.cu:3221-3224). */
+int dsx_topk(const float* in, float* keys, uint32_t* values, uint32_t batch, uint32_t width, uint32_t k);
+
+/* kCalculateTopK(pOutputKey, pOutputValue, pKey, pValue, ...) with float payload (engine/kernels.cu:3992-4188) and
+ * with uint32 payload (engine/kernels.cu:4190-4385): top-k of (key, value) pairs by key. */
+int dsx_topk_kv_f32(const float* in_keys, const float* in_values, float* keys, float* values, uint32_t batch, uint32_t width,
+                    uint32_t k);
+int dsx_topk_kv_u32(const float* in_keys, const uint32_t* in_values, float* keys, uint32_t* values, uint32_t batch, uint32_t width,
+                    uint32_t k);
+
+/* KNN variant kCalculateTopK(out, key, value, batch, width, widthPadding, k) (knn/topk.cu:29-229, knn/topk.h:73):
+ * rows have pitch `width`; only the first width - width_padding columns are candidates. */
+int dsx_knn_topk(const float* in, float* keys, uint32_t* values, uint32_t batch, uint32_t width, uint32_t width_padding, uint32_t k);
+
+/* Filtered recommendations of NNRecsGenerator::generateRecs (utils/NNRecsGenerator.cpp:132-150): the reference copies
+ * the output rows to the host, multiplies score[idx] by the filter value of every (idx, value) entry of the sample's
+ * filter (AbstractFilter::updateRecords, utils/Filters.cpp:49-67), uploads and runs kCalculateTopK.  Here the filter is
+ * applied on the fly while scanning, `in` is not modified.  The filter of batch row b is CSR row r = position + b
+ * (index[position + b] if index != NULL) of (filter_start, filter_end, filter_index, filter_mul); filter_mul == NULL
+ * means every multiplier is 0 (utils/Filters.cpp:108-121).  Indexes outside [0, width) are ignored; an index listed
+ * more than once in a row is applied once.  Passing a sample's own sparse input arrays drops the items already
+ * present in the input. */
+int dsx_topk_filtered(const float* in, float* keys, uint32_t* values, uint32_t batch, uint32_t width, uint32_t k, uint32_t position,
+                      const uint32_t* index, const uint64_t* filter_start, const uint64_t* filter_end, const uint32_t* filter_index,
+                      const float* filter_mul);
+
+/* ---- KNN ------------------------------------------------------------------------------------------------------------- */
+/* Device part of KnnExactGpu::search (knn/KnnExactGpu.cu:99-148): scores = queries . items^T (cublasSgemmEx) followed by
+ * the padded top-K.  items is column-major [rows_padded x dim] as KnnData::load builds it (knn/KnnData.cpp:197-207),
+ * i.e. items[d * rows_padded + m]; queries is row-major [num_queries x dim]; the score matrix is produced in column
+ * blocks inside the call and never stored whole.  workspace (device, workspace_bytes) may be NULL: the library then
+ * allocates what it needs for the call.  elapsed_ms (optional, 2 floats) receives the GEMM and top-K times like
+ * KnnData::elapsedSgemm / elapsedTopK. */
+int dsx_knn_search(const float* items, uint32_t rows_padded, uint32_t padding, uint32_t dim, const float* queries,
+                   uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, void* workspace, size_t workspace_bytes,
+                   float* elapsed_ms);
+size_t dsx_knn_workspace_bytes(uint32_t rows_padded, uint32_t dim, uint32_t num_queries, uint32_t k);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DSX_H */

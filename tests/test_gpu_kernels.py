@@ -1,0 +1,421 @@
+"""Parity of every C-ABI kernel entry point against the CPU oracle on the same seeded inputs (needs an MI355X)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from parity import assert_close, assert_topk_exact, check_topk_invariants
+from test_oracle import random_csr
+
+pytestmark = pytest.mark.gpu
+
+A_SPARSE, A_BOOLEAN, A_INDEXED, A_WEIGHTED = 1, 2, 64, 128
+T_UINT, T_INT, T_LLINT, T_ULLINT, T_FLOAT, T_DOUBLE, _, _, T_UCHAR, T_CHAR = range(10)
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+
+
+def dev(pkg, a):
+    return None if a is None else pkg.DeviceArray.from_numpy(a)
+
+
+# ------------------------------------------------------------------------------------------------------------- plumbing
+
+def test_device_is_gfx950(pkg, dsx):
+    info = pkg.DeviceInfo()
+    pkg.check(dsx.dsx_get_device_info(info))
+    say("device %s %s CUs=%d" % (info.name.decode(), info.arch.decode(), info.compute_units))
+    assert info.arch.decode().startswith("gfx950") and info.wavefront_size == 64
+
+
+def test_malloc_zero_fills_and_copies(pkg, dsx, rng):
+    a = pkg.DeviceArray((1000,), np.float32)
+    assert not a.numpy().any()                      # GpuBuffer constructor zero-fills (engine/GpuTypes.h:523)
+    x = rng.standard_normal(1000).astype(np.float32)
+    a.upload(x)
+    b = pkg.DeviceArray((1000,), np.float32)
+    pkg.check(dsx.dsx_memcpy_d2d(b.ptr, a.ptr, a.nbytes))
+    assert np.array_equal(b.numpy(), x)
+    pkg.check(dsx.dsx_memset(b.ptr, 0, b.nbytes))
+    assert not b.numpy().any()
+    p = C.c_void_p()
+    pkg.check(dsx.dsx_malloc_managed(C.byref(p), 64))   # host-dereferenceable (tst/amazon/dsstne/engine/TestGpuBuffer.cpp:31-68)
+    host = (C.c_float * 16).from_address(p.value)
+    host[3] = 2.5
+    assert host[3] == 2.5 and host[0] == 0.0
+    pkg.check(dsx.dsx_free(p))
+    g = C.c_int()
+    h = C.c_int()
+    pkg.check(dsx.dsx_get_memory_usage(C.byref(g), C.byref(h)))
+    assert g.value > 0
+
+
+def test_bad_arguments_are_rejected(pkg, dsx):
+    a = pkg.DeviceArray((4, 8), np.float32)
+    k = pkg.DeviceArray((4, 8), np.float32)
+    v = pkg.DeviceArray((4, 8), np.uint32)
+    assert dsx.dsx_topk(a.ptr, k.ptr, v.ptr, 4, 8, 0) == -1
+    assert dsx.dsx_topk(a.ptr, k.ptr, v.ptr, 4, 8, 257) == -1
+    assert b"1..256" in dsx.dsx_last_error()
+    assert dsx.dsx_topk(None, k.ptr, v.ptr, 4, 8, 2) == -1
+    assert dsx.dsx_knn_topk(a.ptr, k.ptr, v.ptr, 4, 8, 8, 2) == -1
+    assert dsx.dsx_clear_unit(a.ptr, None, None, None, None, 1, 8, 4) == -1
+    assert dsx.dsx_fc_forward(a.ptr, 8, a.ptr, 0, None, a.ptr, 4, 4, 8, 8, 0, 3, None) == -1     # ldz < n
+    assert dsx.dsx_fc_forward(a.ptr, 8, a.ptr, 0, None, a.ptr, 8, 4, 8, 8, 0, 7, None) == -1     # softmax cannot be fused
+    assert dsx.dsx_sparse_z(A_SPARSE, 6, 0, 1, 8, a.ptr, None, a.ptr, a.ptr, a.ptr, None, a.ptr, a.ptr, 1.0) == -5
+
+
+# ------------------------------------------------------------------------------------------------- bias, loaders, misc
+
+@pytest.mark.parametrize("nbias", [0, 1, 2, 3, 4])
+def test_clear_unit(pkg, dsx, orc, rng, nbias):
+    stride, batch = 77, 9
+    bs = [rng.standard_normal(stride).astype(np.float32) for _ in range(4)]
+    d = [dev(pkg, b) for b in bs]
+    unit = pkg.DeviceArray.from_numpy(np.full((batch, stride), 7.0, dtype=np.float32))
+    ptrs = [d[i].ptr if i < nbias else None for i in range(4)]
+    pkg.check(dsx.dsx_clear_unit(unit.ptr, ptrs[0], ptrs[1], ptrs[2], ptrs[3], nbias, stride, batch))
+    assert np.array_equal(unit.numpy(), orc.clear_unit(bs[:nbias], stride, batch))
+
+
+@pytest.mark.parametrize("dtype,tag", [(np.float32, T_FLOAT), (np.float64, T_DOUBLE), (np.int32, T_INT), (np.uint32, T_UINT),
+                                       (np.int64, T_LLINT), (np.uint64, T_ULLINT), (np.uint8, T_UCHAR), (np.int8, T_CHAR)])
+@pytest.mark.parametrize("indexed", [False, True])
+def test_load_input_unit(pkg, dsx, orc, rng, dtype, tag, indexed):
+    rows, stride, position, batch = 20, 1500, 3, 11
+    if np.issubdtype(dtype, np.floating):
+        data = rng.standard_normal((rows, stride)).astype(dtype)
+    else:
+        info = np.iinfo(dtype)
+        data = rng.integers(max(info.min, -1000), min(info.max, 1000), size=(rows, stride)).astype(dtype)
+    index = rng.permutation(rows).astype(np.uint32) if indexed else None
+    unit = pkg.DeviceArray((batch, stride), np.float32)
+    dd, di = dev(pkg, data), dev(pkg, index)
+    pkg.check(dsx.dsx_load_input_unit(tag, position, batch, stride, unit.ptr, pkg.ptr(di), dd.ptr))
+    assert np.array_equal(unit.numpy(), orc.load_input_unit(tag, position, batch, stride, index, data))
+
+
+@pytest.mark.parametrize("boolean,dtype,tag", [(True, None, T_FLOAT), (False, np.float32, T_FLOAT), (False, np.uint8, T_UCHAR),
+                                               (False, np.int32, T_INT)])
+@pytest.mark.parametrize("indexed,weighted", [(False, False), (True, True)])
+def test_load_sparse_input_unit(pkg, dsx, orc, rng, boolean, dtype, tag, indexed, weighted):
+    rows, width, position, batch = 30, 400, 4, 17
+    start, end, idx = random_csr(rng, rows, width, 50)
+    vals = None if boolean else rng.integers(1, 100, size=len(idx)).astype(dtype)
+    index = rng.permutation(rows).astype(np.uint32) if indexed else None
+    dw = (rng.random(rows, dtype=np.float32) + 0.5) if weighted else None
+    attr = A_SPARSE | (A_BOOLEAN if boolean else 0) | (A_INDEXED if indexed else 0) | (A_WEIGHTED if weighted else 0)
+    unit = pkg.DeviceArray.from_numpy(np.full((batch, width), 9.0, dtype=np.float32))
+    ds, de, dx, dv, di, dwt = (dev(pkg, x) for x in (start, end, idx, vals, index, dw))
+    pkg.check(dsx.dsx_load_sparse_input_unit(attr, tag, position, batch, width, unit.ptr, pkg.ptr(di), ds.ptr, de.ptr, dx.ptr,
+                                             pkg.ptr(dwt), pkg.ptr(dv)))
+    assert np.array_equal(unit.numpy(), orc.load_sparse_input_unit(attr, tag, position, batch, width, index, start, end, idx, dw, vals))
+
+
+def test_add_buffers(pkg, dsx, rng):
+    a = rng.standard_normal(100003).astype(np.float32)
+    b = rng.standard_normal(100003).astype(np.float32)
+    da, db = dev(pkg, a), dev(pkg, b)
+    pkg.check(dsx.dsx_add_buffers(da.ptr, db.ptr, a.size))
+    assert np.array_equal(da.numpy(), a + b)
+
+
+# ------------------------------------------------------------------------------------------------------------- sparse Z
+
+def run_sparse_z(pkg, dsx, attr, tag, position, batch, stride, W, index, start, end, idx, dw, vals, unit0, beta):
+    dW, di, ds, de, dx, dwt, dv = (dev(pkg, x) for x in (W, index, start, end, idx, dw, vals))
+    unit = pkg.DeviceArray.from_numpy(unit0)
+    pkg.check(dsx.dsx_sparse_z(attr, tag, position, batch, stride, dW.ptr, pkg.ptr(di), ds.ptr, de.ptr, dx.ptr, pkg.ptr(dwt), pkg.ptr(dv),
+                               unit.ptr, beta))
+    return unit.numpy()
+
+
+# stride 128/512/1024: 128-bit gathers with 32/128/256 lanes per weight row; 1500: two column tiles; 30: 64-bit gathers
+# (row pitch 120 bytes); 37: scalar path; 4: fewer columns than the 16-lane minimum.
+@pytest.mark.parametrize("stride", [128, 512, 1024, 1500, 30, 37, 4])
+@pytest.mark.parametrize("beta", [0.0, 1.0, 0.5])
+def test_sparse_z_boolean(pkg, dsx, orc, rng, stride, beta):
+    say("sparse_z boolean stride=%d beta=%g" % (stride, beta))
+    rows, width = 64, 3000
+    start, end, idx = random_csr(rng, rows, width, 300, empty_rows=(5, 63))
+    W = rng.standard_normal((width, stride)).astype(np.float32)
+    unit0 = rng.standard_normal((rows, stride)).astype(np.float32)
+    got = run_sparse_z(pkg, dsx, A_SPARSE | A_BOOLEAN, T_FLOAT, 0, rows, stride, W, None, start, end, idx, None, None, unit0, beta)
+    ref = orc.sparse_z(A_SPARSE | A_BOOLEAN, T_FLOAT, 0, rows, stride, W, None, start, end, idx, None, None, unit0, beta)
+    assert_close(got, ref, "sparse Z", rel=1e-4, abs_floor=1.0)   # sums of ~150 N(0,1) terms: compare on an absolute scale of 1
+    assert np.array_equal(got[[5, 63]], unit0[[5, 63]])           # rows without non-zeros stay untouched
+
+
+def test_sparse_z_long_rows_cross_lds_chunks(pkg, dsx, orc, rng):
+    # rows longer than one LDS staging pass (the reference chunks at 4608 non-zeros, engine/GpuTypes.h:131-136)
+    rows, width, stride = 6, 20000, 128
+    counts = [0, 1, 2047, 2048, 2049, 9000]
+    start = np.zeros(rows, dtype=np.uint64)
+    end = np.zeros(rows, dtype=np.uint64)
+    cols, pos = [], 0
+    for r, c in enumerate(counts):
+        cols.append(rng.choice(width, size=c, replace=False).astype(np.uint32))
+        start[r], pos = pos, pos + c
+        end[r] = pos
+    idx = np.concatenate(cols)
+    W = (rng.standard_normal((width, stride)) * 0.1).astype(np.float32)
+    unit0 = np.zeros((rows, stride), dtype=np.float32)
+    got = run_sparse_z(pkg, dsx, A_SPARSE | A_BOOLEAN, T_FLOAT, 0, rows, stride, W, None, start, end, idx, None, None, unit0, 0.0)
+    ref = orc.sparse_z(A_SPARSE | A_BOOLEAN, T_FLOAT, 0, rows, stride, W, None, start, end, idx, None, None, unit0, 0.0)
+    assert_close(got, ref, "sparse Z long rows", rel=1e-4, abs_floor=1.0)
+    assert np.array_equal(got[1], W[idx[0]])   # a single non-zero copies the weight row exactly
+
+
+@pytest.mark.parametrize("dtype,tag", [(np.float32, T_FLOAT), (np.float64, T_DOUBLE), (np.int32, T_INT), (np.uint32, T_UINT),
+                                       (np.int64, T_LLINT), (np.uint64, T_ULLINT), (np.uint8, T_UCHAR), (np.int8, T_CHAR)])
+@pytest.mark.parametrize("indexed,weighted", [(False, False), (True, False), (True, True)])
+def test_sparse_z_analog(pkg, dsx, orc, rng, dtype, tag, indexed, weighted):
+    say("sparse_z analog %s indexed=%s weighted=%s" % (dtype.__name__, indexed, weighted))
+    rows, width, stride, position, batch = 80, 1000, 96, 7, 50
+    start, end, idx = random_csr(rng, rows, width, 120)
+    if np.issubdtype(dtype, np.floating):
+        vals = (rng.integers(1, 11, size=len(idx)) * 0.5).astype(dtype)
+    elif dtype == np.int8:
+        vals = rng.integers(-100, 100, size=len(idx)).astype(dtype)
+    else:
+        vals = rng.integers(0, 200, size=len(idx)).astype(dtype)
+    index = rng.permutation(rows).astype(np.uint32) if indexed else None
+    dw = (rng.random(rows, dtype=np.float32) + 0.5) if weighted else None
+    attr = A_SPARSE | (A_INDEXED if indexed else 0) | (A_WEIGHTED if weighted else 0)
+    W = (rng.standard_normal((width, stride)) * 0.1).astype(np.float32)
+    unit0 = rng.standard_normal((batch, stride)).astype(np.float32)
+    got = run_sparse_z(pkg, dsx, attr, tag, position, batch, stride, W, index, start, end, idx, dw, vals, unit0, 1.0)
+    ref = orc.sparse_z(attr, tag, position, batch, stride, W, index, start, end, idx, dw, vals, unit0, 1.0)
+    scale = float(np.abs(ref).max())
+    assert_close(got, ref, "analog sparse Z", rel=1e-4, abs_floor=max(1.0, scale * 0.05))
+
+
+@pytest.mark.parametrize("act", [0, 1, 2, 3, 10, 11, 12])
+def test_sparse_layer_forward_fused(pkg, dsx, orc, rng, act):
+    rows, width, stride = 48, 2000, 128
+    start, end, idx = random_csr(rng, rows, width, 200, empty_rows=(0,))
+    W = (rng.standard_normal((width, stride)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal(stride).astype(np.float32)
+    params = pkg.ActParams(0.2, 1.5, 1.05)
+    dW, ds, de, dx, db = (dev(pkg, x) for x in (W, start, end, idx, bias))
+    unit = pkg.DeviceArray.from_numpy(np.full((rows, stride), 123.0, dtype=np.float32))
+    pkg.check(dsx.dsx_sparse_layer_forward(A_SPARSE | A_BOOLEAN, T_FLOAT, 0, rows, stride, dW.ptr, None, ds.ptr, de.ptr, dx.ptr, None, None,
+                                           db.ptr, act, C.byref(params), unit.ptr))
+    ref = orc.clear_unit([bias], stride, rows)
+    ref = orc.sparse_z(A_SPARSE | A_BOOLEAN, T_FLOAT, 0, rows, stride, W, None, start, end, idx, None, None, ref, 1.0)
+    ref = orc.activation(ref, act, 0.2, 1.5, 1.05)
+    assert_close(unit.numpy(), ref, "fused first layer act=%d" % act, rel=1e-4, abs_floor=1e-2)
+
+
+# ------------------------------------------------------------------------------------------------------------------ GEMM
+
+# (batch, k, n): tile-aligned, ragged in every dimension, k below one k-step, n odd (scalar loads), n even but not /4
+# (64-bit loads, the 27,278-wide case), small-tile and large-tile paths.
+GEMM_SHAPES = [(128, 128, 128), (1024, 128, 128), (33, 17, 29), (200, 100, 270), (64, 5, 64), (1024, 128, 2730), (300, 64, 27278),
+               (2048, 256, 4096), (1, 1, 1)]
+
+
+@pytest.mark.parametrize("B,k,n", GEMM_SHAPES)
+def test_fc_forward_vs_oracle(pkg, dsx, orc, rng, B, k, n):
+    say("fc_forward B=%d k=%d n=%d" % (B, k, n))
+    X = rng.standard_normal((B, k)).astype(np.float32)
+    W = (rng.standard_normal((k, n)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    dX, dW, db = dev(pkg, X), dev(pkg, W), dev(pkg, bias)
+    Z = pkg.DeviceArray.from_numpy(np.full((B, n), 55.0, dtype=np.float32))
+    pkg.check(dsx.dsx_fc_forward(dX.ptr, k, dW.ptr, 0, db.ptr, Z.ptr, n, B, k, n, 0, 3, None))
+    ref = orc.sgemm_acc(X, W, orc.clear_unit([bias], n, B))
+    scale = float(np.sqrt(k)) * 0.1
+    assert_close(Z.numpy(), ref, "fc forward", rel=1e-4, abs_floor=max(scale, 1e-2))
+    # fp64 cross-check: the GPU must be no further from the exact product than a few fp32 roundings
+    exact = X.astype(np.float64) @ W.astype(np.float64) + bias
+    assert_close(Z.numpy(), exact, "fc forward vs fp64", rel=1e-4, abs_floor=max(scale, 1e-2))
+
+
+@pytest.mark.parametrize("act", [0, 1, 2, 10, 11, 12])
+@pytest.mark.parametrize("accumulate", [0, 1])
+def test_fc_forward_epilogue(pkg, dsx, orc, rng, act, accumulate):
+    B, k, n = 70, 48, 150
+    X = rng.standard_normal((B, k)).astype(np.float32)
+    W = (rng.standard_normal((k, n)) * 0.3).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    Z0 = rng.standard_normal((B, n)).astype(np.float32)
+    params = pkg.ActParams(0.2, 1.5, 1.05)
+    dX, dW, db = dev(pkg, X), dev(pkg, W), dev(pkg, bias)
+    Z = pkg.DeviceArray.from_numpy(Z0)
+    pkg.check(dsx.dsx_fc_forward(dX.ptr, k, dW.ptr, 0, db.ptr, Z.ptr, n, B, k, n, accumulate, act, C.byref(params)))
+    pre = orc.clear_unit([bias], n, B) + (Z0 if accumulate else 0)
+    ref = orc.activation(orc.sgemm_acc(X, W, pre), act, 0.2, 1.5, 1.05)
+    assert_close(Z.numpy(), ref, "fc epilogue", rel=1e-4, abs_floor=1e-2)
+
+
+def test_fc_forward_transposed_and_pitched(pkg, dsx, orc, rng):
+    B, k, n = 90, 70, 130
+    X = rng.standard_normal((B, k + 6)).astype(np.float32)       # row pitch larger than k
+    Wt = (rng.standard_normal((n, k)) * 0.2).astype(np.float32)  # [n][k]: shared transposed weight (engine/NNLayer.cpp:1065-1072)
+    dX, dW = dev(pkg, X), dev(pkg, Wt)
+    Z = pkg.DeviceArray.from_numpy(np.zeros((B, n + 3), dtype=np.float32))
+    pkg.check(dsx.dsx_fc_forward(dX.ptr, k + 6, dW.ptr, 1, None, Z.ptr, n + 3, B, k, n, 0, 3, None))
+    got = Z.numpy()
+    ref = orc.sgemm_acc(np.ascontiguousarray(X[:, :k]), Wt, np.zeros((B, n), dtype=np.float32), transposed=True)
+    assert_close(got[:, :n], ref, "transposed fc", rel=1e-4, abs_floor=0.5)
+    assert not got[:, n:].any()                                   # nothing written past n
+
+
+@pytest.mark.parametrize("act", [0, 1, 2, 3, 7, 10, 11, 12, 5])
+def test_activation(pkg, dsx, orc, rng, act):
+    batch, stride = 37, 501
+    z = (rng.standard_normal((batch, stride)) * 4).astype(np.float32)
+    params = pkg.ActParams(0.2, 1.5, 1.05)
+    d = dev(pkg, z)
+    pkg.check(dsx.dsx_activation(d.ptr, batch, stride, act, C.byref(params)))
+    ref = orc.softmax(z) if act == 7 else orc.activation(z, act, 0.2, 1.5, 1.05)
+    assert_close(d.numpy(), ref, "activation %d" % act, rel=1e-4, abs_floor=1e-6 if act != 7 else 1e-7)
+
+
+# ----------------------------------------------------------------------------------------------------------------- top-K
+
+def run_topk(pkg, dsx, scores, k):
+    batch, width = scores.shape
+    d = dev(pkg, scores)
+    keys = pkg.DeviceArray.from_numpy(np.full((batch, k), 7.0, dtype=np.float32))
+    vals = pkg.DeviceArray.from_numpy(np.full((batch, k), 77, dtype=np.uint32))
+    pkg.check(dsx.dsx_topk(d.ptr, keys.ptr, vals.ptr, batch, width, k))
+    return keys.numpy(), vals.numpy()
+
+
+# tst/gputests/TestSort.cpp:208-211 shapes (pitch padded to 128 with zeros, padded pitch passed as the width)
+@pytest.mark.parametrize("batch,k,nfeat", [(128, 128, 1024), (128, 128, 100000), (128, 64, 1024), (128, 32, 64), (128, 1, 64)])
+def test_topk_testsort_shapes(pkg, dsx, orc, rng, batch, k, nfeat):
+    say("topk TestSort batch=%d k=%d n=%d" % (batch, k, nfeat))
+    stride = (nfeat + 127) // 128 * 128
+    scores = np.zeros((batch, stride), dtype=np.float32)
+    scores[:, :nfeat] = rng.random((batch, nfeat), dtype=np.float32)
+    keys, idx = run_topk(pkg, dsx, scores, k)
+    rk, ri = orc.topk(scores, k)
+    assert_topk_exact(keys, idx, rk, ri)
+
+
+# widths around the 16-byte alignment head/tail logic, k at every list size (64/128/256 slots), rows whose start is
+# misaligned (odd widths), more slots than columns, one workgroup per row and several.
+@pytest.mark.parametrize("batch,width,k", [(5, 1, 1), (3, 2, 4), (9, 7, 3), (4, 64, 64), (6, 65, 65), (7, 255, 128), (3, 257, 129),
+                                           (2, 1000, 256), (33, 4099, 10), (1024, 27278, 10), (3, 1000003, 100), (1, 300000, 256),
+                                           (16, 50001, 200)])
+def test_topk_random(pkg, dsx, orc, rng, batch, width, k):
+    say("topk random batch=%d width=%d k=%d" % (batch, width, k))
+    scores = rng.standard_normal((batch, width)).astype(np.float32)
+    keys, idx = run_topk(pkg, dsx, scores, k)
+    rk, ri = orc.topk(scores, k)
+    assert_topk_exact(keys, idx, rk, ri)
+    if batch * width < 3e6:
+        check_topk_invariants(scores, keys, idx, k)
+
+
+@pytest.mark.parametrize("batch,width,k", [(8, 5000, 10), (4, 700, 100), (2, 40000, 256), (64, 333, 64)])
+def test_topk_many_ties(pkg, dsx, orc, rng, batch, width, k):
+    # saturated sigmoids give long runs of identical scores: the order must be score descending, then index ascending
+    scores = (rng.integers(0, 6, size=(batch, width)).astype(np.float32) - 2) / 2
+    scores[0, :] = 1.0
+    scores[-1, ::2] = -0.0
+    keys, idx = run_topk(pkg, dsx, scores, k)
+    rk, ri = orc.topk(scores, k)
+    assert_topk_exact(keys, idx, rk, ri)
+
+
+def test_topk_extremes(pkg, dsx, orc):
+    scores = np.array([[np.inf, -np.inf, 3.4e38, -3.4e38, 1e-45, -1e-45, 0.0, -0.0, 5.0]], dtype=np.float32)
+    keys, idx = run_topk(pkg, dsx, scores, 9)
+    rk, ri = orc.topk(scores, 9)
+    assert_topk_exact(keys, idx, rk, ri)
+    assert idx[0].tolist() == [0, 2, 8, 4, 6, 7, 5, 3, 1]
+
+
+def test_knn_topk_padding(pkg, dsx, orc, rng):
+    batch, pitch, pad, k = 40, 10008, 5, 100
+    scores = rng.standard_normal((batch, pitch)).astype(np.float32)
+    scores[:, pitch - pad:] = 1e9
+    d = dev(pkg, scores)
+    keys = pkg.DeviceArray((batch, k), np.float32)
+    vals = pkg.DeviceArray((batch, k), np.uint32)
+    pkg.check(dsx.dsx_knn_topk(d.ptr, keys.ptr, vals.ptr, batch, pitch, pad, k))
+    rk, ri = orc.topk(scores, k, width=pitch - pad)
+    assert_topk_exact(keys.numpy(), vals.numpy(), rk, ri)
+
+
+@pytest.mark.parametrize("payload", [np.float32, np.uint32])
+def test_topk_kv(pkg, dsx, orc, rng, payload):
+    batch, width, k = 20, 3000, 128
+    in_keys = rng.standard_normal((batch, width)).astype(np.float32)
+    in_vals = rng.random((batch, width), dtype=np.float32) if payload == np.float32 else rng.integers(0, 1 << 32, size=(batch, width)).astype(np.uint32)
+    dk, dv = dev(pkg, in_keys), dev(pkg, in_vals)
+    keys = pkg.DeviceArray((batch, k), np.float32)
+    vals = pkg.DeviceArray((batch, k), payload)
+    fn = dsx.dsx_topk_kv_f32 if payload == np.float32 else dsx.dsx_topk_kv_u32
+    pkg.check(fn(dk.ptr, dv.ptr, keys.ptr, vals.ptr, batch, width, k))
+    rk, rv = orc.topk_kv(in_keys, in_vals, k)
+    assert np.array_equal(keys.numpy(), rk) and np.array_equal(vals.numpy(), rv)   # uint32 payloads are exact above 2^24 too
+
+
+def run_filtered(pkg, dsx, scores, k, position, index, start, end, fidx, fmul):
+    batch, width = scores.shape
+    d, di, ds, de, dx, dm = (dev(pkg, x) for x in (scores, index, start, end, fidx, fmul))
+    keys = pkg.DeviceArray((batch, k), np.float32)
+    vals = pkg.DeviceArray((batch, k), np.uint32)
+    pkg.check(dsx.dsx_topk_filtered(d.ptr, keys.ptr, vals.ptr, batch, width, k, position, pkg.ptr(di), ds.ptr, de.ptr, dx.ptr, pkg.ptr(dm)))
+    assert np.array_equal(d.numpy(), scores)   # the score matrix itself is not modified
+    return keys.numpy(), vals.numpy()
+
+
+@pytest.mark.parametrize("batch,width,k,maxnnz", [(32, 1024, 10, 16), (64, 27278, 10, 2000), (6, 600000, 100, 1000), (8, 50, 40, 45),
+                                                 (3, 9, 9, 9)])
+@pytest.mark.parametrize("with_mul", [False, True])
+def test_topk_filtered(pkg, dsx, orc, rng, batch, width, k, maxnnz, with_mul):
+    say("topk_filtered batch=%d width=%d k=%d mul=%s" % (batch, width, k, with_mul))
+    scores = rng.random((batch, width), dtype=np.float32)
+    start, end, fidx = random_csr(rng, batch, width, maxnnz, empty_rows=(1,))
+    fmul = (rng.random(len(fidx), dtype=np.float32) * 3).astype(np.float32) if with_mul else None   # multipliers above 1 can promote an item
+    keys, idx = run_filtered(pkg, dsx, scores, k, 0, None, start, end, fidx, fmul)
+    rk, ri = orc.topk_filtered(scores, k, 0, None, start, end, fidx, fmul)
+    assert_topk_exact(keys, idx, rk, ri)
+    if not with_mul and width - maxnnz >= k:
+        for b in range(batch):   # the sample's own items never come back
+            assert not set(idx[b].tolist()) & set(fidx[int(start[b]):int(end[b])].tolist())
+
+
+def test_topk_filtered_indexed_duplicates_and_out_of_range(pkg, dsx, orc, rng):
+    rows, batch, width, k, position = 12, 5, 300, 20, 4
+    scores = rng.random((batch, width), dtype=np.float32)
+    start, end, fidx = random_csr(rng, rows, width + 50, 60)     # some indexes beyond the width: ignored
+    fidx = fidx.copy()
+    fidx[1::7] = fidx[0::7][: len(fidx[1::7])]                   # duplicates inside rows: applied once
+    index = rng.permutation(rows).astype(np.uint32)
+    keys, idx = run_filtered(pkg, dsx, scores, k, position, index, start, end, fidx, None)
+    rk, ri = orc.topk_filtered(scores, k, position, index, start, end, fidx, None)
+    assert_topk_exact(keys, idx, rk, ri)
+
+
+# ------------------------------------------------------------------------------------------------------------------- KNN
+
+@pytest.mark.parametrize("items,queries,dim,k", [(1003, 9, 24, 10), (50000, 64, 256, 100), (300007, 130, 64, 128)])
+def test_knn_search(pkg, dsx, orc, synth, items, queries, dim, k):
+    say("knn items=%d queries=%d dim=%d k=%d" % (items, queries, dim, k))
+    p = synth.knn_config(seed=11, items=items, queries=queries, dim=dim, k=k)
+    cm, rows, pad = p.column_major_padded()
+    cm[:, rows - pad:] = 50.0     # pad rows are uninitialised in the reference (knn/KnnData.cpp:336-340): must never be returned
+    dI, dQ = dev(pkg, cm), dev(pkg, p.queries)
+    scores = pkg.DeviceArray((queries, k), np.float32)
+    idx = pkg.DeviceArray((queries, k), np.uint32)
+    el = (C.c_float * 2)()
+    pkg.check(dsx.dsx_knn_search(dI.ptr, rows, pad, dim, dQ.ptr, queries, k, scores.ptr, idx.ptr, None, 0, el))
+    got_s, got_i = scores.numpy(), idx.numpy()
+    ref_s, ref_i = orc.knn_search(cm, rows, pad, dim, p.queries, k)
+    full = p.queries.astype(np.float64) @ p.items.astype(np.float64).T
+    assert got_i.max() < items
+    mism = got_i != ref_i
+    if mism.any():   # different summation order may swap neighbours whose scores differ by less than 1e-5
+        r, c = np.nonzero(mism)
+        assert np.abs(full[r, got_i[r, c]] - full[r, ref_i[r, c]]).max() < 1e-5
+    assert_close(got_s, np.take_along_axis(full, got_i.astype(np.int64), axis=1), "knn scores", rel=1e-4, abs_floor=0.05)
+    assert el[0] > 0 and el[1] > 0
