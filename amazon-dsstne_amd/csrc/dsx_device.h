@@ -21,9 +21,9 @@ __device__ __forceinline__ float activate(float x, float slope, float alpha, flo
     } else if constexpr (ACT == DSX_ACT_LRELU) {
         return fmaxf(x, x * slope);
     } else if constexpr (ACT == DSX_ACT_ELU) {
-        return (x > 0.0f) ? x : alpha * (__expf(x) - 1.0f);
+        return (x > 0.0f) ? x : alpha * (expf(x) - 1.0f);   // full-precision exp: exp(x) - 1 cancels near 0
     } else if constexpr (ACT == DSX_ACT_SELU) {
-        return (x > 0.0f) ? lambda * x : lambda * alpha * (__expf(x) - 1.0f);
+        return (x > 0.0f) ? lambda * x : lambda * alpha * (expf(x) - 1.0f);
     } else {
         return x;
     }
