@@ -10,6 +10,7 @@ namespace dsx {
 
 struct Context {
     bool initialized = false;
+    int users = 0;          // dsx_init calls not yet matched by dsx_shutdown
     int device = 0;
     hipStream_t stream = nullptr;
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;

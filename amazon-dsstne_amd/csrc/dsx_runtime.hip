@@ -41,7 +41,10 @@ int dsx_init(int device)
 {
     Context& c = ctx();
     if (c.initialized) {
-        if (c.device == device) return DSX_OK;
+        if (c.device == device) {
+            ++c.users;   // every dsx_init is paired with a dsx_shutdown; the last one tears the context down
+            return DSX_OK;
+        }
         return set_error(DSX_EINVAL, "dsx_init: already initialised on device %d (one context per process)", c.device);
     }
     int count = 0;
@@ -59,6 +62,7 @@ int dsx_init(int device)
     c.device = device;
     c.num_cus = prop.multiProcessorCount;
     c.initialized = true;
+    c.users = 1;
     return DSX_OK;
 }
 
@@ -66,6 +70,7 @@ int dsx_shutdown(void)
 {
     Context& c = ctx();
     if (!c.initialized) return DSX_OK;
+    if (--c.users > 0) return DSX_OK;
     hipStreamSynchronize(c.stream);
     {
         std::lock_guard<std::mutex> lock(g_alloc_mutex);

@@ -1,0 +1,126 @@
+// NNLayer.h — one layer of a feed-forward network (public surface of the reference's engine/NNLayer.h:211-263).
+// Only fully connected layers run in this build; activations live in a [batch][stride] fp32 buffer in HBM, and a
+// fast-sparse input layer owns no buffer at all (its dataset feeds the next layer's SpMM directly).
+#ifndef DSSTNE_AMD_NNLAYER_H
+#define DSSTNE_AMD_NNLAYER_H
+
+#include "GpuTypes.h"
+#include "NNDefs.h"
+
+struct NNLayerDescriptor;
+struct NNDataSetBase;
+class NNWeight;
+class NNNetwork;
+
+class NNLayer {
+public:
+    friend class NNNetwork;
+    friend class NNWeight;
+
+    enum Kind { Input, Hidden, Output, Target };
+    static std::map<Kind, string> _sKindMap;
+
+    enum Type { FullyConnected, Convolutional, Pooling };
+    static std::map<Type, string> _sTypeMap;
+
+    enum Attributes { None = 0x0, Sparse = 0x1, Denoising = 0x2, BatchNormalization = 0x4 };
+
+    enum Parallelization { Data, Model, Serial };
+
+private:
+    const string _name;
+    const Kind _kind;
+    const Type _type;
+    const uint32_t _attributes;
+    string _dataSet;
+    NNDataSetBase* _pDataSet;
+    vector<string> _vSource;
+    vector<string> _vSkip;
+    uint32_t _Nx, _Ny, _Nz, _Nw;
+    uint32_t _stride;
+    uint32_t _localStride;
+    uint32_t _maxLocalStride;
+    uint32_t _batch;
+    uint32_t _localBatch;
+    uint32_t _dimensions;
+    uint32_t _minX, _maxX;
+    NNFloat _RELUSlope, _ELUAlpha, _SELULambda;
+    const Activation _activation;
+    const NNFloat _pDropout;
+    bool _bSparse;
+    bool _bFastSparse;
+    bool _bDirty;
+    vector<NNLayer*> _vIncomingLayer;
+    vector<NNWeight*> _vIncomingWeight;
+    vector<NNLayer*> _vOutgoingLayer;
+    vector<NNWeight*> _vOutgoingWeight;
+    vector<NNLayer*> _vIncomingSkip;
+    vector<NNLayer*> _vOutgoingSkip;
+    unique_ptr<GpuBuffer<NNFloat>> _pbUnit;
+    int32_t _priority;
+
+    NNLayer(NNLayerDescriptor& l, uint32_t batch);
+    ~NNLayer();
+    void Allocate(bool validate);
+    void Deallocate();
+    void SetBatch(uint32_t batch);
+    void RefreshState(NNNetwork* pNetwork, TrainingMode trainingMode, bool validate);
+    void LoadPredictionBatch(uint32_t position, uint32_t batch);
+    void ForwardPropagate(uint32_t position, uint32_t batch, bool bTraining = false);
+    void ForwardPropagateFullyConnected(uint32_t position, uint32_t batch, bool bTraining);
+    void CalculateActivation(uint32_t batch);
+    NNFloat* GetIncomingUnitBuffer() { return _pbUnit ? _pbUnit->_pDevData : NULL; }
+    NNFloat* GetUnitBuffer() { return _pbUnit ? _pbUnit->_pDevData : NULL; }
+    uint64_t GetBufferSize() { return (uint64_t)_batch * (uint64_t)_stride; }
+
+public:
+    const string& GetName() const;
+    const string& GetDataSetName() const;
+    Kind GetKind() const;
+    Type GetType() const;
+    uint32_t GetAttributes() const;
+    NNDataSetBase* GetDataSet() const;
+    uint32_t GetNumDimensions() const;
+    tuple<uint32_t, uint32_t, uint32_t, uint32_t> GetDimensions() const;
+    tuple<uint32_t, uint32_t, uint32_t, uint32_t> GetLocalDimensions() const;
+    Activation GetActivation() const { return _activation; }
+    bool GetUnits(vector<NNFloat>& vUnit);
+    bool GetUnits(NNFloat* pUnit);
+    bool SetUnits(const vector<NNFloat>& vUnit);
+};
+
+ostream& operator<<(ostream& out, NNLayer::Kind& k);
+ostream& operator<<(ostream& out, NNLayer::Type& t);
+
+struct NNLayerDescriptor {
+    string _name;
+    NNLayer::Kind _kind;
+    NNLayer::Type _type;
+    PoolingFunction _poolingFunction;
+    string _dataSet;
+    vector<string> _vSource;
+    vector<string> _vSkip;
+    uint32_t _Nx, _Ny, _Nz, _Nw;
+    uint32_t _dimensions;
+    bool _bDimensionsProvided;
+    WeightInitialization _weightInit;
+    NNFloat _weightInitScale;
+    NNFloat _biasInit;
+    uint32_t _kernelX, _kernelY, _kernelZ;
+    uint32_t _kernelStrideX, _kernelStrideY, _kernelStrideZ;
+    uint32_t _kernelPaddingX, _kernelPaddingY, _kernelPaddingZ;
+    uint32_t _kernelDimensions;
+    NNFloat _weightNorm;
+    NNFloat _deltaNorm;
+    NNFloat _pDropout;
+    Activation _activation;
+    NNFloat _sparsenessPenalty_p;
+    NNFloat _sparsenessPenalty_beta;
+    uint32_t _attributes;
+    NNFloat _RELUSlope;
+    NNFloat _ELUAlpha;
+    NNFloat _SELULambda;
+    NNLayerDescriptor();
+};
+
+#endif

@@ -1,0 +1,135 @@
+// NNNetwork.h — the network object of the inference path (public surface of the reference's engine/NNNetwork.h).
+// Graph of fully connected layers, dataset binding, batch position, PredictBatch and top-K.  Training, checkpoints and
+// multi-process buffers are not part of this build.
+#ifndef DSSTNE_AMD_NNNETWORK_H
+#define DSSTNE_AMD_NNNETWORK_H
+
+#include "GpuTypes.h"
+#include "NNDefs.h"
+#include "NNLayer.h"
+#include "NNWeight.h"
+
+struct NNNetworkDescriptor;
+struct NNDataSetBase;
+
+class NNNetwork {
+public:
+    friend class NNLayer;
+    friend class NNWeight;
+    enum Kind { FeedForward, AutoEncoder };
+    static std::map<Kind, string> _sKindMap;
+
+private:
+    friend NNNetwork* LoadNeuralNetworkNetCDF(const string& fname, const uint32_t batch);
+    friend NNNetwork* CreateNeuralNetwork(NNNetworkDescriptor& d, const uint32_t batch);
+    friend bool SaveNeuralNetworkNetCDF(const NNNetwork& net, const string& fname);
+
+    string _name;
+    uint32_t _batch;
+    uint32_t _position;
+    bool _bExamplesFound;
+    bool _bAllDataLoaded;
+    uint32_t _examples;
+    const Kind _kind;
+    ErrorFunction _errorFunction;
+    Mode _mode;
+    bool _bShuffleIndices;
+    NNNetworkDescriptor* _pDescriptor;          // scalar settings kept for SaveNetCDF round trips
+    vector<NNLayer*> _vLayer;
+    vector<NNLayer*> _vInputLayer;
+    vector<NNLayer*> _vOutputLayer;
+    vector<NNWeight*> _vWeight;
+    vector<NNWeight*> _vSharedWeight;
+    vector<NNDataSetBase*> _vData;
+    vector<NNLayer*> _vFPOrder;
+    map<string, NNLayer*> _mLayer;
+    bool _bDirty;
+    bool _verbose;
+
+    NNNetwork(NNNetworkDescriptor& nd, uint32_t batch = DefaultBatch);
+    void CalculatePropagationOrder();
+    void LoadBatch();
+    void RefreshState();
+    void ClearUpdates() {}
+
+public:
+    ~NNNetwork();
+    void ClearDataSets();
+    void LoadDataSets(vector<NNDataSetBase*>& vData);
+    void PredictBatch(uint32_t layers = 0);
+    void CalculateTopK(const string& layer, uint32_t k, GpuBuffer<NNFloat>* pbKey, GpuBuffer<uint32_t>* pbValue);
+    // Filtered recommendations in one device pass: the top-k of `layer` after multiplying, per sample, the scores of the
+    // items listed in the filter dataset (a sparse dataset over the layer's items) by 0, or by the dataset's float values
+    // when bUseValues is set — the device-side form of NNRecsGenerator::generateRecs (utils/NNRecsGenerator.cpp:132-150).
+    // Passing the input dataset drops the items a sample already has.
+    void CalculateFilteredTopK(const string& layer, uint32_t k, NNDataSetBase* pFilter, GpuBuffer<NNFloat>* pbKey,
+                               GpuBuffer<uint32_t>* pbValue, bool bUseValues = false);
+    void SetBatch(uint32_t batch);
+    void SetPosition(uint32_t position);
+    void SetShuffleIndices(bool bShuffleIndices);
+    void SetCPUValidate(bool bValidate);
+    bool SaveNetCDF(const string& fname);
+
+    unsigned int GetBatch() const;
+    uint32_t GetExamples() const;
+    uint32_t GetPosition() const;
+    NNWeight* GetWeight(const string& inputLayer, const string& outputLayer) const;
+    uint64_t GetBufferSize(const string& layer) const;
+    NNLayer* GetLayer(const string& layer) const;
+    vector<const NNLayer*>::iterator GetLayers(NNLayer::Kind layerKind, vector<const NNLayer*>& layers) const;
+    vector<string> GetLayers() const;
+    const string& GetName() const;
+    bool GetDebugLevel() const { return _verbose; }
+    void SetDebugLevel(bool verbose) { _verbose = verbose; }
+
+    NNFloat* GetUnitBuffer(const string& layer);
+    NNFloat* GetWeightBuffer(const string& inputLayer, const string& outputLayer);
+};
+
+ostream& operator<<(ostream& out, NNNetwork::Kind& k);
+
+struct NNNetworkDescriptor {
+    string _name;
+    NNNetwork::Kind _kind;
+    ErrorFunction _errorFunction;
+    vector<NNLayerDescriptor> _vLayerDescriptor;
+    vector<NNWeightDescriptor> _vWeightDescriptor;
+    bool _bShuffleIndices;
+    NNFloat _decay;
+    uint32_t _maxout_k;
+    NNFloat _LRN_k;
+    uint32_t _LRN_n;
+    NNFloat _LRN_alpha;
+    NNFloat _LRN_beta;
+    NNFloat _RELUSlope;
+    NNFloat _ELUAlpha;
+    NNFloat _SELULambda;
+    bool _bSparsenessPenalty;
+    NNFloat _sparsenessPenalty_p;
+    NNFloat _sparsenessPenalty_beta;
+    bool _bDenoising;
+    NNFloat _denoising_p;
+    NNFloat _deltaBoost_one;
+    NNFloat _deltaBoost_zero;
+    NNFloat _SMCE_oneTarget;
+    NNFloat _SMCE_zeroTarget;
+    NNFloat _SMCE_oneScale;
+    NNFloat _SMCE_zeroScale;
+    string _checkpoint_name;
+    int32_t _checkpoint_interval;
+    int32_t _checkpoint_epochs;
+    bool _bConvLayersCalculated;
+    NNNetworkDescriptor();
+};
+
+// Reads a network file with the reference's attribute and variable names (engine/NNNetwork.cpp:3761-4057).
+// Returns NULL after printing a message when the file cannot be read.  Caller owns the network.
+NNNetwork* LoadNeuralNetworkNetCDF(const string& fname, const uint32_t batch = DefaultBatch);
+// Builds a network from an in-memory descriptor (the reference only constructs networks through its file loaders).
+NNNetwork* CreateNeuralNetwork(NNNetworkDescriptor& d, const uint32_t batch = DefaultBatch);
+bool SaveNeuralNetworkNetCDF(const NNNetwork& net, const string& fname);
+// Descriptor-level file I/O, usable without a GPU.
+bool LoadNNNetworkDescriptorNetCDF(const string& fname, NNNetworkDescriptor& nd);
+bool SaveNNNetworkDescriptorNetCDF(const string& fname, const NNNetworkDescriptor& nd);
+
+#endif

@@ -1,0 +1,37 @@
+// DsstneContext.h — owns the device context and one network for an embedding process (the JNI / serving entry point of
+// the reference, runtime/DsstneContext.h:32-69).  One context per process.
+#ifndef DSSTNE_AMD_DSSTNECONTEXT_H
+#define DSSTNE_AMD_DSSTNECONTEXT_H
+
+#include "amazon/dsstne/engine/GpuTypes.h"
+#include "amazon/dsstne/engine/NNTypes.h"
+
+class DsstneContext {
+private:
+    static const int ALL = -1;
+    const std::string networkFilename;
+    const uint32_t batchSize;
+    const uint32_t maxK;
+    std::map<string, GpuBuffer<NNFloat>*> dOutputScores;
+    std::map<string, GpuBuffer<uint32_t>*> dOutputIndexes;
+    std::vector<NNDataSetBase*> ownedDataSets;
+
+public:
+    DsstneContext(const std::string& networkFilename, uint32_t batchSize, int maxK = ALL);
+    ~DsstneContext();
+    NNNetwork* getNetwork() const;
+    // Creates empty datasets for the input layers, binds them and runs one prediction so that every buffer exists;
+    // afterwards callers only refill the same dataset objects (LoadSparseData / LoadDenseData) and predict.
+    void initInputLayerDataSets(const std::vector<NNDataSetDescriptor> datasetDescriptors);
+    GpuBuffer<NNFloat>* getOutputScoresBuffer(const std::string& layerName);     // throws std::out_of_range for an unknown layer
+    GpuBuffer<uint32_t>* getOutputIndexesBuffer(const std::string& layerName);
+
+    static DsstneContext* fromPtr(long ptr)
+    {
+        DsstneContext* dc = (DsstneContext*)ptr;
+        if (dc == nullptr) throw std::runtime_error("Cannot convert nullptr to DsstneContext");
+        return dc;
+    }
+};
+
+#endif

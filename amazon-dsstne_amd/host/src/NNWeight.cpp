@@ -1,0 +1,122 @@
+// NNWeight.cpp — fully connected weights and biases (reference: engine/NNWeight.cpp:289-479 constructor, 938-1057 setters and
+// getters).  Only the inference state exists: the matrix, the bias vector and their host shadows.
+#include <cinttypes>
+
+#include "amazon/dsstne/engine/NNTypes.h"
+
+NNWeightDescriptor::NNWeightDescriptor()
+    : _width(1), _height(1), _length(1), _depth(1), _breadth(1), _bShared(false), _bTransposed(false), _bLocked(false), _norm(0.0f)
+{
+}
+
+NNWeight::NNWeight(NNLayer& inputLayer, NNLayer& outputLayer, bool bShared, bool bTransposed, bool bLocked, NNFloat norm)
+    : _inputLayer(inputLayer), _outputLayer(outputLayer), _bShared(bShared), _bTransposed(bTransposed), _transform(Linear),
+      _bLocked(bLocked), _pSharedWeight(NULL), _sharingCount(1), _dimensionality(2), _width(1), _height(1), _length(1), _depth(1),
+      _breadth(1), _size(0), _biasSize(0), _localSize(0), _localBiasSize(0), _norm(norm)
+{
+    inputLayer._vOutgoingLayer.push_back(&outputLayer);
+    outputLayer._vIncomingLayer.push_back(&inputLayer);
+    inputLayer._vOutgoingWeight.push_back(this);
+    outputLayer._vIncomingWeight.push_back(this);
+
+    if (outputLayer._type != NNLayer::Type::FullyConnected) {
+        printf("NNWeight::NNWeight: only fully connected layers are supported by this build (layer %s).\n", outputLayer._name.c_str());
+        getGpu().Shutdown();
+        exit(-1);
+    }
+
+    // W[input unit][output unit], output unit contiguous
+    _width = outputLayer._stride;
+    _height = inputLayer._stride;
+    _localSize = _width * _height * _length * _depth * _breadth;
+    _localBiasSize = outputLayer._localStride;
+    _size = (uint64_t)outputLayer._stride * inputLayer._stride * _length * _depth * _breadth;
+    _biasSize = outputLayer._stride;
+
+    if (!_bShared) {
+        printf("NNWeight::NNWeight: Allocating %" PRIu64 " bytes (%" PRIu64 ", %" PRIu64 ") for fully connected weights between layers %s and %s\n",
+               _localSize * sizeof(NNFloat), _width, _height, inputLayer._name.c_str(), outputLayer._name.c_str());
+        _vWeight.resize(_localSize);
+        _pbWeight.reset(new GpuBuffer<NNFloat>(_localSize));
+    }
+    _vBias.resize(_localBiasSize);
+    _pbBias.reset(new GpuBuffer<NNFloat>(_localBiasSize));
+}
+
+NNWeight::~NNWeight() {}
+
+bool NNWeight::CopyWeights(const NNWeight* pSrcWeight)
+{
+    NNWeight* pDstWeight = _bShared ? _pSharedWeight : this;
+    if (!pSrcWeight) {
+        printf("NNWeight::CopyWeights: Invalid weight pointer.\n");
+        return false;
+    }
+    const NNWeight* pSrc = _bShared ? pSrcWeight->_pSharedWeight : pSrcWeight;
+    if (!pSrc || (pSrc->_width != pDstWeight->_width) || (pSrc->_height != pDstWeight->_height) || (pSrc->_length != pDstWeight->_length)) {
+        printf("NNWeight::CopyWeights: Mismatched weight dimensions.\n");
+        return false;
+    }
+    pDstWeight->_vWeight = pSrc->_vWeight;
+    _vBias = pSrcWeight->_vBias;
+    if (pDstWeight->_pbWeight) pDstWeight->_pbWeight->Upload(pDstWeight->_vWeight.data());
+    if (_pbBias) _pbBias->Upload(_vBias.data());
+    return true;
+}
+
+bool NNWeight::SetWeights(const vector<NNFloat>& vWeight)
+{
+    NNWeight* pWeight = _bShared ? _pSharedWeight : this;
+    if (vWeight.size() < pWeight->_vWeight.size()) {
+        printf("NNWeight::SetWeights: Input vector smaller than weight vector.\n");
+        return false;
+    }
+    std::copy(vWeight.begin(), vWeight.begin() + pWeight->_vWeight.size(), pWeight->_vWeight.begin());
+    if (pWeight->_pbWeight) pWeight->_pbWeight->Upload(pWeight->_vWeight.data());
+    return true;
+}
+
+bool NNWeight::SetBiases(const vector<NNFloat>& vBias)
+{
+    if (vBias.size() < _vBias.size()) {
+        printf("NNWeight::SetBiases: Input vector smaller than bias vector.\n");
+        return false;
+    }
+    std::copy(vBias.begin(), vBias.begin() + _vBias.size(), _vBias.begin());
+    if (_pbBias) _pbBias->Upload(_vBias.data());
+    return true;
+}
+
+bool NNWeight::GetWeights(vector<NNFloat>& vWeight)
+{
+    if (vWeight.size() < _vWeight.size()) vWeight.resize(_vWeight.size());
+    if (_pbWeight)
+        _pbWeight->Download(vWeight.data());
+    else
+        vWeight = _vWeight;
+    return true;
+}
+
+bool NNWeight::GetBiases(vector<NNFloat>& vBias)
+{
+    if (vBias.size() < _vBias.size()) vBias.resize(_vBias.size());
+    if (_pbBias)
+        _pbBias->Download(vBias.data());
+    else
+        vBias = _vBias;
+    return true;
+}
+
+bool NNWeight::GetDimensions(vector<uint64_t>& dimensions)
+{
+    if (_dimensionality < 2 || _dimensionality > 5) {
+        printf("NNWeight::GetDimensions: _dimensionality = %u\n", _dimensionality);
+        return false;
+    }
+    dimensions.push_back(_width);
+    dimensions.push_back(_height);
+    if (_dimensionality >= 3) dimensions.push_back(_length);
+    if (_dimensionality >= 4) dimensions.push_back(_depth);
+    if (_dimensionality == 5) dimensions.push_back(_breadth);
+    return true;
+}

@@ -88,6 +88,7 @@ typedef struct dsx_device_info {
 } dsx_device_info;
 
 /* ---- context: GpuContext::Startup / Shutdown (engine/GpuTypes.cpp:62-406, 434-472) ------------------------------ */
+/* dsx_init may be called more than once (same device); the context lives until the matching number of dsx_shutdown calls. */
 int dsx_init(int device);
 int dsx_shutdown(void);
 int dsx_is_initialized(void);

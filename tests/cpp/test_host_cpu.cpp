@@ -1,0 +1,248 @@
+// Host-only checks (no GPU): dataset dimensions, network/dataset file round trips, filter parsing and application,
+// CPU top-K, KNN text reader and merge.  Mirrors tst/amazon/dsstne/engine/TestNNDataSetDimensions.cpp and the parsing
+// tests of tst/unittests.
+#include <cmath>
+#include <fstream>
+#include <unordered_map>
+
+#include "amazon/dsstne/engine/NNTypes.h"
+#include "amazon/dsstne/knn/KnnExactGpu.h"
+#include "amazon/dsstne/utils/Filters.h"
+#include "amazon/dsstne/utils/Utils.h"
+#include "NcClassic.h"
+#include "check.h"
+
+using namespace std;
+
+static void testDimensions()
+{
+    NNDataSetDimensions zero_d(1), one_d(2), two_d(2, 2), three_d(2, 2, 2);
+    CHECK_EQ(0U, zero_d._dimensions);
+    CHECK_EQ(1U, one_d._dimensions);
+    CHECK_EQ(2U, two_d._dimensions);
+    CHECK_EQ(3U, three_d._dimensions);
+    NNDataSetDimensions dflt;
+    CHECK(dflt._width == 1 && dflt._height == 1 && dflt._length == 1 && dflt._dimensions == 0);
+}
+
+static NNNetworkDescriptor sampleDescriptor()
+{
+    NNNetworkDescriptor nd;
+    nd._name = "roundtrip";
+    nd._kind = NNNetwork::Kind::AutoEncoder;
+    nd._errorFunction = ErrorFunction::ScaledMarginalCrossEntropy;
+    nd._SMCE_zeroScale = 0.25f;
+    nd._checkpoint_interval = 7;
+    const char* names[] = {"Input", "Hidden", "Output"};
+    const uint32_t widths[] = {6, 3, 6};
+    for (int i = 0; i < 3; i++) {
+        NNLayerDescriptor ld;
+        ld._name = names[i];
+        ld._kind = i == 0 ? NNLayer::Kind::Input : (i == 2 ? NNLayer::Kind::Output : NNLayer::Kind::Hidden);
+        ld._Nx = widths[i];
+        ld._activation = i == 1 ? Activation::LeakyRectifiedLinear : Activation::Sigmoid;
+        ld._RELUSlope = 0.125f;
+        ld._ELUAlpha = 1.5f;
+        ld._SELULambda = 1.25f;
+        ld._attributes = i == 0 ? NNLayer::Attributes::Sparse : NNLayer::Attributes::None;
+        ld._dataSet = i == 1 ? "" : "data";
+        if (i > 0) ld._vSource.push_back(names[i - 1]);
+        if (i == 2) ld._vSkip.push_back("Input");
+        nd._vLayerDescriptor.push_back(ld);
+    }
+    NNWeightDescriptor w0;
+    w0._inputLayer = "Input";
+    w0._outputLayer = "Hidden";
+    w0._width = 3;
+    w0._height = 6;
+    for (int i = 0; i < 18; i++) w0._vWeight.push_back(0.5f * i - 3);
+    w0._vBias = {0.1f, -0.2f, 0.3f};
+    nd._vWeightDescriptor.push_back(w0);
+    NNWeightDescriptor w1;
+    w1._inputLayer = "Hidden";
+    w1._outputLayer = "Output";
+    w1._width = 6;
+    w1._height = 3;
+    w1._bShared = true;
+    w1._bTransposed = true;
+    w1._sourceInputLayer = "Input";
+    w1._sourceOutputLayer = "Hidden";
+    w1._vBias = {1, 2, 3, 4, 5, 6};
+    nd._vWeightDescriptor.push_back(w1);
+    return nd;
+}
+
+static void testNetworkFileRoundTrip(const string& dir)
+{
+    NNNetworkDescriptor nd = sampleDescriptor();
+    const string f = dir + "/net.nc";
+    CHECK(SaveNNNetworkDescriptorNetCDF(f, nd));
+    NNNetworkDescriptor rd;
+    CHECK(LoadNNNetworkDescriptorNetCDF(f, rd));
+    CHECK_EQ(rd._name, nd._name);
+    CHECK_EQ(rd._kind, nd._kind);
+    CHECK_EQ(rd._errorFunction, nd._errorFunction);
+    CHECK_EQ(rd._SMCE_zeroScale, 0.25f);
+    CHECK_EQ(rd._checkpoint_interval, 7);
+    CHECK_EQ(rd._checkpoint_name, string("checkpoint"));
+    CHECK_EQ(rd._vLayerDescriptor.size(), (size_t)3);
+    CHECK_EQ(rd._vLayerDescriptor[1]._activation, Activation::LeakyRectifiedLinear);
+    CHECK_EQ(rd._vLayerDescriptor[1]._RELUSlope, 0.125f);
+    CHECK_EQ(rd._vLayerDescriptor[0]._attributes, (uint32_t)NNLayer::Attributes::Sparse);
+    CHECK_EQ(rd._vLayerDescriptor[2]._vSource.size(), (size_t)1);
+    CHECK_EQ(rd._vLayerDescriptor[2]._vSource[0], string("Hidden"));
+    CHECK_EQ(rd._vLayerDescriptor[2]._vSkip[0], string("Input"));
+    CHECK_EQ(rd._vLayerDescriptor[2]._dataSet, string("data"));
+    CHECK_EQ(rd._vWeightDescriptor.size(), (size_t)2);
+    CHECK(rd._vWeightDescriptor[0]._vWeight == nd._vWeightDescriptor[0]._vWeight);
+    CHECK(rd._vWeightDescriptor[0]._vBias == nd._vWeightDescriptor[0]._vBias);
+    CHECK_EQ(rd._vWeightDescriptor[0]._width, (uint64_t)3);
+    CHECK_EQ(rd._vWeightDescriptor[0]._height, (uint64_t)6);
+    CHECK(rd._vWeightDescriptor[1]._bShared && rd._vWeightDescriptor[1]._bTransposed);
+    CHECK_EQ(rd._vWeightDescriptor[1]._sourceOutputLayer, string("Hidden"));
+    CHECK(rd._vWeightDescriptor[1]._vWeight.empty());
+    CHECK(rd._vWeightDescriptor[1]._vBias == nd._vWeightDescriptor[1]._vBias);
+    // unreadable inputs are reported, not fatal, at the descriptor level
+    NNNetworkDescriptor bad;
+    CHECK(!LoadNNNetworkDescriptorNetCDF(dir + "/does-not-exist.nc", bad));
+    ofstream(dir + "/garbage.nc") << "this is not a NetCDF file";
+    CHECK(!LoadNNNetworkDescriptorNetCDF(dir + "/garbage.nc", bad));
+    ofstream h(dir + "/hdf5.nc", ios::binary);
+    h.write("\x89HDF\r\n\x1a\n", 8);
+    h.close();
+    CHECK(!LoadNNNetworkDescriptorNetCDF(dir + "/hdf5.nc", bad));
+}
+
+static void testFilters(const string& dir)
+{
+    unordered_map<string, unsigned int> items = {{"a", 0}, {"b", 1}, {"c", 2}, {"d", 3}};
+    unordered_map<string, unsigned int> samples = {{"u0", 0}, {"u1", 1}, {"u2", 2}};
+    {
+        ofstream f(dir + "/filter.txt");
+        f << "u0\ta:c,0.5:zzz\n";       // a -> 0 (no value), c -> 0.5, unknown item ignored
+        f << "nobody\tb\n";            // unknown sample ignored
+        f << "u2\td,2\n";
+    }
+    unique_ptr<FilterConfig> fc(loadFilters(dir + "/filter.txt", dir + "/recs.txt", items, samples));
+    CHECK_EQ(fc->getOutputFileName(), dir + "/recs.txt");
+    float row0[4] = {1, 1, 1, 1}, row1[4] = {1, 1, 1, 1}, row2[4] = {1, 1, 1, 1};
+    fc->applySamplesFilter(row0, 0, 0, 4);
+    fc->applySamplesFilter(row1, 1, 0, 4);   // no filter for u1: untouched
+    fc->applySamplesFilter(row2, 2, 0, 4);
+    CHECK(row0[0] == 0 && row0[1] == 1 && row0[2] == 0.5f && row0[3] == 1);
+    CHECK(row1[0] == 1 && row1[1] == 1 && row1[2] == 1 && row1[3] == 1);
+    CHECK(row2[3] == 2);
+    // offset / width window (utils/Filters.cpp:49-67): only indexes inside [offset, offset + width) are touched
+    float part[2] = {1, 1};
+    fc->applySamplesFilter(part, 0, 2, 2);   // covers items 2, 3
+    CHECK(part[0] == 0.5f && part[1] == 1);
+    // a path that does not exist yields an empty filter set (listFiles reports it), not an exception
+    SamplesFilter none;
+    none.loadFilter(items, samples, dir + "/no-such-filter");
+    CHECK_EQ(none.samples(), (size_t)3);
+    float keep[4] = {1, 2, 3, 4};
+    none.applyFilter(keep, 1, 0, 4);
+    CHECK(keep[0] == 1 && keep[3] == 4);
+}
+
+static void testTopKsort()
+{
+    float keys[8] = {0.5f, 0.9f, 0.1f, 0.9f, 0.3f, 0.7f, 0.9f, 0.2f};
+    float tk[4];
+    unsigned int tv[4];
+    topKsort<float, unsigned int>(keys, NULL, 8, tk, tv, 4);
+    CHECK(tk[0] == 0.9f && tk[1] == 0.9f && tk[2] == 0.9f && tk[3] == 0.7f);
+    CHECK(tv[0] == 1 && tv[1] == 3 && tv[2] == 6 && tv[3] == 5);   // equal keys: lower position first
+    float vals[8] = {8, 7, 6, 5, 4, 3, 2, 1}, tvf[3];
+    topKsort<float, float>(keys, vals, 8, tk, tvf, 3);
+    CHECK(tvf[0] == 7 && tvf[1] == 5 && tvf[2] == 2);
+}
+
+static void testKnnHost(const string& dir)
+{
+    {
+        ofstream f(dir + "/vectors.txt");
+        f << "k0\t1.0 2.0 3.0\n";
+        f << "k1\t-1 0.5 4\n";
+    }
+    uint32_t rows = 0;
+    int cols = 0;
+    TextFileDataReader::findDataDimensions(dir + "/vectors.txt", rows, cols);
+    CHECK_EQ(rows, 2u);
+    CHECK_EQ(cols, 3);
+    TextFileDataReader r(dir + "/vectors.txt");
+    string key;
+    float v[3];
+    CHECK(r.readRow(&key, v));
+    CHECK(key == "k0" && v[0] == 1 && v[1] == 2 && v[2] == 3);
+    CHECK(r.readRow(&key, v));
+    CHECK(key == "k1" && v[0] == -1 && v[1] == 0.5f && v[2] == 4);
+    CHECK(!r.readRow(&key, v));
+
+    using namespace astdl::knn;
+    // two "devices", batch 1, width 3: strict '<' keeps the lower device on ties (knn/KnnExactGpu.cu:183)
+    float s0[3] = {0.9f, 0.5f, 0.1f}, s1[3] = {0.9f, 0.7f, 0.2f};
+    uint32_t i0[3] = {0, 1, 2}, i1[3] = {0, 1, 2};
+    vector<float*> as = {s0, s1};
+    vector<uint32_t*> ai = {i0, i1};
+    vector<vector<string>> keys = {{"a0", "a1", "a2"}, {"b0", "b1", "b2"}};
+    float out[3];
+    string outk[3];
+    mergeKnn(3, 1, 3, 2, as, ai, keys, out, outk);
+    CHECK(out[0] == 0.9f && out[1] == 0.9f && out[2] == 0.7f);
+    CHECK(outk[0] == "a0" && outk[1] == "b0" && outk[2] == "b1");
+    CHECK(getDataTypeFromString("fp32") == DataType::FP32 && getDataTypeString(DataType::FP16) == "fp16");
+    checkThrows<std::invalid_argument>("bad data type", [] { getDataTypeFromString("int8"); });
+}
+
+// --dump-network file: prints what LoadNNNetworkDescriptorNetCDF sees, for comparison with an independent writer.
+static int dumpNetwork(const string& file)
+{
+    NNNetworkDescriptor nd;
+    if (!LoadNNNetworkDescriptorNetCDF(file, nd)) return 1;
+    printf("name=%s kind=%d errorFunction=%d layers=%zu weights=%zu\n", nd._name.c_str(), (int)nd._kind, (int)nd._errorFunction,
+           nd._vLayerDescriptor.size(), nd._vWeightDescriptor.size());
+    for (auto& l : nd._vLayerDescriptor)
+        printf("layer %s kind=%d Nx=%u activation=%d attributes=%u dataSet=%s sources=%zu\n", l._name.c_str(), (int)l._kind, l._Nx,
+               (int)l._activation, l._attributes, l._dataSet.c_str(), l._vSource.size());
+    for (auto& w : nd._vWeightDescriptor) {
+        double sw = 0, sb = 0;
+        for (size_t i = 0; i < w._vWeight.size(); i++) sw += (double)w._vWeight[i] * (double)(i + 1);
+        for (size_t i = 0; i < w._vBias.size(); i++) sb += (double)w._vBias[i] * (double)(i + 1);
+        printf("weight %s->%s width=%lu height=%lu shared=%d nweights=%zu wsum=%.9g bsum=%.9g\n", w._inputLayer.c_str(),
+               w._outputLayer.c_str(), (unsigned long)w._width, (unsigned long)w._height, (int)w._bShared, w._vWeight.size(), sw, sb);
+    }
+    return 0;
+}
+
+// --write-cdf2 file: a small CDF-2 file from this build's writer, to be read back by an independent reader.
+static int writeCdf2(const string& file)
+{
+    ncc::Writer nc;
+    nc.setVersion(2);
+    nc.putAttString("title", "written by NcClassic");
+    nc.putAttInt("answer", 42);
+    nc.putAttFloat("ratio", 0.375f);
+    static float fv[5] = {1.5f, -2.25f, 3.0f, 1e-3f, 7.0f};
+    static int32_t iv[3] = {-7, 0, 123456789};
+    static double dv[2] = {3.141592653589793, -1e100};
+    uint32_t d5 = nc.addDim("five", 5), d3 = nc.addDim("three", 3), d2 = nc.addDim("two", 2);
+    nc.addVar("fv", ncc::NC_FLOAT, d5, fv);
+    nc.addVar("iv", ncc::NC_INT, d3, iv);
+    nc.addVar("dv", ncc::NC_DOUBLE, d2, dv);
+    nc.write(file);
+    return 0;
+}
+
+int main(int argc, char** argv)
+{
+    if (argc > 2 && string(argv[1]) == "--dump-network") return dumpNetwork(argv[2]);
+    if (argc > 2 && string(argv[1]) == "--write-cdf2") return writeCdf2(argv[2]);
+    const string dir = argc > 1 ? argv[1] : "/tmp";
+    testDimensions();
+    testNetworkFileRoundTrip(dir);
+    testFilters(dir);
+    testTopKsort();
+    testKnnHost(dir);
+    return finish("test_host_cpu");
+}

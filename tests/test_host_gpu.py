@@ -1,0 +1,187 @@
+"""The C++ inference classes (NNNetwork, NNDataSet<T>, DsstneContext, KnnExactGpu) on the GPU, driven through their
+C ABI and through C++ programs that mirror the reference's own tests and its native embedding example."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from parity import assert_close, assert_topk_parity
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CPP = os.path.join(ROOT, "tests", "cpp")
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+
+
+def run_exe(name, *args, timeout=300):
+    exe = os.path.join(CPP, name)
+    if not os.path.exists(exe):
+        pytest.fail("%s is missing: run __graft_entry__.build()" % exe)
+    r = subprocess.run([exe] + [str(a) for a in args], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=timeout)
+    return r.returncode, r.stdout
+
+
+def test_reference_dataset_and_buffer_unit_tests():
+    """tst/amazon/dsstne/engine/TestNNDataSet.cpp and TestGpuBuffer.cpp, re-typed against this build's headers."""
+    rc, out = run_exe("test_dataset_gpu")
+    assert rc == 0 and "0 failed" in out, out[-3000:]
+
+
+def host_forward(pkg, dsx, orc, p, filtered=True, boolean=None, position=0):
+    from amazon_dsstne_amd import host_api
+    net = host_api.Network(p, max_k=p.k)
+    try:
+        net.bind_input(boolean=boolean)
+        net.predict_batch(position)
+        rows = min(p.batch, p.examples - position)
+        net.topk(p.k, filter_dataset="input" if filtered else None)
+        keys, idx = net.get_topk(rows)
+        unit = net.units(rows=p.batch)[:rows]
+    finally:
+        net.close()
+    _, ref_unit, _, _ = orc.forward(p, position, rows, filtered=False, want_unit=True, want_topk=False)
+    _, _, ref_keys, ref_idx = orc.forward(p, position, rows, filtered=filtered)
+    assert_close(unit, ref_unit, p.name + " units via NNNetwork", rel=1e-4, abs_floor=1e-3)
+    ref_scores = ref_unit.copy()
+    if filtered:
+        orc.lib().orc_apply_filter(ref_scores.ctypes.data, rows, ref_scores.shape[1], 0, position,
+                                   p.index.ctypes.data if p.index is not None else None, p.start.ctypes.data, p.end.ctypes.data,
+                                   p.sparse_index.ctypes.data, None)
+    n = assert_topk_parity(keys, idx, ref_keys, ref_idx, ref_scores, p.name + " via NNNetwork")
+    say("%s through NNNetwork::PredictBatch: parity ok (%d tie-equivalent)" % (p.name, n))
+
+
+def test_network_api_cfg1(pkg, dsx, orc, synth):
+    host_forward(pkg, dsx, orc, synth.config(1), filtered=True)
+    host_forward(pkg, dsx, orc, synth.config(1), filtered=False)
+
+
+def test_network_api_public_constructor_data_runs_analog_kernel(pkg, dsx, orc, synth):
+    # 0/1 data fed through the public API is Sparse but not Boolean and runs the analog kernel with values 1
+    # (engine/NNTypes.cpp:501-524, dispatch engine/NNTypes.h:527-545); the result must equal the Boolean path's.
+    host_forward(pkg, dsx, orc, synth.config(1), filtered=True, boolean=False)
+
+
+def test_network_api_cfg2_full(pkg, dsx, orc, synth):
+    host_forward(pkg, dsx, orc, synth.config(2), filtered=True)
+
+
+def test_network_api_positions_and_short_last_batch(pkg, dsx, orc, synth):
+    p = synth.autoencoder("three-batches", 21, 2000, [96], 64, 12, batches=3, zipf_s=1.0, nnz_mean=25, nnz_sigma=0.8, nnz_clip=(0, 300),
+                          bias_std=0.2)
+    p.examples -= 20            # 172 rows: the last batch is short (engine/NNNetwork.cpp:1415-1417)
+    p.unique_examples -= 20
+    p.start, p.end = p.start[:172], p.end[:172]
+    host_forward(pkg, dsx, orc, p, position=64)
+    host_forward(pkg, dsx, orc, p, position=128)
+
+
+def test_network_api_analog_indexed(pkg, dsx, orc, synth):
+    p = synth.autoencoder("analog-indexed-small", 1003, 27278, [256, 256], 128, 10, 1, 1.0, 144, 1.0, (5, 2000), analog=True, indexed=True)
+    host_forward(pkg, dsx, orc, p)
+
+
+def test_native_embedding_example(pkg, dsx, orc, synth, tmp_path):
+    """java/src/test/native/main.cpp flow in C++: network file -> DsstneContext -> descriptors -> LoadSparseData ->
+    PredictBatch -> kCalculateTopK; compared with the oracle's unfiltered top-K."""
+    from amazon_dsstne_amd import host_api
+    p = synth.config(1)
+    net = host_api.Network(p)
+    netfile = str(tmp_path / "cfg1.nc")
+    net.save(netfile)
+    net.close()
+    inputs = tmp_path / "inputs.txt"
+    with open(inputs, "w") as f:
+        for r in range(p.batch):
+            f.write(" ".join(str(int(i)) for i in p.sparse_index[int(p.start[r]):int(p.end[r])]) + "\n")
+    rc, out = run_exe("predict_main", netfile, inputs, p.batch, p.k)
+    assert rc == 0, out[-3000:]
+    rows = [l for l in out.splitlines() if l and l[0].isdigit() and "\t" in l]
+    assert len(rows) == p.batch, out[-2000:]
+    idx = np.zeros((p.batch, p.k), dtype=np.uint32)
+    keys = np.zeros((p.batch, p.k), dtype=np.float32)
+    for r, line in enumerate(rows):
+        cells = [c for c in line.split("\t")[1].split(",") if c]
+        for j, c in enumerate(cells):
+            i, s = c.split(":")
+            idx[r, j], keys[r, j] = int(i), float(s)
+    _, ref_unit, ref_keys, ref_idx = orc.forward(p, filtered=False, want_unit=True)
+    assert_topk_parity(keys, idx, ref_keys, ref_idx, ref_unit, "native embedding example")
+
+
+def test_soft_errors_do_not_abort(pkg, dsx, synth, capfd):
+    from amazon_dsstne_amd import host_api
+    p = synth.config(1)
+    net = host_api.Network(p, max_k=20)
+    try:
+        net.bind_input()
+        lib = net.lib
+        # SetPosition out of range: message, position unchanged (engine/NNNetwork.cpp:732-745); prediction still works
+        assert lib.dsstne_predict_batch(net.ctx, 10_000) == 0
+        # k above the context's maxK is refused
+        assert lib.dsstne_topk(net.ctx, b"Output", 21, None) != 0
+        assert b"maxK" in lib.dsstne_last_error()
+        assert lib.dsstne_topk(net.ctx, b"NoSuchLayer", 5, None) != 0
+        assert lib.dsstne_get_units(net.ctx, b"Input", None, 1) != 0      # a fast-sparse input layer has no unit buffer
+        assert lib.dsstne_load_sparse_data(net.ctx, b"nope", None, None, None, None) != 0
+        # loader exceptions surface as error codes: start[0] != 0, and more non-zeros than the dataset can hold
+        s = np.ones(p.examples, dtype=np.uint64)
+        e = np.full(p.examples, 2, dtype=np.uint64)
+        i = np.zeros(4, dtype=np.uint32)
+        assert lib.dsstne_load_sparse_data(net.ctx, b"input", s.ctypes.data, e.ctypes.data, None, i.ctypes.data) != 0
+        assert b"zero indexed" in lib.dsstne_last_error()
+        s[:] = 0
+        e[:] = 10_000_000
+        assert lib.dsstne_load_sparse_data(net.ctx, b"input", s.ctypes.data, e.ctypes.data, None, i.ctypes.data) != 0
+        assert b"Not enough space" in lib.dsstne_last_error()
+    finally:
+        net.close()
+    assert "Invalid position setting" in capfd.readouterr().out
+
+
+def test_knn_api(pkg, dsx, orc, synth, tmp_path):
+    import ctypes as C
+    from amazon_dsstne_amd import host_api
+    lib = host_api.load_host_library()
+    p = synth.knn_config(seed=5, items=20011, queries=37, dim=48, k=20)
+    knn = lib.dsstne_knn_create(64, 32)
+    assert knn
+    try:
+        items = np.ascontiguousarray(p.items)
+        assert lib.dsstne_knn_load(knn, items.ctypes.data, items.shape[0], items.shape[1], None) == 0, lib.dsstne_last_error()
+        scores = np.empty((37, 20), dtype=np.float32)
+        idx = np.empty((37, 20), dtype=np.uint32)
+        q = np.ascontiguousarray(p.queries)
+        assert lib.dsstne_knn_search(knn, 20, q.ctypes.data, 37, scores.ctypes.data, idx.ctypes.data) == 0, lib.dsstne_last_error()
+        full = p.queries.astype(np.float64) @ p.items.astype(np.float64).T
+        order = np.argsort(-full, axis=1, kind="stable")[:, :20]
+        mism = idx != order
+        if mism.any():
+            r, c = np.nonzero(mism)
+            assert np.abs(full[r, idx[r, c]] - full[r, order[r, c]]).max() < 1e-5
+        assert_close(scores, np.take_along_axis(full, idx.astype(np.int64), axis=1), "knn scores", rel=1e-4, abs_floor=0.05)
+        g, t = C.c_float(), C.c_float()
+        lib.dsstne_knn_elapsed(knn, C.byref(g), C.byref(t))
+        assert g.value > 0 and t.value > 0
+        # k > maxK -> std::invalid_argument (knn/KnnExactGpu.cu:49-54); size > batch likewise
+        assert lib.dsstne_knn_search(knn, 33, q.ctypes.data, 37, scores.ctypes.data, idx.ctypes.data) != 0
+        assert b"maxK" in lib.dsstne_last_error()
+        assert lib.dsstne_knn_search(knn, 20, q.ctypes.data, 65, scores.ctypes.data, idx.ctypes.data) != 0
+        # text-file loading: keys are labels, results come back in load order
+        path = tmp_path / "items.txt"
+        with open(path, "w") as f:
+            for i in range(50):
+                f.write("item%d\t%s\n" % (i, " ".join("%.8g" % v for v in p.items[i])))
+        assert lib.dsstne_knn_load_file(knn, str(path).encode(), b"\t", b" ") == 0, lib.dsstne_last_error()
+        s2 = np.empty((5, 3), dtype=np.float32)
+        i2 = np.empty((5, 3), dtype=np.uint32)
+        q2 = np.ascontiguousarray(p.items[:5])
+        assert lib.dsstne_knn_search(knn, 3, q2.ctypes.data, 5, s2.ctypes.data, i2.ctypes.data) == 0, lib.dsstne_last_error()
+        assert i2[:, 0].tolist() == [0, 1, 2, 3, 4] and np.allclose(s2[:, 0], 1.0, atol=1e-5)
+    finally:
+        lib.dsstne_knn_destroy(knn)
