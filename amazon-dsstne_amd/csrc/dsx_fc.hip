@@ -14,7 +14,6 @@ namespace dsx {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kFcThreads = 256;
-constexpr int kFcBK = 16;
 constexpr int kXcds = 8;
 
 struct FcArgs {
@@ -32,10 +31,10 @@ struct FcArgs {
 
 // MI, NI: 32x32 MFMA blocks per wavefront in M and N.  XV / WV: vector width (floats) of the global loads of X / W.
 // TRANS: W is stored [n][k].
-template <int MI, int NI, int XV, int WV, bool TRANS, int ACT>
-__global__ __launch_bounds__(kFcThreads) void fc_gemm_kernel(FcArgs a)
+template <int MI, int NI, int BK, int XV, int WV, bool TRANS, int ACT>
+__global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_kernel(FcArgs a)
 {
-    constexpr int BM = 64 * MI, BN = 64 * NI, BK = kFcBK;
+    constexpr int BM = 64 * MI, BN = 64 * NI;
     constexpr int LDA = BM + 4, LDB = BN + 4;
     constexpr int A_ELEMS = BM * BK / kFcThreads;   // floats of the X tile per lane
     constexpr int B_ELEMS = BN * BK / kFcThreads;
@@ -239,6 +238,26 @@ __global__ __launch_bounds__(kFcThreads) void fc_gemm_kernel(FcArgs a)
     }
 
     // Epilogue: accumulator register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 block.
+    const bool full_tile = (row0 + BM <= a.batch) && (col0 + BN <= a.n);
+    if (full_tile) {
+#pragma unroll
+        for (int j = 0; j < NI; j++) {
+            const uint32_t c = col0 + wn * 32 * NI + j * 32 + l32;
+            const float bias = a.bias ? a.bias[c] : 0.0f;
+#pragma unroll
+            for (int i = 0; i < MI; i++) {
+                float* base = a.Z + (uint64_t)(row0 + wm * 32 * MI + i * 32 + 4 * lhi) * a.ldz + c;
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    float* dst = base + (uint64_t)(8 * (v / 4) + (v % 4)) * a.ldz;
+                    float x = acc[i][j][v] + bias;
+                    if (a.accumulate) x += *dst;
+                    *dst = activate<ACT>(x, a.slope, a.alpha, a.lambda);
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < NI; j++) {
         const uint32_t c = col0 + wn * 32 * NI + j * 32 + l32;
@@ -260,12 +279,12 @@ __global__ __launch_bounds__(kFcThreads) void fc_gemm_kernel(FcArgs a)
     }
 }
 
-template <int MI, int NI, int XV, int WV, bool TRANS>
+template <int MI, int NI, int BK, int XV, int WV, bool TRANS>
 static void launch_fc_act(const FcArgs& a, uint32_t grid)
 {
     hipStream_t s = ctx().stream;
 #define DSX_ACT_CASE(A) \
-    case A: hipLaunchKernelGGL((fc_gemm_kernel<MI, NI, XV, WV, TRANS, A>), dim3(grid), dim3(kFcThreads), 0, s, a); break;
+    case A: hipLaunchKernelGGL((fc_gemm_kernel<MI, NI, BK, XV, WV, TRANS, A>), dim3(grid), dim3(kFcThreads), 0, s, a); break;
     switch (a.act) {
         DSX_ACT_CASE(DSX_ACT_SIGMOID)
         DSX_ACT_CASE(DSX_ACT_TANH)
@@ -273,12 +292,12 @@ static void launch_fc_act(const FcArgs& a, uint32_t grid)
         DSX_ACT_CASE(DSX_ACT_LRELU)
         DSX_ACT_CASE(DSX_ACT_ELU)
         DSX_ACT_CASE(DSX_ACT_SELU)
-    default: hipLaunchKernelGGL((fc_gemm_kernel<MI, NI, XV, WV, TRANS, DSX_ACT_LINEAR>), dim3(grid), dim3(kFcThreads), 0, s, a); break;
+    default: hipLaunchKernelGGL((fc_gemm_kernel<MI, NI, BK, XV, WV, TRANS, DSX_ACT_LINEAR>), dim3(grid), dim3(kFcThreads), 0, s, a); break;
     }
 #undef DSX_ACT_CASE
 }
 
-template <int MI, int NI> static void launch_fc_shape(FcArgs& a, int xv, int wv, bool trans)
+template <int MI, int NI, int BK> static void launch_fc_shape(FcArgs& a, int xv, int wv, bool trans)
 {
     constexpr int BM = 64 * MI, BN = 64 * NI;
     a.tiles_m = (a.batch + BM - 1) / BM;
@@ -286,18 +305,18 @@ template <int MI, int NI> static void launch_fc_shape(FcArgs& a, int xv, int wv,
     const uint32_t total = a.tiles_m * a.tiles_n;
     const uint32_t grid = ((total + kXcds - 1) / kXcds) * kXcds;
     if (trans) {
-        if (xv == 4 && wv == 4) launch_fc_act<MI, NI, 4, 4, true>(a, grid);
-        else if (xv == 4) launch_fc_act<MI, NI, 4, 1, true>(a, grid);
-        else if (wv == 4) launch_fc_act<MI, NI, 1, 4, true>(a, grid);
-        else launch_fc_act<MI, NI, 1, 1, true>(a, grid);
+        if (xv == 4 && wv == 4) launch_fc_act<MI, NI, BK, 4, 4, true>(a, grid);
+        else if (xv == 4) launch_fc_act<MI, NI, BK, 4, 1, true>(a, grid);
+        else if (wv == 4) launch_fc_act<MI, NI, BK, 1, 4, true>(a, grid);
+        else launch_fc_act<MI, NI, BK, 1, 1, true>(a, grid);
     } else if (xv == 4) {
-        if (wv == 4) launch_fc_act<MI, NI, 4, 4, false>(a, grid);
-        else if (wv == 2) launch_fc_act<MI, NI, 4, 2, false>(a, grid);
-        else launch_fc_act<MI, NI, 4, 1, false>(a, grid);
+        if (wv == 4) launch_fc_act<MI, NI, BK, 4, 4, false>(a, grid);
+        else if (wv == 2) launch_fc_act<MI, NI, BK, 4, 2, false>(a, grid);
+        else launch_fc_act<MI, NI, BK, 4, 1, false>(a, grid);
     } else {
-        if (wv == 4) launch_fc_act<MI, NI, 1, 4, false>(a, grid);
-        else if (wv == 2) launch_fc_act<MI, NI, 1, 2, false>(a, grid);
-        else launch_fc_act<MI, NI, 1, 1, false>(a, grid);
+        if (wv == 4) launch_fc_act<MI, NI, BK, 1, 4, false>(a, grid);
+        else if (wv == 2) launch_fc_act<MI, NI, BK, 1, 2, false>(a, grid);
+        else launch_fc_act<MI, NI, BK, 1, 1, false>(a, grid);
     }
 }
 
@@ -320,9 +339,9 @@ int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int trans
     // Large tiles when they still give every CU a few workgroups, small tiles otherwise.
     const uint64_t big_tiles = (uint64_t)((batch + 127) / 128) * ((n + 127) / 128);
     if (big_tiles >= (uint64_t)ctx().num_cus * 2)
-        launch_fc_shape<2, 2>(a, xv, wv, transposed != 0);
+        launch_fc_shape<2, 2, 16>(a, xv, wv, transposed != 0);
     else
-        launch_fc_shape<1, 1>(a, xv, wv, transposed != 0);
+        launch_fc_shape<1, 1, 32>(a, xv, wv, transposed != 0);   // few workgroups: deep k-steps, fewer barrier round trips
     DSX_LAUNCH_CHECK("fc_gemm_kernel");
     return DSX_OK;
 }

@@ -48,6 +48,31 @@ template <int VEC> __device__ __forceinline__ void store_vec(float* p, const flo
     }
 }
 
+// U gathers of one lane in flight (non-zeros t, t+G, ..., t+(U-1)G of the staged chunk), then accumulated in that order.
+// Long rows are latency bound on the gather, so the depth of this block sets the time of the longest row.
+template <int U, int VEC, bool UNITVAL>
+__device__ __forceinline__ void gather_block(const float* wcol, uint32_t stride, const uint32_t* sIdx, const float* sVal, uint32_t t,
+                                             uint32_t G, float (&acc)[VEC])
+{
+    float x[U][VEC];
+#pragma unroll
+    for (int u = 0; u < U; u++) load_vec<VEC>(wcol + (uint64_t)sIdx[t + u * G] * stride, x[u]);
+    if constexpr (UNITVAL) {
+#pragma unroll
+        for (int u = 0; u < U; u++)
+#pragma unroll
+            for (int v = 0; v < VEC; v++) acc[v] += x[u][v];
+    } else {
+        float sv[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) sv[u] = sVal[t + u * G];
+#pragma unroll
+        for (int u = 0; u < U; u++)
+#pragma unroll
+            for (int v = 0; v < VEC; v++) acc[v] = fmaf(x[u][v], sv[u], acc[v]);
+    }
+}
+
 struct SparseZArgs {
     uint32_t position, stride;
     const float* weight;
@@ -125,39 +150,9 @@ __global__ __launch_bounds__(kSparseThreads) void sparse_z_kernel(SparseZArgs a)
         __syncthreads();
         if (active) {
             uint32_t t = g;
-            for (; t + 3 * G < n; t += 4 * G) {
-                const uint32_t i0 = sIdx[t], i1 = sIdx[t + G], i2 = sIdx[t + 2 * G], i3 = sIdx[t + 3 * G];
-                float x0[VEC], x1[VEC], x2[VEC], x3[VEC];
-                load_vec<VEC>(wcol + (uint64_t)i0 * a.stride, x0);
-                load_vec<VEC>(wcol + (uint64_t)i1 * a.stride, x1);
-                load_vec<VEC>(wcol + (uint64_t)i2 * a.stride, x2);
-                load_vec<VEC>(wcol + (uint64_t)i3 * a.stride, x3);
-                if constexpr (UNITVAL) {
-#pragma unroll
-                    for (int v = 0; v < VEC; v++) acc[v] = ((acc[v] + x0[v]) + x1[v]) + x2[v] + x3[v];
-                } else {
-                    const float s0 = sVal[t], s1 = sVal[t + G], s2 = sVal[t + 2 * G], s3 = sVal[t + 3 * G];
-#pragma unroll
-                    for (int v = 0; v < VEC; v++) {
-                        acc[v] = fmaf(x0[v], s0, acc[v]);
-                        acc[v] = fmaf(x1[v], s1, acc[v]);
-                        acc[v] = fmaf(x2[v], s2, acc[v]);
-                        acc[v] = fmaf(x3[v], s3, acc[v]);
-                    }
-                }
-            }
-            for (; t < n; t += G) {
-                float x0[VEC];
-                load_vec<VEC>(wcol + (uint64_t)sIdx[t] * a.stride, x0);
-                if constexpr (UNITVAL) {
-#pragma unroll
-                    for (int v = 0; v < VEC; v++) acc[v] += x0[v];
-                } else {
-                    const float s0 = sVal[t];
-#pragma unroll
-                    for (int v = 0; v < VEC; v++) acc[v] = fmaf(x0[v], s0, acc[v]);
-                }
-            }
+            for (; t + 15 * G < n; t += 16 * G) gather_block<16, VEC, UNITVAL>(wcol, a.stride, sIdx, sVal, t, G, acc);
+            for (; t + 3 * G < n; t += 4 * G) gather_block<4, VEC, UNITVAL>(wcol, a.stride, sIdx, sVal, t, G, acc);
+            for (; t < n; t += G) gather_block<1, VEC, UNITVAL>(wcol, a.stride, sIdx, sVal, t, G, acc);
         }
     }
 

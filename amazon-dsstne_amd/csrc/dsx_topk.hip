@@ -264,6 +264,23 @@ __global__ __launch_bounds__(kTopkThreads) void topk_scan_kernel(TopKArgs a)
     List list;
     list.init(sStage[wave], lane, a.k);
 
+    // Software pipeline: the first four 16-byte groups of this lane are requested before the filter is built (its chain of
+    // dependent loads would otherwise sit in front of the scan), and inside the loop the next four are requested before the
+    // current four are examined.
+    const float4* body = reinterpret_cast<const float4*>(row + head);
+    const uint32_t step = kTopkThreads;
+    uint32_t span = g0;   // block-uniform
+    bool have = span + 4 * step <= g1;
+    float4 cur0, cur1, cur2, cur3;
+    cur0 = cur1 = cur2 = cur3 = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (have) {
+        const uint32_t g = span + threadIdx.x;
+        cur0 = body[g];
+        cur1 = body[g + step];
+        cur2 = body[g + 2 * step];
+        cur3 = body[g + 3 * step];
+    }
+
     if constexpr (FILTERED) {
         const uint32_t words = (hi - lo + 31) / 32;
         for (uint32_t i = threadIdx.x; i < words; i += kTopkThreads) sBitmap[i] = 0;
@@ -315,17 +332,30 @@ __global__ __launch_bounds__(kTopkThreads) void topk_scan_kernel(TopKArgs a)
         }
     };
 
-    // Body: the block walks the segment in 4 KiB spans, wave w takes the w-th KiB of each span; four spans in flight.
-    const float4* body = reinterpret_cast<const float4*>(row + head);
-    const uint32_t step = kTopkThreads;
-    uint32_t span = g0;   // block-uniform
-    for (; span + 4 * step <= g1; span += 4 * step) {
+    // Body: the block walks the segment in 4 KiB spans, wave w takes the w-th KiB of each span.
+    while (have) {
         const uint32_t g = span + threadIdx.x;
-        const float4 v0 = body[g], v1 = body[g + step], v2 = body[g + 2 * step], v3 = body[g + 3 * step];
-        consider4(v0, head + 4 * g);
-        consider4(v1, head + 4 * (g + step));
-        consider4(v2, head + 4 * (g + 2 * step));
-        consider4(v3, head + 4 * (g + 3 * step));
+        const uint32_t nspan = span + 4 * step;
+        const bool have_next = nspan + 4 * step <= g1;
+        float4 n0, n1, n2, n3;
+        n0 = n1 = n2 = n3 = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (have_next) {
+            const uint32_t gn = nspan + threadIdx.x;
+            n0 = body[gn];
+            n1 = body[gn + step];
+            n2 = body[gn + 2 * step];
+            n3 = body[gn + 3 * step];
+        }
+        consider4(cur0, head + 4 * g);
+        consider4(cur1, head + 4 * (g + step));
+        consider4(cur2, head + 4 * (g + 2 * step));
+        consider4(cur3, head + 4 * (g + 3 * step));
+        cur0 = n0;
+        cur1 = n1;
+        cur2 = n2;
+        cur3 = n3;
+        span = nspan;
+        have = have_next;
     }
     for (; span < g1; span += step) {
         const uint32_t g = span + threadIdx.x;
