@@ -4,15 +4,20 @@
 //   * every (score, column) pair is packed into one 64-bit unsigned word, order-preserving for the score in the high half
 //     and the complemented column in the low half, so "largest word" == "highest score, then lowest column": the whole
 //     selection runs on unsigned 64-bit max/min and the result order is total and reproducible;
-//   * each wavefront streams 128-bit loads of its share of the row and keeps a running top-L list (L = 64, 128 or 256
-//     >= k) in registers, one to four words per lane, sorted descending across (register, lane);
-//   * a score enters only if it beats the list's current k-th word; survivors are compacted with a 64-bit ballot into a
-//     per-wave LDS staging area and, once L of them are waiting, bitonic-sorted (cross-lane exchanges) and merged into the
-//     register list, which tightens the threshold;
+//   * each wavefront streams 128-bit loads of its share of the row, two spans of eight loads per lane in flight, and keeps
+//     a running top-L list (L = 64, 128 or 256 >= k) in registers, one to four words per lane, sorted descending across
+//     (register, lane);
+//   * a score enters only if it beats the list's current k-th word; the common case costs three vector instructions per
+//     16-byte group; survivors are compacted with a 64-bit ballot into a per-wave LDS staging area and, once L of them are
+//     waiting, bitonic-sorted (cross-lane exchanges) and merged into the register list, which tightens the threshold;
+//   * for k <= 32 the threshold is primed before the scan from the k-th best of the lanes' first-span maxima (a binary
+//     search over key bits), so a 27k-column row stages about forty words, no wave ever sorts, and the final order comes
+//     from counting, for each staged word, how many staged words are larger;
+//   * the kernel is bound by instruction issue as much as by HBM (four waves per SIMD run the same phases in step), so the
+//     code keeps rarely-taken work (packing, filter lookups) inside wave-uniform branches;
 //   * the filter (items to multiply, normally by 0, e.g. the sample's own inputs) is a per-segment bitmap in LDS:
-//     listed columns are dropped from the scan and re-injected once with score * multiplier;
-//   * the four wave lists are merged through LDS; rows split over several segments write packed partial lists that a
-//     second small kernel merges.
+//     listed columns are dropped from the scan and injected once, after the scan, with score * multiplier;
+//   * rows split over several segments write packed partial lists that a second small kernel merges.
 #include <algorithm>
 #include "dsx_device.h"
 #include "dsx_internal.h"
@@ -23,19 +28,45 @@ constexpr int kTopkThreads = 256;
 constexpr int kTopkWaves = kTopkThreads / kWave;
 constexpr uint32_t kMaxBitmapBits = 256 * 1024;   // 32 KiB of LDS per workgroup
 
-__device__ __forceinline__ uint64_t pack_score(float key, uint32_t col)
+// Unsigned key with the order of the scores (NaN patterns land above +inf or below -inf; callers keep NaN out).
+__device__ __forceinline__ uint32_t score_key(float key)
 {
     key += 0.0f;   // -0.0 -> +0.0 so that both zeros tie and fall back to the column order
     uint32_t u = __float_as_uint(key);
     u ^= (uint32_t)((int32_t)u >> 31) | 0x80000000u;
-    return ((uint64_t)u << 32) | (uint32_t)~col;
+    return u;
+}
+
+__device__ __forceinline__ float key_score(uint32_t u)
+{
+    u ^= ((u >> 31) - 1u) | 0x80000000u;
+    return __uint_as_float(u);
+}
+
+__device__ __forceinline__ uint64_t pack_score(float key, uint32_t col)
+{
+    return ((uint64_t)score_key(key) << 32) | (uint32_t)~col;
+}
+
+// Largest t such that at least k of the wave's 64*N keys are >= t: the k-th largest key (0 if k > 64*N).  A binary
+// search over the 32 key bits; each step is one vector compare per key and scalar bookkeeping.
+template <int N> __device__ __forceinline__ uint32_t wave_kth_key(const uint32_t (&key)[N], uint32_t k)
+{
+    uint32_t t = 0;
+#pragma unroll 1
+    for (int bit = 31; bit >= 0; bit--) {
+        const uint32_t cand = t | (1u << bit);
+        uint32_t cnt = 0;
+#pragma unroll
+        for (int n = 0; n < N; n++) cnt += (uint32_t)__popcll(__ballot(key[n] >= cand));
+        if (cnt >= k) t = cand;
+    }
+    return t;
 }
 
 __device__ __forceinline__ void unpack_score(uint64_t p, float& key, uint32_t& col)
 {
-    uint32_t u = (uint32_t)(p >> 32);
-    u ^= ((u >> 31) - 1u) | 0x80000000u;
-    key = __uint_as_float(u);
+    key = key_score((uint32_t)(p >> 32));
     col = ~(uint32_t)p;
 }
 
@@ -117,12 +148,14 @@ template <int R> __device__ __forceinline__ void bitonic_merge_desc(uint64_t (&v
 // Running top-L list of one wavefront plus its LDS staging area.
 template <int R> struct WaveTopK {
     static constexpr int L = kWave * R;
-    static constexpr int kStageWords = L + kWave;
+    static constexpr int kBurst = 5 * kWave;            // most words staged between two checks of the fill level
+    static constexpr int kStageWords = L + kBurst;
 
     uint64_t q[R];        // sorted descending over position r*64 + lane; 0 = empty slot
     uint64_t thr;         // current k-th word: candidates must be strictly larger
     float thr_key;        // its score: cheap first test is score >= thr_key
     uint32_t count;       // staged candidates (wave-uniform)
+    bool flushed;         // the register list holds something
     uint64_t* stage;      // LDS, kStageWords words, private to this wave
     uint32_t lane;
     uint32_t k;
@@ -134,6 +167,7 @@ template <int R> struct WaveTopK {
         thr = 0;
         thr_key = -__builtin_inff();
         count = 0;
+        flushed = false;
         stage = stage_;
         lane = lane_;
         k = k_;
@@ -155,38 +189,70 @@ template <int R> struct WaveTopK {
         for (int r = 0; r < R; r++) q[r] = umax64(q[r], c[r]);   // top L of the union, bitonic
         bitonic_merge_desc<R>(q, lane);
         // k-th word -> threshold
+        flushed = true;
         const uint32_t kr = (k - 1) / kWave, kl = (k - 1) % kWave;
         uint64_t t = q[0];
 #pragma unroll
         for (int r = 1; r < R; r++) t = (kr == (uint32_t)r) ? q[r] : t;
-        thr = shfl_u64(t, (int)kl);
-        if (thr != 0) {
-            float key;
-            uint32_t col;
-            unpack_score(thr, key, col);
-            thr_key = key;
-        }
-        // keep what did not fit
+        raise_threshold(shfl_u64(t, (int)kl));
+        // keep what did not fit: move it to the front, 64 words at a time (source and destination of one step never overlap
+        // because L >= 64, and later sources lie above every earlier destination)
         const uint32_t rest = (count > (uint32_t)L) ? count - L : 0;
-        uint64_t keep = 0;
-        if (lane < rest) keep = stage[L + lane];
-        __builtin_amdgcn_wave_barrier();
-        if (lane < rest) stage[lane] = keep;
+        for (uint32_t i = 0; i < rest; i += kWave) {
+            uint64_t keep = 0;
+            if (i + lane < rest) keep = stage[L + i + lane];
+            __builtin_amdgcn_wave_barrier();
+            if (i + lane < rest) stage[i + lane] = keep;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
         count = rest;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
     }
 
-    // Offer one word per lane (valid lanes only).  All 64 lanes must call this together.
-    __device__ __forceinline__ void offer(bool valid, uint64_t word)
+    // Words at or below t can no longer reach the top k.
+    __device__ __forceinline__ void raise_threshold(uint64_t t)
+    {
+        if (t > thr) {
+            thr = t;
+            float key;
+            uint32_t col;
+            unpack_score(t, key, col);
+            thr_key = key;
+        }
+    }
+
+    // Every word whose score key is below t can no longer reach the top k (t must be the key of a real score).
+    __device__ __forceinline__ void prime(uint32_t t)
+    {
+        const uint64_t w = ((uint64_t)t << 32) - 1;
+        if (w > thr) {
+            thr = w;
+            thr_key = key_score(t);
+        }
+    }
+
+    // Stage the lanes' words that beat the threshold.  All 64 lanes must call this together.  Nothing is merged here: after
+    // at most five calls the caller runs drain(), which keeps count < L between bursts.
+    __device__ __forceinline__ void stage_only(bool valid, uint64_t word)
     {
         const bool cand = valid && (word > thr);
         const uint64_t m = __ballot(cand);
         if (m == 0) return;
-        const uint64_t below = m & ((1ull << lane) - 1ull);
-        if (cand) stage[count + __popcll(below)] = word;
+        const uint32_t before = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+        if (cand) stage[count + before] = word;
         count += (uint32_t)__popcll(m);
-        if (count >= (uint32_t)L) flush();
+    }
+
+    __device__ __forceinline__ void drain()
+    {
+        while (count >= (uint32_t)L) flush();
+    }
+
+    // Offer one word per lane (valid lanes only) and merge when L are waiting.
+    __device__ __forceinline__ void offer(bool valid, uint64_t word)
+    {
+        stage_only(valid, word);
+        drain();
     }
 
     __device__ __forceinline__ void finish()
@@ -264,50 +330,82 @@ __global__ __launch_bounds__(kTopkThreads) void topk_scan_kernel(TopKArgs a)
     List list;
     list.init(sStage[wave], lane, a.k);
 
-    // Software pipeline: the first four 16-byte groups of this lane are requested before the filter is built (its chain of
-    // dependent loads would otherwise sit in front of the scan), and inside the loop the next four are requested before the
-    // current four are examined.
+    // Software pipeline: the lane's first 2 * CH 16-byte groups are requested before anything else happens (the filter's
+    // chain of dependent loads would otherwise sit in front of the scan), and inside the loop two spans are in flight while
+    // one is examined.  Groups beyond the segment are filled with NaN, which fails every comparison below.
+    constexpr int CH = 8;
     const float4* body = reinterpret_cast<const float4*>(row + head);
     const uint32_t step = kTopkThreads;
-    uint32_t span = g0;   // block-uniform
-    bool have = span + 4 * step <= g1;
-    float4 cur0, cur1, cur2, cur3;
-    cur0 = cur1 = cur2 = cur3 = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (have) {
-        const uint32_t g = span + threadIdx.x;
-        cur0 = body[g];
-        cur1 = body[g + step];
-        cur2 = body[g + 2 * step];
-        cur3 = body[g + 3 * step];
+    auto load_span = [&](float4 (&d)[CH], uint32_t first) {   // first: block-uniform group number
+        const uint32_t g = first + threadIdx.x;
+        if (first + CH * step <= g1) {
+#pragma unroll
+            for (int u = 0; u < CH; u++) d[u] = body[g + u * step];
+        } else {
+            const float nan = __uint_as_float(0x7fc00000u);
+#pragma unroll
+            for (int u = 0; u < CH; u++) {
+                d[u] = make_float4(nan, nan, nan, nan);
+                if (g + u * step < g1) d[u] = body[g + u * step];
+            }
+        }
+    };
+    // the filter's row range first: it heads a chain of dependent loads
+    uint64_t fs = 0, fe = 0;
+    if constexpr (FILTERED) {
+        uint32_t r = a.position + b;
+        if (a.index) r = a.index[r];
+        fs = a.fstart[r];
+        fe = a.fend[r];
     }
+    uint32_t span = g0;
+    float4 cur[CH], nxt[CH];
+    load_span(cur, span);
 
+    // Filter, part one: mark the listed columns in the bitmap, note which lanes hold a listed column in their first CH groups
+    // (they sit out the priming below), and request the scores of the first kFU * 256 listed columns.  The listed items
+    // themselves are injected after the scan, when the threshold is tight and nearly all of them fail the first compare.
+    // Vector loads complete in the order they were issued, so the column numbers are requested between the first and the
+    // second span: waiting for them then costs no more than waiting for the first span, which priming needs anyway, and the
+    // listed scores (requested last) are not waited for until the scan is over.
+    constexpr int kFU = 4;
+    __shared__ uint32_t sTaint[kTopkThreads / 4];   // one byte per lane: bit u = group u of the first span holds a listed column
+    uint32_t fcol[kFU];
+    float fm[kFU], fv[kFU];
+    if constexpr (FILTERED) {
+#pragma unroll
+        for (int u = 0; u < kFU; u++) {
+            const uint64_t t = fs + (uint64_t)u * kTopkThreads + threadIdx.x;
+            fcol[u] = 0xffffffffu;
+            fm[u] = 0.0f;   // utils/Filters.cpp:62 with the default multiplier
+            if (t < fe) {
+                fcol[u] = a.fidx[t];
+                if (a.fmul) fm[u] = a.fmul[t];
+            }
+        }
+    }
+    load_span(nxt, span + CH * step);
     if constexpr (FILTERED) {
         const uint32_t words = (hi - lo + 31) / 32;
         for (uint32_t i = threadIdx.x; i < words; i += kTopkThreads) sBitmap[i] = 0;
+        if (threadIdx.x < kTopkThreads / 4) sTaint[threadIdx.x] = 0;
         __syncthreads();
-        uint32_t r = a.position + b;
-        if (a.index) r = a.index[r];
-        const uint64_t fs = a.fstart[r], fe = a.fend[r];
-        // Mark the listed columns; the lane that sets a bit first owns the entry and injects score * multiplier.
-        for (uint64_t base = fs; base < fe; base += kTopkThreads) {
-            const uint64_t t = base + threadIdx.x;
-            bool own = false;
-            uint64_t word = 0;
-            if (t < fe) {
-                const uint32_t col = a.fidx[t];
-                if (col >= lo && col < hi) {
-                    const uint32_t bit = 1u << ((col - lo) & 31);
-                    const uint32_t old = atomicOr(&sBitmap[(col - lo) >> 5], bit);
-                    if (!(old & bit)) {
-                        const float mul = a.fmul ? a.fmul[t] : 0.0f;
-                        const float v = mul * row[col];           // utils/Filters.cpp:62
-                        own = !(v != v);                          // NaN never enters (it fails every comparison)
-                        word = pack_score(v, col);
-                    }
+        auto mark = [&](uint32_t c) {
+            if (c >= lo && c < hi) {
+                atomicOr(&sBitmap[(c - lo) >> 5], 1u << ((c - lo) & 31));
+                if (c >= head && c < tail0) {
+                    const uint32_t gi = (c - head) / 4 - g0;
+                    if (gi < CH * step) atomicOr(&sTaint[(gi % step) >> 2], 1u << (((gi % step) & 3) * 8 + gi / step));
                 }
             }
-            list.offer(own, word);
+        };
+#pragma unroll
+        for (int u = 0; u < kFU; u++) {
+            fv[u] = 0.0f;
+            if (fcol[u] >= lo && fcol[u] < hi) fv[u] = row[fcol[u]];
+            mark(fcol[u]);
         }
+        for (uint64_t t = fs + (uint64_t)kFU * kTopkThreads + threadIdx.x; t < fe; t += kTopkThreads) mark(a.fidx[t]);
         __syncthreads();
     }
 
@@ -319,61 +417,92 @@ __global__ __launch_bounds__(kTopkThreads) void topk_scan_kernel(TopKArgs a)
         }
     };
 
-    auto consider4 = [&](const float4& v, uint32_t col) {
-        const float t = list.thr_key;
-        const bool any = (v.x >= t) | (v.y >= t) | (v.z >= t) | (v.w >= t);
-        if (__ballot(any) == 0) return;
-        const float e[4] = {v.x, v.y, v.z, v.w};
+    // Priming (k <= 32): before anything is admitted, every lane takes the best score of its first CH groups.  The k-th
+    // best of a wave's 64 lane maxima is a score that at least k unfiltered items reach, so nothing below it can be in the
+    // result; the k-th best of the 4k scores the four waves publish is a bound for the whole workgroup.  It is found by
+    // binary search on the key bits (no sorting), and the scan then admits a few dozen items per row instead of a few
+    // hundred.  Groups that hold a listed column are left out, and a lane with nothing else contributes -inf, which only
+    // weakens the bound.
+    if (R == 1 && a.k <= 32 && g0 < g1) {
+        __shared__ uint32_t sPrime[kTopkWaves][32];
+        float m = -__builtin_inff();
+        uint32_t taint = 0;
+        if constexpr (FILTERED) taint = (sTaint[threadIdx.x >> 2] >> ((threadIdx.x & 3) * 8)) & 0xffu;
+#pragma unroll
+        for (int u = 0; u < CH; u++) {
+            const float gm = fmaxf(fmaxf(cur[u].x, cur[u].y), fmaxf(cur[u].z, cur[u].w));   // fmaxf drops NaN
+            m = fmaxf(m, ((taint >> u) & 1u) ? -__builtin_inff() : gm);
+        }
+        const uint32_t key[1] = {score_key(m)};
+        const uint32_t tw = wave_kth_key<1>(key, a.k);
+        const bool pub = key[0] >= tw;   // at least k lanes
+        const uint64_t pm = __ballot(pub);
+        const uint32_t pos = __builtin_amdgcn_mbcnt_hi((uint32_t)(pm >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)pm, 0u));
+        if (pub && pos < a.k) sPrime[wave][pos] = key[0];
+        __syncthreads();
+        uint32_t all[2];
+#pragma unroll
+        for (int n = 0; n < 2; n++) {
+            const uint32_t i = n * kWave + lane;
+            all[n] = (i < kTopkWaves * a.k) ? sPrime[i / a.k][i % a.k] : 0u;
+        }
+        const uint32_t t = wave_kth_key<2>(all, a.k);
+        if (t > score_key(-__builtin_inff())) list.prime(t);
+    }
+
+    // The four scores of one 16-byte group; at most 4 * 64 words are staged.
+    auto stage_group = [&](const float4& v, uint32_t col) {
+        float e[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int c = 0; c < 4; c++) {
+            asm volatile("" : "+v"(e[c]));   // keeps the packing below inside the (rarely taken) branch instead of hoisted for all groups
             bool ok = e[c] >= list.thr_key;
-            if (ok) ok = !filtered_out(col + c);
-            list.offer(ok, pack_score(e[c], col + c));
+            if (__ballot(ok) == 0) continue;
+            if constexpr (FILTERED) {
+                if (ok) ok = !filtered_out(col + c);
+            }
+            list.stage_only(ok, pack_score(e[c], col + c));
         }
     };
+    static_assert(CH == 8, "the scan selects among eight groups");
+    static_assert(List::kBurst >= 4 * kWave, "a group stages up to 256 words between drains");
 
-    // Body: the block walks the segment in 4 KiB spans, wave w takes the w-th KiB of each span.
-    while (have) {
-        const uint32_t g = span + threadIdx.x;
-        const uint32_t nspan = span + 4 * step;
-        const bool have_next = nspan + 4 * step <= g1;
-        float4 n0, n1, n2, n3;
-        n0 = n1 = n2 = n3 = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (have_next) {
-            const uint32_t gn = nspan + threadIdx.x;
-            n0 = body[gn];
-            n1 = body[gn + step];
-            n2 = body[gn + 2 * step];
-            n3 = body[gn + 3 * step];
-        }
-        consider4(cur0, head + 4 * g);
-        consider4(cur1, head + 4 * (g + step));
-        consider4(cur2, head + 4 * (g + 2 * step));
-        consider4(cur3, head + 4 * (g + 3 * step));
-        cur0 = n0;
-        cur1 = n1;
-        cur2 = n2;
-        cur3 = n3;
-        span = nspan;
-        have = have_next;
-    }
-    for (; span < g1; span += step) {
-        const uint32_t g = span + threadIdx.x;
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        const bool in = g < g1;
-        if (in) v = body[g];
-        const float t = list.thr_key;
-        const bool any = in && ((v.x >= t) | (v.y >= t) | (v.z >= t) | (v.w >= t));
-        if (__ballot(any) == 0) continue;
-        const float e[4] = {v.x, v.y, v.z, v.w};
-        const uint32_t col = head + 4 * g;
+    // Body: the block walks the segment in spans of CH * 4 KiB, wave w takes the w-th KiB of each 4 KiB.  The common case
+    // costs three vector instructions per group (maximum of four, one compare); groups with a survivor somewhere in the wave
+    // are then walked one at a time.
+    while (span < g1) {
+        const uint32_t gbase = span + threadIdx.x;
+        uint32_t hot = 0;
+        {
+            const float t = list.thr_key;
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            bool ok = in && (e[c] >= list.thr_key);
-            if (ok) ok = !filtered_out(col + c);
-            list.offer(ok, pack_score(e[c], col + c));
+            for (int u = 0; u < CH; u++) {
+                const float m = fmaxf(fmaxf(cur[u].x, cur[u].y), fmaxf(cur[u].z, cur[u].w));
+                if (__ballot(m >= t) != 0) hot |= 1u << u;
+            }
         }
+        while (hot != 0) {
+            const int u = __ffs(hot) - 1;
+            hot &= hot - 1;
+            const uint32_t col = head + 4 * (gbase + (uint32_t)u * step);
+            switch (u) {
+            case 0: stage_group(cur[0], col); break;
+            case 1: stage_group(cur[1], col); break;
+            case 2: stage_group(cur[2], col); break;
+            case 3: stage_group(cur[3], col); break;
+            case 4: stage_group(cur[4], col); break;
+            case 5: stage_group(cur[5], col); break;
+            case 6: stage_group(cur[6], col); break;
+            default: stage_group(cur[7], col); break;
+            }
+            list.drain();
+        }
+#pragma unroll
+        for (int u = 0; u < CH; u++) cur[u] = nxt[u];
+        span += CH * step;
+        load_span(nxt, span + CH * step);
     }
+
     // Head (segment 0) and tail (last segment): at most 3 + 3 columns, taken by wave 0.
     if (wave == 0) {
         uint32_t col = 0xffffffffu;
@@ -385,51 +514,129 @@ __global__ __launch_bounds__(kTopkThreads) void topk_scan_kernel(TopKArgs a)
             v = row[col];
             ok = (v >= list.thr_key) && !filtered_out(col);
         }
-        list.offer(ok, pack_score(v, col));
+        list.stage_only(ok, pack_score(v, col));
     }
-    list.finish();
 
-    // Merge the four wave lists: waves 1..3 publish their first k words, wave 0 takes them as candidates.
-    __syncthreads();
-    // staging areas are idle now; wave w > 0 publishes into its own area
-    if (wave != 0) {
+    // Filter, part two: every listed column is injected once with score * multiplier.  The lane that clears a column's bit
+    // owns it (a column listed twice is injected once).  The bitmap is no longer consulted after the barrier.
+    if constexpr (FILTERED) {
+        __syncthreads();
+        for (uint64_t base = fs; base < fe; base += (uint64_t)kFU * kTopkThreads) {
+            if (base != fs) {
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            const uint32_t p = r * kWave + lane;
-            if (p < a.k) sStage[wave][p] = list.q[r];
+                for (int u = 0; u < kFU; u++) {
+                    const uint64_t t = base + (uint64_t)u * kTopkThreads + threadIdx.x;
+                    fcol[u] = 0xffffffffu;
+                    fm[u] = 0.0f;
+                    if (t < fe) {
+                        fcol[u] = a.fidx[t];
+                        if (a.fmul) fm[u] = a.fmul[t];
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < kFU; u++) {
+                    fv[u] = 0.0f;
+                    if (fcol[u] >= lo && fcol[u] < hi) fv[u] = row[fcol[u]];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kFU; u++) {
+                if (base + (uint64_t)u * kTopkThreads + wave * kWave >= fe) break;   // wave-uniform
+                bool own = false;
+                if (fcol[u] >= lo && fcol[u] < hi) {
+                    const uint32_t bit = 1u << ((fcol[u] - lo) & 31);
+                    own = (atomicAnd(&sBitmap[(fcol[u] - lo) >> 5], ~bit) & bit) != 0;
+                }
+                const float v = fm[u] * fv[u];   // utils/Filters.cpp:62
+                list.stage_only(own && v == v, pack_score(v, fcol[u]));   // NaN never enters (it fails every comparison)
+            }
+            list.drain();
+        }
+    }
+
+    // Merge the four waves into wave 0.  A wave that never had to flush hands over its staged words as they are (they
+    // already sit in LDS); a wave with a register list flushes what is left and publishes its first k words.
+    __shared__ uint32_t sPublished[kTopkWaves];
+    __shared__ uint32_t sFlushed[kTopkWaves];
+    if (wave != 0) {
+        if (list.flushed) {
+            list.finish();
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const uint32_t p = r * kWave + lane;
+                if (p < a.k) sStage[wave][p] = list.q[r];
+            }
+        }
+        if (lane == 0) {
+            sPublished[wave] = list.flushed ? a.k : list.count;
+            sFlushed[wave] = list.flushed ? 1u : 0u;
         }
     }
     __syncthreads();
     if (wave != 0) return;
+
+    uint64_t* partial = a.partial ? a.partial + ((uint64_t)b * a.partial_slots + a.partial_slot0 + seg) * a.k : nullptr;
+    float* keys = a.keys + (uint64_t)b * a.k;
+    uint32_t* values = a.values + (uint64_t)b * a.k;
+    // result slot p of this (row, segment): a packed word for the merge kernel, or the final (score, column) pair
+    auto write_slot = [&](uint32_t p, uint64_t word) {
+        float key = -kMaxValue;   // engine/kernels.cu:3221-3224: unfilled slots
+        uint32_t col = 0;
+        if (word != 0) {
+            unpack_score(word, key, col);
+            col += a.col_offset;
+        }
+        if (partial) {
+            partial[p] = (word != 0) ? ((word & 0xffffffff00000000ull) | (uint32_t)~col) : 0ull;
+        } else {
+            keys[p] = key;
+            values[p] = col;
+        }
+    };
+
+    const uint32_t n0 = list.count, n1 = sPublished[1], n2 = sPublished[2], n3 = sPublished[3];
+    const uint32_t total = n0 + n1 + n2 + n3;
+    const bool any_flushed = list.flushed || (sFlushed[1] | sFlushed[2] | sFlushed[3]) != 0;
+    if (!any_flushed && total <= kWave) {
+        // Common case for small k: at most 64 staged words in all.  Lane i takes the i-th of them and counts how many are
+        // larger; that count is its place in the result, so no sorting network runs at all.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        uint64_t word = 0;
+        if (lane < total) {
+            const uint32_t w = (lane >= n0) + (lane >= n0 + n1) + (lane >= n0 + n1 + n2);
+            const uint32_t first = (w == 0) ? 0 : (w == 1) ? n0 : (w == 2) ? n0 + n1 : n0 + n1 + n2;
+            word = sStage[w][lane - first];
+        }
+        // all words side by side in LDS (wave 0's own staging area is free once its words sit in registers)
+        __builtin_amdgcn_wave_barrier();
+        sStage[0][lane] = word;   // 0 beyond total: never larger than anything
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        uint32_t place = 0;
+        for (uint32_t i = 0; i < total; i += 4) {   // broadcast reads, four in flight; total <= 64 = row length
+            const uint64_t o0 = sStage[0][i], o1 = sStage[0][i + 1], o2 = sStage[0][i + 2], o3 = sStage[0][i + 3];
+            place += (o0 > word ? 1u : 0u) + (o1 > word ? 1u : 0u) + (o2 > word ? 1u : 0u) + (o3 > word ? 1u : 0u);
+        }
+        if (lane < total && place < a.k) write_slot(place, word);
+        if (lane >= total && lane < a.k) write_slot(lane, 0ull);
+        return;
+    }
+
     for (uint32_t w = 1; w < kTopkWaves; w++) {
-        for (uint32_t p0 = 0; p0 < a.k; p0 += kWave) {
+        const uint32_t n = sPublished[w];
+        for (uint32_t p0 = 0; p0 < n; p0 += kWave) {
             const uint32_t p = p0 + lane;
             uint64_t word = 0;
-            if (p < a.k) word = sStage[w][p];
-            // sStage[0] is wave 0's own staging area, distinct from the published lists of waves 1..3
+            if (p < n) word = sStage[w][p];
             list.offer(word != 0, word);
         }
     }
     list.finish();
-
-    if (a.partial) {
-        uint64_t* dst = a.partial + ((uint64_t)b * a.partial_slots + a.partial_slot0 + seg) * a.k;
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            const uint32_t p = r * kWave + lane;
-            if (p < a.k) {
-                uint64_t word = list.q[r];
-                if (word != 0 && a.col_offset != 0) {
-                    float key;
-                    uint32_t col;
-                    unpack_score(word, key, col);
-                    word = (word & 0xffffffff00000000ull) | (uint32_t)~(col + a.col_offset);
-                }
-                dst[p] = word;
-            }
-        }
-    } else {
-        write_final<R>(list.q, lane, a.k, a.col_offset, a.keys + (uint64_t)b * a.k, a.values + (uint64_t)b * a.k);
+    for (int r = 0; r < R; r++) {
+        const uint32_t p = r * kWave + lane;
+        if (p < a.k) write_slot(p, list.q[r]);
     }
 }
 
