@@ -26,6 +26,35 @@ import __graft_entry__ as entry  # noqa: E402
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP32_MFMA_PEAK_TF = 157.3    # MI355X dense fp32 matrix, published
 
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), scaled by what the same counters
+# read for a plain 256 MiB device-to-device copy (FETCH_SIZE reads half of the bytes, factor 2.0; WRITE_SIZE factor 1.0).
+# Measured on the cfg2 workload; the summary with the commands is profiles/pmc_cfg2_hbm_traffic.md.
+MEASURED_TRAFFIC = {
+    "cfg2-catalogue-27278": {
+        "sparse_z_kernel": {"fetch": 15080 * 1024 * 2.0, "write": 512 * 1024 * 1.0},
+        "fc_gemm_kernel[1024x128x128]": {"fetch": 683 * 1024 * 2.0, "write": 512 * 1024 * 1.0},
+        "fc_gemm_kernel[1024x128x27278]": {"fetch": 11370 * 1024 * 2.0, "write": 142900 * 1024 * 1.0},
+        "topk_scan_kernel": {"fetch": 58550 * 1024 * 2.0, "write": 128 * 1024 * 1.0},
+    },
+}
+
+
+class StdoutToStderr:
+    """Sends everything written to file descriptor 1 (the C++ host layer logs there, like the reference) to stderr, so that
+    the JSON line is the only thing on stdout."""
+
+    def __enter__(self):
+        sys.stdout.flush()
+        self.saved = os.dup(1)
+        os.dup2(2, 1)
+        return self
+
+    def __exit__(self, *exc):
+        sys.stdout.flush()
+        os.dup2(self.saved, 1)
+        os.close(self.saved)
+        return False
+
 
 def time_launches(pkg, lib, fn, reps):
     """Average milliseconds of one call of fn(), measured with HIP events on the library stream over `reps` launches."""
@@ -43,20 +72,35 @@ def network_bench(args, pkg, lib):
     from amazon_dsstne_amd import ATTR_BOOLEAN, ATTR_INDEXED, synth
     from amazon_dsstne_amd.pipeline import DevicePipeline
 
+    from amazon_dsstne_amd.host_api import Network
+
     p = synth.config(args.config)
-    pipe = DevicePipeline(p, lib)
     B, H, N, K = p.batch, p.widths[1], p.widths[-1], p.k
     nnzB = p.batch_nnz()
 
+    # The timed step goes through the C++ host layer, as a DSSTNE caller would: NNNetwork::PredictBatch on the resident input
+    # dataset, then NNNetwork::CalculateFilteredTopK with the sample's own items as the filter.  Inputs, weights and
+    # results stay in HBM.
+    net = Network(p)
+    net.bind_input()
+
+    def step():
+        net.predict_batch(0)
+        net.topk(K, filter_dataset=net.dataset)
     for _ in range(args.warmup):
-        pipe.step()
-    pkg.check(lib.dsx_sync())
+        step()
+    net.sync()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        pipe.step()
-    pkg.check(lib.dsx_sync())
+        step()
+    net.sync()
     t1 = time.perf_counter()
     ms_step = (t1 - t0) * 1e3 / args.steps
+
+    # The same kernels one at a time on the same shapes (raw C ABI of the kernel library, same stream).
+    pipe = DevicePipeline(p, lib)
+    pipe.step()
+    pkg.check(lib.dsx_sync())
 
     # per-kernel figures (HIP events around back-to-back launches of one kernel)
     reps = max(10, min(100, args.steps))
@@ -95,23 +139,36 @@ def network_bench(args, pkg, lib):
     for v in kernels.values():
         v["frac"] = v["achieved"] / v["peak"]
 
+    for n, t in MEASURED_TRAFFIC.get(p.name, {}).items():
+        if n in kernels:
+            kernels[n]["traffic"] = int(t["fetch"] + t["write"])
+
     dominant = max(kernels, key=lambda n: kernels[n]["ms"])
     d = kernels[dominant]
     roofline = {"kernel": dominant, "bound": d["bound"], "achieved": round(d["achieved"], 3), "peak": d["peak"], "unit": d["unit"],
-                "frac": round(d["frac"], 4), "traffic": None, "avg_launch_ms": round(d["ms"], 5)}
+                "frac": round(d["frac"], 4), "traffic": d.get("traffic"), "avg_launch_ms": round(d["ms"], 5)}
+    if args.calibrate_copy:
+        # plain device-to-device copy of known size: what FETCH_SIZE / WRITE_SIZE read for it calibrates the counters
+        nbytes = args.calibrate_copy << 20
+        src = pkg.DeviceArray((nbytes // 4,), np.float32)
+        dst = pkg.DeviceArray((nbytes // 4,), np.float32)
+        for _ in range(3):
+            pkg.check(lib.dsx_memcpy_d2d(dst.ptr, src.ptr, nbytes))
+        pkg.check(lib.dsx_sync())
 
     # CPU baseline: the oracle (scalar C++ restatement of the reference kernels, OpenMP over rows) on whole batches of the
     # same workload, bounded to about 10-20 s.
-    orc = entry.load_oracle()
-    cores = orc.lib().orc_num_threads()
-    secs, nb = 0.0, 0
-    budget = args.cpu_seconds
-    while nb < 1 or (secs < budget and nb < 64):
-        s, _, _, _ = orc.forward(p, 0, B, K, filtered=True)
-        secs += s
-        nb += 1
-    cpu = {"value": round(B * nb / secs, 1), "unit": "samples/s", "cores": cores, "kind": "port",
-           "sample": "%d full batches of %d rows of the same workload (%s), %.1f s" % (nb, B, p.name, secs)}
+    cpu = None
+    if args.cpu_seconds > 0:
+        orc = entry.load_oracle()
+        cores = orc.lib().orc_num_threads()
+        secs, nb = 0.0, 0
+        while secs < args.cpu_seconds and nb < 4096:
+            s, _, _, _ = orc.forward(p, 0, B, K, filtered=True)
+            secs += s
+            nb += 1
+        cpu = {"value": round(B * nb / secs, 1), "unit": "samples/s", "cores": cores, "kind": "port",
+               "sample": "%d passes over one batch of %d rows of the same workload (%s), %.1f s" % (nb, B, p.name, secs)}
 
     out = {
         "metric": "predicted samples/sec (sparse-in -> filtered top-K) at batch %d" % B,
@@ -183,14 +240,16 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=2, help="1..4 = networks of the benchmark definition, 5 = KNN")
     ap.add_argument("--knn-items", type=int, default=2000000)
-    ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget; 0 skips it")
+    ap.add_argument("--calibrate-copy", type=int, default=0, help="also run a plain d2d copy of this many MiB (counter calibration)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (the whole model lives in one MI355X's HBM); --gpus %d is not supported"
                  % args.gpus)
-    pkg = entry.load_package()
-    lib = pkg.init(0)
-    out = knn_bench(args, pkg, lib) if args.config == 5 else network_bench(args, pkg, lib)
+    with StdoutToStderr():
+        pkg = entry.load_package()
+        lib = pkg.init(0)
+        out = knn_bench(args, pkg, lib) if args.config == 5 else network_bench(args, pkg, lib)
     print(json.dumps(out), flush=True)
 
 
