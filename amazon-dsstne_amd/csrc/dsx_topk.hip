@@ -48,18 +48,24 @@ __device__ __forceinline__ uint64_t pack_score(float key, uint32_t col)
     return ((uint64_t)score_key(key) << 32) | (uint32_t)~col;
 }
 
-// Largest t such that at least k of the wave's 64*N keys are >= t: the k-th largest key (0 if k > 64*N).  A binary
-// search over the 32 key bits; each step is one vector compare per key and scalar bookkeeping.
+// A lower bound of the k-th largest of the wave's 64*N keys, exact in its upper 20 bits (0 if k > 64*N): at least k keys are
+// >= the result.  A radix-4 search over key bits 31..12; each step is three vector compares per key and scalar bookkeeping.
+// Twelve bits of slack admit a handful of extra candidates, and save a third of a dependent chain that every wave runs
+// before it can ask for more data.
 template <int N> __device__ __forceinline__ uint32_t wave_kth_key(const uint32_t (&key)[N], uint32_t k)
 {
     uint32_t t = 0;
 #pragma unroll 1
-    for (int bit = 31; bit >= 0; bit--) {
-        const uint32_t cand = t | (1u << bit);
-        uint32_t cnt = 0;
+    for (int bit = 30; bit >= 12; bit -= 2) {
+        const uint32_t c1 = t | (1u << bit), c2 = t | (2u << bit), c3 = t | (3u << bit);
+        uint32_t n1 = 0, n2 = 0, n3 = 0;
 #pragma unroll
-        for (int n = 0; n < N; n++) cnt += (uint32_t)__popcll(__ballot(key[n] >= cand));
-        if (cnt >= k) t = cand;
+        for (int n = 0; n < N; n++) {
+            n1 += (uint32_t)__popcll(__ballot(key[n] >= c1));
+            n2 += (uint32_t)__popcll(__ballot(key[n] >= c2));
+            n3 += (uint32_t)__popcll(__ballot(key[n] >= c3));
+        }
+        t = (n3 >= k) ? c3 : (n2 >= k) ? c2 : (n1 >= k) ? c1 : t;
     }
     return t;
 }
@@ -304,7 +310,7 @@ __device__ __forceinline__ void write_final(const uint64_t (&q)[R], uint32_t lan
 }
 
 template <int R, bool FILTERED>
-__global__ __launch_bounds__(kTopkThreads) void topk_scan_kernel(TopKArgs a)
+__global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kernel(TopKArgs a)
 {
     using List = WaveTopK<R>;
     __shared__ uint64_t sStage[kTopkWaves][List::kStageWords];
@@ -361,6 +367,14 @@ __global__ __launch_bounds__(kTopkThreads) void topk_scan_kernel(TopKArgs a)
     uint32_t span = g0;
     float4 cur[CH], nxt[CH];
     load_span(cur, span);
+    // Head (segment 0) and tail (last segment): at most 3 + 3 columns, taken by wave 0 and examined after the scan.
+    uint32_t ht_col = 0xffffffffu;
+    float ht_val = 0.0f;
+    if (wave == 0) {
+        if (seg == 0 && lane < head) ht_col = lane;
+        if (seg == a.segments - 1 && lane >= 32 && (lane - 32) < a.width - tail0) ht_col = tail0 + (lane - 32);
+        if (ht_col != 0xffffffffu) ht_val = row[ht_col];
+    }
 
     // Filter, part one: mark the listed columns in the bitmap, note which lanes hold a listed column in their first CH groups
     // (they sit out the priming below), and request the scores of the first kFU * 256 listed columns.  The listed items
@@ -503,18 +517,10 @@ __global__ __launch_bounds__(kTopkThreads) void topk_scan_kernel(TopKArgs a)
         load_span(nxt, span + CH * step);
     }
 
-    // Head (segment 0) and tail (last segment): at most 3 + 3 columns, taken by wave 0.
+    // Head and tail columns (requested at the start of the kernel).
     if (wave == 0) {
-        uint32_t col = 0xffffffffu;
-        if (seg == 0 && lane < head) col = lane;
-        if (seg == a.segments - 1 && lane >= 32 && (lane - 32) < a.width - tail0) col = tail0 + (lane - 32);
-        bool ok = col != 0xffffffffu;
-        float v = 0.0f;
-        if (ok) {
-            v = row[col];
-            ok = (v >= list.thr_key) && !filtered_out(col);
-        }
-        list.stage_only(ok, pack_score(v, col));
+        const bool ok = (ht_col != 0xffffffffu) && (ht_val >= list.thr_key) && !filtered_out(ht_col);
+        list.stage_only(ok, pack_score(ht_val, ht_col));
     }
 
     // Filter, part two: every listed column is injected once with score * multiplier.  The lane that clears a column's bit
@@ -597,29 +603,34 @@ __global__ __launch_bounds__(kTopkThreads) void topk_scan_kernel(TopKArgs a)
     const uint32_t n0 = list.count, n1 = sPublished[1], n2 = sPublished[2], n3 = sPublished[3];
     const uint32_t total = n0 + n1 + n2 + n3;
     const bool any_flushed = list.flushed || (sFlushed[1] | sFlushed[2] | sFlushed[3]) != 0;
-    if (!any_flushed && total <= kWave) {
-        // Common case for small k: at most 64 staged words in all.  Lane i takes the i-th of them and counts how many are
-        // larger; that count is its place in the result, so no sorting network runs at all.
+    if (!any_flushed && total <= 2 * kWave) {
+        // Common case for small k: at most 128 staged words in all.  Lane i takes the i-th (and the 64 + i-th) of them and
+        // counts how many are larger; that count is its place in the result, so no sorting network runs at all.
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        uint64_t word = 0;
-        if (lane < total) {
-            const uint32_t w = (lane >= n0) + (lane >= n0 + n1) + (lane >= n0 + n1 + n2);
+        auto fetch = [&](uint32_t i) -> uint64_t {
+            if (i >= total) return 0ull;   // never larger than anything
+            const uint32_t w = (i >= n0) + (i >= n0 + n1) + (i >= n0 + n1 + n2);
             const uint32_t first = (w == 0) ? 0 : (w == 1) ? n0 : (w == 2) ? n0 + n1 : n0 + n1 + n2;
-            word = sStage[w][lane - first];
-        }
+            return sStage[w][i - first];
+        };
+        const bool two = total > kWave;   // wave-uniform
+        const uint64_t word0 = fetch(lane), word1 = two ? fetch(kWave + lane) : 0ull;
         // all words side by side in LDS (wave 0's own staging area is free once its words sit in registers)
         __builtin_amdgcn_wave_barrier();
-        sStage[0][lane] = word;   // 0 beyond total: never larger than anything
+        sStage[0][lane] = word0;
+        sStage[0][kWave + lane] = word1;
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        uint32_t place = 0;
-        for (uint32_t i = 0; i < total; i += 4) {   // broadcast reads, four in flight; total <= 64 = row length
+        uint32_t place0 = 0, place1 = 0;
+        for (uint32_t i = 0; i < total; i += 4) {   // broadcast reads, four in flight; the row has room beyond 128 + 3
             const uint64_t o0 = sStage[0][i], o1 = sStage[0][i + 1], o2 = sStage[0][i + 2], o3 = sStage[0][i + 3];
-            place += (o0 > word ? 1u : 0u) + (o1 > word ? 1u : 0u) + (o2 > word ? 1u : 0u) + (o3 > word ? 1u : 0u);
+            place0 += (o0 > word0 ? 1u : 0u) + (o1 > word0 ? 1u : 0u) + (o2 > word0 ? 1u : 0u) + (o3 > word0 ? 1u : 0u);
+            if (two) place1 += (o0 > word1 ? 1u : 0u) + (o1 > word1 ? 1u : 0u) + (o2 > word1 ? 1u : 0u) + (o3 > word1 ? 1u : 0u);
         }
-        if (lane < total && place < a.k) write_slot(place, word);
-        if (lane >= total && lane < a.k) write_slot(lane, 0ull);
+        if (word0 != 0 && place0 < a.k) write_slot(place0, word0);
+        if (word1 != 0 && place1 < a.k) write_slot(place1, word1);
+        for (uint32_t p = total + lane; p < a.k; p += kWave) write_slot(p, 0ull);
         return;
     }
 
