@@ -70,6 +70,7 @@ SIGNATURES = {
     "dsx_sparse_layer_forward": [_u32, _u32, _u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32,
                                  C.POINTER(ActParams), _vp],
     "dsx_fc_forward": [_vp, _u32, _vp, _int, _vp, _vp, _u32, _u32, _u32, _u32, _int, _u32, C.POINTER(ActParams)],
+    "dsx_fc_forward_segmax": [_vp, _u32, _vp, _int, _vp, _vp, _u32, _u32, _u32, _u32, _u32, C.POINTER(ActParams), _vp, C.POINTER(_u32)],
     "dsx_activation": [_vp, _u32, _u32, _u32, C.POINTER(ActParams)],
     "dsx_add_buffers": [_vp, _vp, _u64],
     "dsx_topk": [_vp, _vp, _vp, _u32, _u32, _u32],
@@ -77,6 +78,7 @@ SIGNATURES = {
     "dsx_topk_kv_u32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32],
     "dsx_knn_topk": [_vp, _vp, _vp, _u32, _u32, _u32, _u32],
     "dsx_topk_filtered": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp],
+    "dsx_topk_guided": [_vp, _vp, _vp, _u32, _u32, _u32, _vp, _u32, _u32, _vp, _vp, _vp, _vp, _vp],
     "dsx_knn_search": [_vp, _u32, _u32, _u32, _vp, _u32, _u32, _vp, _vp, _vp, _sz, C.POINTER(_f32)],
 }
 SPECIAL_RESTYPES = {"dsx_last_error": C.c_char_p, "dsx_stream": C.c_void_p, "dsx_knn_workspace_bytes": C.c_size_t}

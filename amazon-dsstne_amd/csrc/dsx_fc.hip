@@ -26,6 +26,8 @@ struct FcArgs {
     uint32_t tiles_m, tiles_n;
     int accumulate;
     uint32_t act;
+    float* seg_max;      // optional: [batch][nseg] maxima of the activated outputs over 64-column segments
+    uint32_t nseg;
     float slope, alpha, lambda;
 };
 
@@ -238,6 +240,15 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
     }
 
     // Epilogue: accumulator register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 block.
+    // With seg_max set (128 x 128 tiles only), every wavefront also reduces the 64 columns it owns to one maximum per row:
+    // a later top-K can then skip the column segments that cannot hold a result.
+    constexpr bool kCanSegMax = (MI == 2 && NI == 2);
+    const bool want_max = kCanSegMax && a.seg_max != nullptr;
+    float smax[kCanSegMax ? 32 : 1];
+    if constexpr (kCanSegMax) {
+#pragma unroll
+        for (int q = 0; q < 32; q++) smax[q] = -__builtin_inff();
+    }
     const bool full_tile = (row0 + BM <= a.batch) && (col0 + BN <= a.n);
     if (full_tile) {
 #pragma unroll
@@ -252,29 +263,55 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
                     float* dst = base + (uint64_t)(8 * (v / 4) + (v % 4)) * a.ldz;
                     float x = acc[i][j][v] + bias;
                     if (a.accumulate) x += *dst;
-                    *dst = activate<ACT>(x, a.slope, a.alpha, a.lambda);
+                    const float y = activate<ACT>(x, a.slope, a.alpha, a.lambda);
+                    *dst = y;
+                    if constexpr (kCanSegMax) smax[i * 16 + v] = fmaxf(smax[i * 16 + v], y);
                 }
             }
         }
-        return;
-    }
+    } else {
 #pragma unroll
-    for (int j = 0; j < NI; j++) {
-        const uint32_t c = col0 + wn * 32 * NI + j * 32 + l32;
-        if (c >= a.n) continue;
-        const float bias = a.bias ? a.bias[c] : 0.0f;
+        for (int j = 0; j < NI; j++) {
+            const uint32_t c = col0 + wn * 32 * NI + j * 32 + l32;
+            if (c >= a.n) continue;
+            const float bias = a.bias ? a.bias[c] : 0.0f;
 #pragma unroll
-        for (int i = 0; i < MI; i++) {
+            for (int i = 0; i < MI; i++) {
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const uint32_t r = row0 + wm * 32 * MI + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
-                if (r < a.batch) {
-                    float* dst = a.Z + (uint64_t)r * a.ldz + c;
-                    float x = acc[i][j][v] + bias;
-                    if (a.accumulate) x += *dst;
-                    *dst = activate<ACT>(x, a.slope, a.alpha, a.lambda);
+                for (int v = 0; v < 16; v++) {
+                    const uint32_t r = row0 + wm * 32 * MI + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
+                    if (r < a.batch) {
+                        float* dst = a.Z + (uint64_t)r * a.ldz + c;
+                        float x = acc[i][j][v] + bias;
+                        if (a.accumulate) x += *dst;
+                        const float y = activate<ACT>(x, a.slope, a.alpha, a.lambda);
+                        *dst = y;
+                        if constexpr (kCanSegMax) smax[i * 16 + v] = fmaxf(smax[i * 16 + v], y);
+                    }
                 }
             }
+        }
+    }
+    if constexpr (kCanSegMax) {
+        if (want_max) {
+            // Reduce-scatter over the 32 lanes of each half wave: step s pairs the values whose index differs in bit s, the
+            // lane whose own bit s is set keeps the upper one and hands the other over.  31 exchanges later lane l holds
+            // the maximum of value index q = l % 32, i.e. of one of the wave's 64 rows.
+#pragma unroll
+            for (int s = 4; s >= 0; s--) {
+                const int half = 1 << s;
+                const bool upper = (l32 >> s) & 1;
+#pragma unroll
+                for (int q = 0; q < half; q++) {
+                    const float keep = upper ? smax[q + half] : smax[q];
+                    const float send = upper ? smax[q] : smax[q + half];
+                    smax[q] = fmaxf(keep, __shfl_xor(send, half, 64));
+                }
+            }
+            const int q = l32, i = q >> 4, v = q & 15;
+            const uint32_t r = row0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * lhi + (v & 3);
+            const uint32_t seg = (col0 + wn * 64) / 64;
+            if (r < a.batch && seg < a.nseg) a.seg_max[(uint64_t)r * a.nseg + seg] = smax[0];
         }
     }
 }
@@ -321,8 +358,10 @@ template <int MI, int NI, int BK> static void launch_fc_shape(FcArgs& a, int xv,
 }
 
 int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int transposed, const float* bias, float* Z, uint32_t ldz,
-           uint32_t batch, uint32_t k, uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params)
+           uint32_t batch, uint32_t k, uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params, float* seg_max,
+           uint32_t* seg_width)
 {
+    if (seg_width) *seg_width = 0;
     FcArgs a{};
     a.X = X; a.W = W; a.bias = bias; a.Z = Z;
     a.ldx = ldx; a.ldw = ldw; a.ldz = ldz;
@@ -338,9 +377,14 @@ int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int trans
     else if (!transposed && ((uintptr_t)W % 8) == 0 && (ldw % 2) == 0) wv = 2;
     // Large tiles when they still give every CU a few workgroups, small tiles otherwise.
     const uint64_t big_tiles = (uint64_t)((batch + 127) / 128) * ((n + 127) / 128);
-    if (big_tiles >= (uint64_t)ctx().num_cus * 2)
+    if (big_tiles >= (uint64_t)ctx().num_cus * 2) {
+        if (seg_max && seg_width && !accumulate) {   // maxima of sums still to be accumulated into would be of no use
+            a.seg_max = seg_max;
+            a.nseg = (n + 63) / 64;
+            *seg_width = 64;
+        }
         launch_fc_shape<2, 2, 16>(a, xv, wv, transposed != 0);
-    else
+    } else
         launch_fc_shape<1, 1, 32>(a, xv, wv, transposed != 0);   // few workgroups: deep k-steps, fewer barrier round trips
     DSX_LAUNCH_CHECK("fc_gemm_kernel");
     return DSX_OK;
@@ -395,6 +439,20 @@ int dsx_fc_forward(const float* X, uint32_t ldx, const float* W, int transposed,
     DSX_CHECK_ARG(is_elementwise_activation(activation), "dsx_fc_forward: activation %u is a row operation; pass DSX_ACT_LINEAR and call dsx_activation", activation);
     if (batch == 0) return DSX_OK;
     return fc_run(X, ldx, W, transposed ? k : n, transposed, bias, Z, ldz, batch, k, n, accumulate, activation, params);
+}
+
+int dsx_fc_forward_segmax(const float* X, uint32_t ldx, const float* W, int transposed, const float* bias, float* Z, uint32_t ldz,
+                          uint32_t batch, uint32_t k, uint32_t n, uint32_t activation, const dsx_act_params* params, float* seg_max,
+                          uint32_t* seg_width)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(X && W && Z && seg_max && seg_width, "dsx_fc_forward_segmax: null pointer");
+    DSX_CHECK_ARG(k > 0 && n > 0, "dsx_fc_forward_segmax: k = %u, n = %u", k, n);
+    DSX_CHECK_ARG(ldx >= k && ldz >= n, "dsx_fc_forward_segmax: row pitch smaller than the row (ldx %u < k %u or ldz %u < n %u)", ldx, k, ldz, n);
+    DSX_CHECK_ARG(is_elementwise_activation(activation), "dsx_fc_forward_segmax: activation %u is a row operation", activation);
+    *seg_width = 0;
+    if (batch == 0) return DSX_OK;
+    return fc_run(X, ldx, W, transposed ? k : n, transposed, bias, Z, ldz, batch, k, n, 0, activation, params, seg_max, seg_width);
 }
 
 int dsx_activation(float* unit, uint32_t batch, uint32_t stride, uint32_t activation, const dsx_act_params* params)

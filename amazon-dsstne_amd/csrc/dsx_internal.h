@@ -61,5 +61,6 @@ int topk_run(const float* in, uint32_t pitch, uint32_t width, uint32_t batch, ui
 int topk_merge(const uint64_t* partial, uint32_t slots, uint32_t k, float* keys, uint32_t* values, uint32_t batch);
 // GEMM building block shared with the KNN search (dsx_fc.hip): Z = X.W (+bias, activation), see dsx_fc_forward.
 int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int transposed, const float* bias, float* Z, uint32_t ldz,
-           uint32_t batch, uint32_t k, uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params);
+           uint32_t batch, uint32_t k, uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params,
+           float* seg_max = nullptr, uint32_t* seg_width = nullptr);
 }  // namespace dsx

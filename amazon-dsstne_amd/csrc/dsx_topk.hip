@@ -287,6 +287,9 @@ struct TopKArgs {
     uint64_t* partial;          // [batch][partial_slots][k]
     uint32_t partial_slots;
     uint32_t partial_slot0;     // this launch writes slots partial_slot0 + segment
+    // guided variant: maxima of the row's 64-column segments, left by the producer of `in`
+    const float* seg_max;       // [batch][nseg]
+    uint32_t nseg;
 };
 
 template <int R>
@@ -306,6 +309,103 @@ __device__ __forceinline__ void write_final(const uint64_t (&q)[R], uint32_t lan
             keys[p] = key;
             values[p] = col;
         }
+    }
+}
+
+// End of a (row, segment): merges the lists of the four waves into wave 0 and writes the result (final pairs, or packed words
+// for the merge kernel).  Every lane of the workgroup must call it.
+template <int R>
+__device__ __forceinline__ void finish_row(WaveTopK<R>& list, uint64_t (*sStage)[WaveTopK<R>::kStageWords], const TopKArgs& a,
+                                           uint32_t b, uint32_t seg, uint32_t wave, uint32_t lane)
+{
+    // Merge the four waves into wave 0.  A wave that never had to flush hands over its staged words as they are (they
+    // already sit in LDS); a wave with a register list flushes what is left and publishes its first k words.
+    __shared__ uint32_t sPublished[kTopkWaves];
+    __shared__ uint32_t sFlushed[kTopkWaves];
+    if (wave != 0) {
+        if (list.flushed) {
+            list.finish();
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const uint32_t p = r * kWave + lane;
+                if (p < a.k) sStage[wave][p] = list.q[r];
+            }
+        }
+        if (lane == 0) {
+            sPublished[wave] = list.flushed ? a.k : list.count;
+            sFlushed[wave] = list.flushed ? 1u : 0u;
+        }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+
+    uint64_t* partial = a.partial ? a.partial + ((uint64_t)b * a.partial_slots + a.partial_slot0 + seg) * a.k : nullptr;
+    float* keys = a.keys + (uint64_t)b * a.k;
+    uint32_t* values = a.values + (uint64_t)b * a.k;
+    // result slot p of this (row, segment): a packed word for the merge kernel, or the final (score, column) pair
+    auto write_slot = [&](uint32_t p, uint64_t word) {
+        float key = -kMaxValue;   // engine/kernels.cu:3221-3224: unfilled slots
+        uint32_t col = 0;
+        if (word != 0) {
+            unpack_score(word, key, col);
+            col += a.col_offset;
+        }
+        if (partial) {
+            partial[p] = (word != 0) ? ((word & 0xffffffff00000000ull) | (uint32_t)~col) : 0ull;
+        } else {
+            keys[p] = key;
+            values[p] = col;
+        }
+    };
+
+    const uint32_t n0 = list.count, n1 = sPublished[1], n2 = sPublished[2], n3 = sPublished[3];
+    const uint32_t total = n0 + n1 + n2 + n3;
+    const bool any_flushed = list.flushed || (sFlushed[1] | sFlushed[2] | sFlushed[3]) != 0;
+    if (!any_flushed && total <= 2 * kWave) {
+        // Common case for small k: at most 128 staged words in all.  Lane i takes the i-th (and the 64 + i-th) of them and
+        // counts how many are larger; that count is its place in the result, so no sorting network runs at all.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        auto fetch = [&](uint32_t i) -> uint64_t {
+            if (i >= total) return 0ull;   // never larger than anything
+            const uint32_t w = (i >= n0) + (i >= n0 + n1) + (i >= n0 + n1 + n2);
+            const uint32_t first = (w == 0) ? 0 : (w == 1) ? n0 : (w == 2) ? n0 + n1 : n0 + n1 + n2;
+            return sStage[w][i - first];
+        };
+        const bool two = total > kWave;   // wave-uniform
+        const uint64_t word0 = fetch(lane), word1 = two ? fetch(kWave + lane) : 0ull;
+        // all words side by side in LDS (wave 0's own staging area is free once its words sit in registers)
+        __builtin_amdgcn_wave_barrier();
+        sStage[0][lane] = word0;
+        sStage[0][kWave + lane] = word1;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        uint32_t place0 = 0, place1 = 0;
+        for (uint32_t i = 0; i < total; i += 4) {   // broadcast reads, four in flight; the row has room beyond 128 + 3
+            const uint64_t o0 = sStage[0][i], o1 = sStage[0][i + 1], o2 = sStage[0][i + 2], o3 = sStage[0][i + 3];
+            place0 += (o0 > word0 ? 1u : 0u) + (o1 > word0 ? 1u : 0u) + (o2 > word0 ? 1u : 0u) + (o3 > word0 ? 1u : 0u);
+            if (two) place1 += (o0 > word1 ? 1u : 0u) + (o1 > word1 ? 1u : 0u) + (o2 > word1 ? 1u : 0u) + (o3 > word1 ? 1u : 0u);
+        }
+        if (word0 != 0 && place0 < a.k) write_slot(place0, word0);
+        if (word1 != 0 && place1 < a.k) write_slot(place1, word1);
+        for (uint32_t p = total + lane; p < a.k; p += kWave) write_slot(p, 0ull);
+        return;
+    }
+
+    for (uint32_t w = 1; w < kTopkWaves; w++) {
+        const uint32_t n = sPublished[w];
+        for (uint32_t p0 = 0; p0 < n; p0 += kWave) {
+            const uint32_t p = p0 + lane;
+            uint64_t word = 0;
+            if (p < n) word = sStage[w][p];
+            list.offer(word != 0, word);
+        }
+    }
+    list.finish();
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const uint32_t p = r * kWave + lane;
+        if (p < a.k) write_slot(p, list.q[r]);
     }
 }
 
@@ -560,95 +660,214 @@ __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kern
         }
     }
 
-    // Merge the four waves into wave 0.  A wave that never had to flush hands over its staged words as they are (they
-    // already sit in LDS); a wave with a register list flushes what is left and publishes its first k words.
-    __shared__ uint32_t sPublished[kTopkWaves];
-    __shared__ uint32_t sFlushed[kTopkWaves];
-    if (wave != 0) {
-        if (list.flushed) {
-            list.finish();
+    finish_row<R>(list, sStage, a, b, seg, wave, lane);
+}
+
+// Guided top-K (k <= 32): the producer of the scores also left the maximum of every 64-column segment of every row (the
+// dense layer's epilogue has them in registers anyway).  The k-th largest of a row's segment maxima is a score that at least
+// k items reach, so only segments whose maximum reaches it can hold a result: about k of them.  The kernel reads the
+// row's maxima (1/64 of the row), picks that bound with the same key-bit search the scan uses for priming, and then reads
+// just those segments.  With the filter, a maximum that is the score of a listed column says nothing about the unlisted
+// ones: it is left out of the bound (its segment is still read).  Rows full of ties read more segments and still come out
+// right: the survivors go through the same lists as in the scan.
+constexpr uint32_t kGuidedSegWidth = 64;
+constexpr uint32_t kGuidedMaxSegs = 2048;
+
+template <bool FILTERED>
+__global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a)
+{
+    using List = WaveTopK<1>;
+    constexpr int E = kGuidedMaxSegs / kTopkThreads;   // maxima per lane
+    __shared__ uint64_t sStage[kTopkWaves][List::kStageWords];
+    __shared__ uint32_t sPrime[kTopkWaves][32];
+    __shared__ uint32_t sListCount;
+    extern __shared__ uint32_t sDyn[];   // segments to read [nseg] | best listed score per segment [nseg] | bitmap of listed columns
+    uint32_t* sList = sDyn;
+    uint32_t* sFiltMax = sDyn + a.nseg;
+    uint32_t* sBitmap = sDyn + 2 * a.nseg;
+
+    const uint32_t b = blockIdx.x;
+    const uint32_t wave = threadIdx.x / kWave;
+    const uint32_t lane = threadIdx.x % kWave;
+    const float* row = a.in + (uint64_t)b * a.pitch;
+    List list;
+    list.init(sStage[wave], lane, a.k);
+
+    uint64_t fs = 0, fe = 0;
+    if constexpr (FILTERED) {
+        uint32_t r = a.position + b;
+        if (a.index) r = a.index[r];
+        fs = a.fstart[r];
+        fe = a.fend[r];
+    }
+    uint32_t mk[E];   // keys of this lane's segment maxima; 0 = no such segment
+    {
+        const float* mrow = a.seg_max + (uint64_t)b * a.nseg;
 #pragma unroll
-            for (int r = 0; r < R; r++) {
-                const uint32_t p = r * kWave + lane;
-                if (p < a.k) sStage[wave][p] = list.q[r];
+        for (int e = 0; e < E; e++) {
+            const uint32_t idx = e * kTopkThreads + threadIdx.x;
+            mk[e] = (idx < a.nseg) ? score_key(mrow[idx]) : 0u;
+        }
+    }
+    if (lane < 32) sPrime[wave][lane] = 0;
+    if (threadIdx.x == 0) sListCount = 0;
+
+    constexpr int kFU = 4;
+    uint32_t fcol[kFU];
+    float fm[kFU], fv[kFU];
+    if constexpr (FILTERED) {
+        const uint32_t words = (a.width + 31) / 32;
+        for (uint32_t i = threadIdx.x; i < words; i += kTopkThreads) sBitmap[i] = 0;
+        for (uint32_t i = threadIdx.x; i < a.nseg; i += kTopkThreads) sFiltMax[i] = 0;
+        __syncthreads();
+        auto mark = [&](uint32_t c, float v) {
+            atomicOr(&sBitmap[c >> 5], 1u << (c & 31));
+            if (v == v) atomicMax(&sFiltMax[c / kGuidedSegWidth], score_key(v));   // a NaN is never a segment's maximum
+        };
+#pragma unroll
+        for (int u = 0; u < kFU; u++) {
+            const uint64_t t = fs + (uint64_t)u * kTopkThreads + threadIdx.x;
+            fcol[u] = 0xffffffffu;
+            fm[u] = 0.0f;   // utils/Filters.cpp:62 with the default multiplier
+            if (t < fe) {
+                fcol[u] = a.fidx[t];
+                if (a.fmul) fm[u] = a.fmul[t];
             }
         }
-        if (lane == 0) {
-            sPublished[wave] = list.flushed ? a.k : list.count;
-            sFlushed[wave] = list.flushed ? 1u : 0u;
+#pragma unroll
+        for (int u = 0; u < kFU; u++) {
+            fv[u] = 0.0f;
+            if (fcol[u] < a.width) fv[u] = row[fcol[u]];
+        }
+#pragma unroll
+        for (int u = 0; u < kFU; u++)
+            if (fcol[u] < a.width) mark(fcol[u], fv[u]);
+        for (uint64_t t = fs + (uint64_t)kFU * kTopkThreads + threadIdx.x; t < fe; t += kTopkThreads) {
+            const uint32_t c = a.fidx[t];
+            if (c < a.width) mark(c, row[c]);
         }
     }
     __syncthreads();
-    if (wave != 0) return;
 
-    uint64_t* partial = a.partial ? a.partial + ((uint64_t)b * a.partial_slots + a.partial_slot0 + seg) * a.k : nullptr;
-    float* keys = a.keys + (uint64_t)b * a.k;
-    uint32_t* values = a.values + (uint64_t)b * a.k;
-    // result slot p of this (row, segment): a packed word for the merge kernel, or the final (score, column) pair
-    auto write_slot = [&](uint32_t p, uint64_t word) {
-        float key = -kMaxValue;   // engine/kernels.cu:3221-3224: unfilled slots
-        uint32_t col = 0;
-        if (word != 0) {
-            unpack_score(word, key, col);
-            col += a.col_offset;
-        }
-        if (partial) {
-            partial[p] = (word != 0) ? ((word & 0xffffffff00000000ull) | (uint32_t)~col) : 0ull;
+    auto filtered_out = [&](uint32_t col) -> bool {
+        if constexpr (FILTERED) {
+            return (sBitmap[col >> 5] >> (col & 31)) & 1u;
         } else {
-            keys[p] = key;
-            values[p] = col;
+            return false;
         }
     };
 
-    const uint32_t n0 = list.count, n1 = sPublished[1], n2 = sPublished[2], n3 = sPublished[3];
-    const uint32_t total = n0 + n1 + n2 + n3;
-    const bool any_flushed = list.flushed || (sFlushed[1] | sFlushed[2] | sFlushed[3]) != 0;
-    if (!any_flushed && total <= 2 * kWave) {
-        // Common case for small k: at most 128 staged words in all.  Lane i takes the i-th (and the 64 + i-th) of them and
-        // counts how many are larger; that count is its place in the result, so no sorting network runs at all.
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        auto fetch = [&](uint32_t i) -> uint64_t {
-            if (i >= total) return 0ull;   // never larger than anything
-            const uint32_t w = (i >= n0) + (i >= n0 + n1) + (i >= n0 + n1 + n2);
-            const uint32_t first = (w == 0) ? 0 : (w == 1) ? n0 : (w == 2) ? n0 + n1 : n0 + n1 + n2;
-            return sStage[w][i - first];
-        };
-        const bool two = total > kWave;   // wave-uniform
-        const uint64_t word0 = fetch(lane), word1 = two ? fetch(kWave + lane) : 0ull;
-        // all words side by side in LDS (wave 0's own staging area is free once its words sit in registers)
-        __builtin_amdgcn_wave_barrier();
-        sStage[0][lane] = word0;
-        sStage[0][kWave + lane] = word1;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        uint32_t place0 = 0, place1 = 0;
-        for (uint32_t i = 0; i < total; i += 4) {   // broadcast reads, four in flight; the row has room beyond 128 + 3
-            const uint64_t o0 = sStage[0][i], o1 = sStage[0][i + 1], o2 = sStage[0][i + 2], o3 = sStage[0][i + 3];
-            place0 += (o0 > word0 ? 1u : 0u) + (o1 > word0 ? 1u : 0u) + (o2 > word0 ? 1u : 0u) + (o3 > word0 ? 1u : 0u);
-            if (two) place1 += (o0 > word1 ? 1u : 0u) + (o1 > word1 ? 1u : 0u) + (o2 > word1 ? 1u : 0u) + (o3 > word1 ? 1u : 0u);
+    // The bound: k-th largest of the maxima that are not a listed column's score, first per wave, then over the 4k the waves
+    // publish.  With fewer than k such maxima there is no bound and every segment is read.
+    uint32_t bound = 0;
+    {
+        uint32_t tk[E];
+#pragma unroll
+        for (int e = 0; e < E; e++) {
+            tk[e] = mk[e];
+            if constexpr (FILTERED) {
+                const uint32_t idx = e * kTopkThreads + threadIdx.x;
+                if (idx < a.nseg && sFiltMax[idx] == mk[e]) tk[e] = 0;
+            }
         }
-        if (word0 != 0 && place0 < a.k) write_slot(place0, word0);
-        if (word1 != 0 && place1 < a.k) write_slot(place1, word1);
-        for (uint32_t p = total + lane; p < a.k; p += kWave) write_slot(p, 0ull);
-        return;
+        const uint32_t tw = wave_kth_key<E>(tk, a.k);
+        uint32_t published = 0;   // wave-uniform
+#pragma unroll
+        for (int e = 0; e < E; e++) {
+            const bool pub = tk[e] != 0 && tk[e] >= tw;
+            const uint64_t pm = __ballot(pub);
+            const uint32_t pos = published + __builtin_amdgcn_mbcnt_hi((uint32_t)(pm >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)pm, 0u));
+            if (pub && pos < a.k) sPrime[wave][pos] = tk[e];
+            published += (uint32_t)__popcll(pm);
+        }
+        __syncthreads();
+        uint32_t all[2];
+#pragma unroll
+        for (int n = 0; n < 2; n++) {
+            const uint32_t i = n * kWave + lane;
+            all[n] = (i < kTopkWaves * a.k) ? sPrime[i / a.k][i % a.k] : 0u;
+        }
+        const uint32_t t = wave_kth_key<2>(all, a.k);
+        if (t > score_key(-__builtin_inff())) {
+            bound = t;
+            list.prime(t);
+        }
     }
 
-    for (uint32_t w = 1; w < kTopkWaves; w++) {
-        const uint32_t n = sPublished[w];
-        for (uint32_t p0 = 0; p0 < n; p0 += kWave) {
-            const uint32_t p = p0 + lane;
-            uint64_t word = 0;
-            if (p < n) word = sStage[w][p];
-            list.offer(word != 0, word);
+    // Segments whose maximum (listed or not) reaches the bound.
+#pragma unroll
+    for (int e = 0; e < E; e++) {
+        const uint32_t idx = e * kTopkThreads + threadIdx.x;
+        const bool flagged = idx < a.nseg && mk[e] >= bound;
+        const uint64_t m = __ballot(flagged);
+        if (m == 0) continue;
+        uint32_t base = 0;
+        if (lane == 0) base = atomicAdd(&sListCount, (uint32_t)__popcll(m));
+        base = (uint32_t)__builtin_amdgcn_readfirstlane((int)base);
+        if (flagged) sList[base + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u))] = idx;
+    }
+    __syncthreads();
+
+    // One lane per column of a segment, four segments in flight per wave.
+    const uint32_t count = sListCount;
+    for (uint32_t i0 = wave * 4; i0 < count; i0 += kTopkWaves * 4) {
+        float v[4];
+        uint32_t col[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            v[u] = __uint_as_float(0x7fc00000u);   // NaN fails the compare below
+            col[u] = 0;
+            if (i0 + u < count) {
+                col[u] = sList[i0 + u] * kGuidedSegWidth + lane;
+                if (col[u] < a.width) v[u] = row[col[u]];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            bool ok = v[u] >= list.thr_key;
+            if (__ballot(ok) == 0) continue;
+            if (ok) ok = !filtered_out(col[u]);
+            list.stage_only(ok, pack_score(v[u], col[u]));
+        }
+        list.drain();
+    }
+
+    // Every listed column is injected once with score * multiplier; the lane that clears a column's bit owns it.
+    if constexpr (FILTERED) {
+        __syncthreads();
+        for (uint64_t base = fs; base < fe; base += (uint64_t)kFU * kTopkThreads) {
+            if (base != fs) {
+#pragma unroll
+                for (int u = 0; u < kFU; u++) {
+                    const uint64_t t = base + (uint64_t)u * kTopkThreads + threadIdx.x;
+                    fcol[u] = 0xffffffffu;
+                    fm[u] = 0.0f;
+                    if (t < fe) {
+                        fcol[u] = a.fidx[t];
+                        if (a.fmul) fm[u] = a.fmul[t];
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < kFU; u++) {
+                    fv[u] = 0.0f;
+                    if (fcol[u] < a.width) fv[u] = row[fcol[u]];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kFU; u++) {
+                if (base + (uint64_t)u * kTopkThreads + wave * kWave >= fe) break;   // wave-uniform
+                bool own = false;
+                if (fcol[u] < a.width) {
+                    const uint32_t bit = 1u << (fcol[u] & 31);
+                    own = (atomicAnd(&sBitmap[fcol[u] >> 5], ~bit) & bit) != 0;
+                }
+                const float v = fm[u] * fv[u];   // utils/Filters.cpp:62
+                list.stage_only(own && v == v, pack_score(v, fcol[u]));
+            }
+            list.drain();
         }
     }
-    list.finish();
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-        const uint32_t p = r * kWave + lane;
-        if (p < a.k) write_slot(p, list.q[r]);
-    }
+    finish_row<1>(list, sStage, a, b, 0, wave, lane);
 }
 
 // Second stage: one wavefront per row merges `slots` packed partial lists of k words each.
@@ -792,6 +1011,41 @@ int topk_merge(const uint64_t* partial, uint32_t slots, uint32_t k, float* keys,
     return launch_merge<4>(partial, slots, k, keys, values, batch);
 }
 
+// Guided top-K when it applies (k <= 32, 64-column segments, at most kGuidedMaxSegs of them), the scan otherwise.
+int topk_guided_run(const float* in, uint32_t width, uint32_t batch, uint32_t k, float* keys, uint32_t* values, const float* seg_max,
+                    uint32_t seg_width, uint32_t position, const uint32_t* index, const uint64_t* fstart, const uint64_t* fend,
+                    const uint32_t* fidx, const float* fmul)
+{
+    const bool filtered = fidx != nullptr;
+    const uint32_t nseg = (width + kGuidedSegWidth - 1) / kGuidedSegWidth;
+    size_t lds = (size_t)nseg * 4;
+    if (filtered) lds += (size_t)nseg * 4 + ((size_t)(width + 31) / 32) * 4;
+    if (!seg_max || seg_width != kGuidedSegWidth || k > 32 || nseg > kGuidedMaxSegs || lds > 40 * 1024)
+        return topk_run(in, width, width, batch, k, keys, values, position, index, fstart, fend, fidx, fmul, 0, nullptr, 0, 0, 0);
+    TopKArgs a{};
+    a.in = in;
+    a.pitch = width;
+    a.width = width;
+    a.k = k;
+    a.segments = 1;
+    a.position = position;
+    a.index = index;
+    a.fstart = fstart;
+    a.fend = fend;
+    a.fidx = fidx;
+    a.fmul = fmul;
+    a.keys = keys;
+    a.values = values;
+    a.seg_max = seg_max;
+    a.nseg = nseg;
+    if (filtered)
+        hipLaunchKernelGGL(topk_guided_kernel<true>, dim3(batch), dim3(kTopkThreads), lds, ctx().stream, a);
+    else
+        hipLaunchKernelGGL(topk_guided_kernel<false>, dim3(batch), dim3(kTopkThreads), lds, ctx().stream, a);
+    DSX_LAUNCH_CHECK("topk_guided_kernel");
+    return DSX_OK;
+}
+
 static int check_topk(const char* fn, const float* in, const float* keys, const void* values, uint32_t width, uint32_t k)
 {
     DSX_CHECK_ARG(in && keys && values, "%s: null device pointer", fn);
@@ -837,6 +1091,19 @@ int dsx_topk_filtered(const float* in, float* keys, uint32_t* values, uint32_t b
     if (batch == 0) return DSX_OK;
     return topk_run(in, width, width, batch, k, keys, values, position, index, filter_start, filter_end, filter_index, filter_mul, 0,
                     nullptr, 0, 0, 0);
+}
+
+int dsx_topk_guided(const float* in, float* keys, uint32_t* values, uint32_t batch, uint32_t width, uint32_t k, const float* seg_max,
+                    uint32_t seg_width, uint32_t position, const uint32_t* index, const uint64_t* filter_start,
+                    const uint64_t* filter_end, const uint32_t* filter_index, const float* filter_mul)
+{
+    DSX_REQUIRE_INIT();
+    int rc = check_topk("dsx_topk_guided", in, keys, values, width, k);
+    if (rc) return rc;
+    DSX_CHECK_ARG(!filter_index || (filter_start && filter_end), "dsx_topk_guided: filter_index without filter_start / filter_end");
+    if (batch == 0) return DSX_OK;
+    return topk_guided_run(in, width, batch, k, keys, values, seg_max, seg_width, position, index, filter_start, filter_end,
+                           filter_index, filter_mul);
 }
 
 int dsx_topk_kv_f32(const float* in_keys, const float* in_values, float* keys, float* values, uint32_t batch, uint32_t width, uint32_t k)

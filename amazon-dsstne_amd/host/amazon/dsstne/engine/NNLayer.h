@@ -57,6 +57,10 @@ private:
     vector<NNLayer*> _vIncomingSkip;
     vector<NNLayer*> _vOutgoingSkip;
     unique_ptr<GpuBuffer<NNFloat>> _pbUnit;
+    // Maxima of the 64-unit segments of every row of _pbUnit, left by the dense kernel that produced the current batch
+    // (_segWidth == 0: none): NNNetwork::CalculateTopK then reads only the segments that can hold a result.
+    unique_ptr<GpuBuffer<NNFloat>> _pbSegMax;
+    uint32_t _segWidth = 0;
     int32_t _priority;
 
     NNLayer(NNLayerDescriptor& l, uint32_t batch);

@@ -56,7 +56,12 @@ NNLayer::NNLayer(NNLayerDescriptor& d, uint32_t batch)
 
 NNLayer::~NNLayer() { Deallocate(); }
 
-void NNLayer::Deallocate() { _pbUnit.reset(); }
+void NNLayer::Deallocate()
+{
+    _pbUnit.reset();
+    _pbSegMax.reset();
+    _segWidth = 0;
+}
 
 void NNLayer::SetBatch(uint32_t batch)
 {
@@ -119,6 +124,9 @@ void NNLayer::ForwardPropagate(uint32_t position, uint32_t batch, bool bTraining
     ForwardPropagateFullyConnected(position, batch, bTraining);
 }
 
+// Narrower layers are cheap to scan in full.
+static const uint32_t kSegMaxMinWidth = 8192;
+
 void NNLayer::ForwardPropagateFullyConnected(uint32_t position, uint32_t batch, bool bTraining)
 {
     (void)bTraining;
@@ -131,6 +139,7 @@ void NNLayer::ForwardPropagateFullyConnected(uint32_t position, uint32_t batch, 
     }
     dsx_act_params params = {_RELUSlope, _ELUAlpha, _SELULambda};
     NNFloat* pUnit = GetIncomingUnitBuffer();
+    _segWidth = 0;   // whatever described the previous batch no longer holds
 
     // One source, no skips, elementwise activation: a single fused kernel.
     if (nIn == 1 && _vIncomingSkip.empty() && _activation != SoftMax) {
@@ -140,6 +149,14 @@ void NNLayer::ForwardPropagateFullyConnected(uint32_t position, uint32_t batch, 
         if (src->_bFastSparse) {
             src->_pDataSet->CalculateSparseLayer(position, batch, _stride, wsrc->_pbWeight->_pDevData, w->_pbBias->_pDevData, _activation,
                                                  _RELUSlope, _ELUAlpha, _SELULambda, pUnit);
+        } else if (_kind == Output && _localStride >= kSegMaxMinWidth) {
+            // wide output layer: the kernel also leaves segment maxima for the top-K that usually follows
+            const size_t need = (size_t)_batch * ((_localStride + 63) / 64);
+            if (!_pbSegMax || _pbSegMax->_length < need) _pbSegMax.reset(new GpuBuffer<NNFloat>(need));
+            dsxFatal(dsx_fc_forward_segmax(src->GetUnitBuffer(), src->_stride, wsrc->_pbWeight->_pDevData, w->_bTransposed ? 1 : 0,
+                                           w->_pbBias->_pDevData, pUnit, _stride, batch, src->_stride, _localStride, (uint32_t)_activation,
+                                           &params, _pbSegMax->_pDevData, &_segWidth),
+                     "NNLayer::ForwardPropagate: GEMM failure");
         } else {
             dsxFatal(dsx_fc_forward(src->GetUnitBuffer(), src->_stride, wsrc->_pbWeight->_pDevData, w->_bTransposed ? 1 : 0,
                                     w->_pbBias->_pDevData, pUnit, _stride, batch, src->_stride, _localStride, 0, (uint32_t)_activation, &params),
@@ -220,5 +237,6 @@ bool NNLayer::SetUnits(const vector<NNFloat>& vUnit)
         return false;
     }
     _pbUnit->Upload(vUnit.data());
+    _segWidth = 0;
     return true;
 }

@@ -294,7 +294,12 @@ void NNNetwork::CalculateTopK(const string& layer, uint32_t k, GpuBuffer<NNFloat
     }
     uint32_t batch = _batch;
     if (_position + batch > _examples) batch = _examples - _position;
-    kCalculateTopK(pLayer->_pbUnit->_pDevData, pbKey->_pDevData, pbValue->_pDevData, batch, pLayer->_localStride, k);
+    if (pLayer->_segWidth != 0 && pLayer->_pbSegMax)
+        dsxFatal(dsx_topk_guided(pLayer->_pbUnit->_pDevData, pbKey->_pDevData, pbValue->_pDevData, batch, pLayer->_localStride, k,
+                                 pLayer->_pbSegMax->_pDevData, pLayer->_segWidth, 0, NULL, NULL, NULL, NULL, NULL),
+                 "NNNetwork::CalculateTopK");
+    else
+        kCalculateTopK(pLayer->_pbUnit->_pDevData, pbKey->_pDevData, pbValue->_pDevData, batch, pLayer->_localStride, k);
 }
 
 void NNNetwork::CalculateFilteredTopK(const string& layer, uint32_t k, NNDataSetBase* pFilter, GpuBuffer<NNFloat>* pbKey,
@@ -327,9 +332,11 @@ void NNNetwork::CalculateFilteredTopK(const string& layer, uint32_t k, NNDataSet
         if (pf && pf->_pbSparseData) pMul = pf->_pbSparseData->_pDevData;
     }
     const uint32_t* pIndex = (pFilter->_attributes & NNDataSetEnums::Indexed) ? pFilter->_pbIndex->_pDevData : NULL;
-    dsxFatal(dsx_topk_filtered(pLayer->_pbUnit->_pDevData, pbKey->_pDevData, pbValue->_pDevData, batch, pLayer->_localStride, k, _position,
-                               pIndex, pFilter->_pbSparseStart->_pDevData, pFilter->_pbSparseEnd->_pDevData,
-                               pFilter->_pbSparseIndex->_pDevData, pMul),
+    // with segment maxima of the current batch (left by the layer's dense kernel) only the segments that can hold a result are read
+    const NNFloat* pSegMax = (pLayer->_segWidth != 0 && pLayer->_pbSegMax) ? pLayer->_pbSegMax->_pDevData : NULL;
+    dsxFatal(dsx_topk_guided(pLayer->_pbUnit->_pDevData, pbKey->_pDevData, pbValue->_pDevData, batch, pLayer->_localStride, k, pSegMax,
+                             pLayer->_segWidth, _position, pIndex, pFilter->_pbSparseStart->_pDevData, pFilter->_pbSparseEnd->_pDevData,
+                             pFilter->_pbSparseIndex->_pDevData, pMul),
              "NNNetwork::CalculateFilteredTopK");
 }
 
@@ -404,6 +411,8 @@ NNFloat* NNNetwork::GetUnitBuffer(const string& layer)
         printf("NNNetwork::GetUnitBuffer: Unknown layer %s.\n", layer.c_str());
         return NULL;
     }
+    // the caller gets a writable device pointer: the segment maxima of the batch may not describe the units any longer
+    itr->second->_segWidth = 0;
     return itr->second->GetUnitBuffer();
 }
 

@@ -12,9 +12,13 @@ from . import ACT_SOFTMAX, ActParams, DeviceArray, check, load_library, ptr
 
 
 class DevicePipeline:
-    def __init__(self, problem, lib=None):
+    def __init__(self, problem, lib=None, guided=False):
+        """guided: the output layer also leaves segment maxima (dsx_fc_forward_segmax) and the top-K uses them."""
         self.lib = lib or load_library()
         p = self.p = problem
+        self.guided = guided
+        self.seg_max = DeviceArray((p.batch, (p.widths[-1] + 63) // 64), np.float32, self.lib) if guided else None
+        self.seg_width = C.c_uint32(0)
         self.W = [DeviceArray.from_numpy(w, self.lib) for w in p.weights]
         self.b = [DeviceArray.from_numpy(b, self.lib) for b in p.biases]
         self.start = DeviceArray.from_numpy(p.start, self.lib)
@@ -42,6 +46,10 @@ class DevicePipeline:
             k, n = p.widths[l], p.widths[l + 1]
             act = p.acts[l]
             fused = act if act != ACT_SOFTMAX else 3
+            if self.guided and l == len(self.W) - 1 and act != ACT_SOFTMAX:
+                check(lib.dsx_fc_forward_segmax(ptr(self.units[l - 1]), k, ptr(self.W[l]), 0, ptr(self.b[l]), ptr(self.units[l]), n, batch, k,
+                                                n, fused, C.byref(self.params), ptr(self.seg_max), C.byref(self.seg_width)))
+                continue
             check(lib.dsx_fc_forward(ptr(self.units[l - 1]), k, ptr(self.W[l]), 0, ptr(self.b[l]), ptr(self.units[l]), n, batch, k, n, 0,
                                      fused, C.byref(self.params)))
             if act == ACT_SOFTMAX:
@@ -52,7 +60,12 @@ class DevicePipeline:
         batch = p.batch if batch is None else batch
         k = p.k if k is None else k
         N = p.widths[-1]
-        if filtered:
+        if self.guided:
+            f = filtered
+            check(lib.dsx_topk_guided(ptr(self.units[-1]), ptr(self.keys), ptr(self.vals), batch, N, k, ptr(self.seg_max),
+                                      self.seg_width.value, position, ptr(self.index) if f else None, ptr(self.start) if f else None,
+                                      ptr(self.end) if f else None, ptr(self.sidx) if f else None, None))
+        elif filtered:
             check(lib.dsx_topk_filtered(ptr(self.units[-1]), ptr(self.keys), ptr(self.vals), batch, N, k, position, ptr(self.index),
                                         ptr(self.start), ptr(self.end), ptr(self.sidx), None))
         else:

@@ -163,6 +163,15 @@ int dsx_sparse_layer_forward(uint32_t attributes, uint32_t data_type, uint32_t p
 int dsx_fc_forward(const float* X, uint32_t ldx, const float* W, int transposed, const float* bias, float* Z, uint32_t ldz,
                    uint32_t batch, uint32_t k, uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params);
 
+/* dsx_fc_forward that also leaves, for a later top-K over Z, the maximum of every 64-column segment of every row of the
+ * activated result: seg_max[b][s] = max over columns 64 s .. 64 s + 63 (< n) of Z[b][.], row pitch ceil(n / 64).  The epilogue
+ * of the wide-layer kernel has these values in registers; other shapes leave seg_max untouched and set *seg_width = 0,
+ * otherwise *seg_width = 64.  No counterpart in the reference (it is the by-product that lets dsx_topk_guided skip most of
+ * the score matrix the reference's kCalculateTopK, engine/kernels.cu:3202-3989, reads in full). */
+int dsx_fc_forward_segmax(const float* X, uint32_t ldx, const float* W, int transposed, const float* bias, float* Z, uint32_t ldz,
+                          uint32_t batch, uint32_t k, uint32_t n, uint32_t activation, const dsx_act_params* params, float* seg_max,
+                          uint32_t* seg_width);
+
 /* kCalculateSigmoidActivation ... kCalculateSELUActivation (engine/kActivation.cu:46-153) and
  * kCalculateSoftMaxActivation (engine/kActivation.cu:155-236), in place on a [batch x stride] buffer. */
 int dsx_activation(float* unit, uint32_t batch, uint32_t stride, uint32_t activation, const dsx_act_params* params);
@@ -199,6 +208,14 @@ int dsx_knn_topk(const float* in, float* keys, uint32_t* values, uint32_t batch,
 int dsx_topk_filtered(const float* in, float* keys, uint32_t* values, uint32_t batch, uint32_t width, uint32_t k, uint32_t position,
                       const uint32_t* index, const uint64_t* filter_start, const uint64_t* filter_end, const uint32_t* filter_index,
                       const float* filter_mul);
+
+/* Top-K (optionally filtered, as dsx_topk_filtered; filter_index == NULL: unfiltered, as dsx_topk) of a score matrix whose
+ * producer left segment maxima (dsx_fc_forward_segmax): same results as the scanning calls, but only the segments that can
+ * hold a result are read.  seg_max must describe `in` exactly (same batch rows, seg_width 64); with seg_max == NULL,
+ * seg_width == 0, k > 32 or more than 2048 segments the call is the scanning one. */
+int dsx_topk_guided(const float* in, float* keys, uint32_t* values, uint32_t batch, uint32_t width, uint32_t k, const float* seg_max,
+                    uint32_t seg_width, uint32_t position, const uint32_t* index, const uint64_t* filter_start,
+                    const uint64_t* filter_end, const uint32_t* filter_index, const float* filter_mul);
 
 /* ---- KNN ------------------------------------------------------------------------------------------------------------- */
 /* Device part of KnnExactGpu::search (knn/KnnExactGpu.cu:99-148): scores = queries . items^T (cublasSgemmEx) followed by

@@ -398,6 +398,107 @@ def test_topk_filtered_indexed_duplicates_and_out_of_range(pkg, dsx, orc, rng):
     assert_topk_exact(keys, idx, rk, ri)
 
 
+def segment_maxima(scores):
+    batch, width = scores.shape
+    nseg = (width + 63) // 64
+    pad = np.full((batch, nseg * 64), -np.inf, dtype=np.float32)
+    pad[:, :width] = np.where(np.isnan(scores), -np.inf, scores)   # a NaN is never a maximum
+    return pad.reshape(batch, nseg, 64).max(axis=2)
+
+
+def run_guided(pkg, dsx, scores, k, seg_max, position=0, index=None, start=None, end=None, fidx=None, fmul=None, seg_width=64):
+    batch, width = scores.shape
+    d, dsm, di, ds, de, dx, dm = (dev(pkg, x) for x in (scores, seg_max, index, start, end, fidx, fmul))
+    keys = pkg.DeviceArray((batch, k), np.float32)
+    vals = pkg.DeviceArray((batch, k), np.uint32)
+    pkg.check(dsx.dsx_topk_guided(d.ptr, keys.ptr, vals.ptr, batch, width, k, pkg.ptr(dsm), seg_width, position, pkg.ptr(di), pkg.ptr(ds),
+                                  pkg.ptr(de), pkg.ptr(dx), pkg.ptr(dm)))
+    return keys.numpy(), vals.numpy()
+
+
+@pytest.mark.parametrize("batch,width,k", [(16, 27278, 10), (5, 64, 8), (7, 65, 32), (9, 1000, 1), (4, 131072, 32), (3, 40, 32),
+                                           (6, 5000, 64), (2, 200000, 10)])
+def test_topk_guided_plain(pkg, dsx, orc, rng, batch, width, k):
+    # the last two shapes are outside the guided kernel's range (k > 32, more than 2048 segments): the call scans instead
+    say("topk_guided batch=%d width=%d k=%d" % (batch, width, k))
+    scores = rng.standard_normal((batch, width), dtype=np.float32)
+    keys, idx = run_guided(pkg, dsx, scores, k, segment_maxima(scores))
+    rk, ri = orc.topk(scores, k)
+    assert_topk_exact(keys, idx, rk, ri)
+
+
+def test_topk_guided_ties_nan_and_constant_rows(pkg, dsx, orc, rng):
+    batch, width, k = 12, 9000, 10
+    scores = rng.integers(0, 4, (batch, width)).astype(np.float32)   # four distinct values: whole segments tie at the bound
+    scores[1] = 1.0                                                   # a constant row: every segment is read
+    scores[2, ::3] = np.nan
+    scores[3] = -np.inf
+    scores[3, 77] = 2.5
+    scores[4, :] = np.nan                                              # nothing to report: sentinels
+    keys, idx = run_guided(pkg, dsx, scores, k, segment_maxima(scores))
+    sk, si = run_topk(pkg, dsx, scores, k)
+    assert_topk_exact(keys, idx, sk, si)          # NaN never enters, in either kernel (rows of NaN give sentinels)
+    clean = ~np.isnan(scores).any(axis=1)
+    rk, ri = orc.topk(scores[clean], k)
+    assert_topk_exact(keys[clean], idx[clean], rk, ri)
+    assert np.all(keys[4] == np.float32(-999999999999999.0)) and np.all(idx[4] == 0)
+
+
+@pytest.mark.parametrize("batch,width,k,maxnnz", [(32, 1024, 10, 16), (64, 27278, 10, 2000), (8, 70, 32, 60), (16, 27278, 32, 5000)])
+@pytest.mark.parametrize("with_mul", [False, True])
+def test_topk_guided_filtered(pkg, dsx, orc, rng, batch, width, k, maxnnz, with_mul):
+    say("topk_guided filtered batch=%d width=%d k=%d mul=%s" % (batch, width, k, with_mul))
+    scores = rng.random((batch, width), dtype=np.float32)
+    start, end, fidx = random_csr(rng, batch, width, maxnnz, empty_rows=(1,))
+    # make the best scores of many segments listed ones: their maxima must not count towards the bound
+    for b in range(batch):
+        cols = fidx[int(start[b]):int(end[b])]
+        scores[b, cols[: len(cols) // 2]] += np.float32(1.0)
+    fmul = (rng.random(len(fidx), dtype=np.float32) * 3).astype(np.float32) if with_mul else None
+    keys, idx = run_guided(pkg, dsx, scores, k, segment_maxima(scores), 0, None, start, end, fidx, fmul)
+    rk, ri = orc.topk_filtered(scores, k, 0, None, start, end, fidx, fmul)
+    assert_topk_exact(keys, idx, rk, ri)
+    sk, si = run_filtered(pkg, dsx, scores, k, 0, None, start, end, fidx, fmul)
+    assert_topk_exact(keys, idx, sk, si)
+
+
+def test_topk_guided_indexed_filter_and_position(pkg, dsx, orc, rng):
+    rows, batch, width, k, position = 40, 17, 3000, 20, 9
+    scores = rng.random((batch, width), dtype=np.float32)
+    start, end, fidx = random_csr(rng, rows, width + 50, 300)     # some indexes beyond the width: ignored
+    fidx = fidx.copy()
+    fidx[1::7] = fidx[0::7][: len(fidx[1::7])]                    # duplicates inside rows: applied once
+    index = rng.permutation(rows).astype(np.uint32)
+    keys, idx = run_guided(pkg, dsx, scores, k, segment_maxima(scores), position, index, start, end, fidx, None)
+    rk, ri = orc.topk_filtered(scores, k, position, index, start, end, fidx, None)
+    assert_topk_exact(keys, idx, rk, ri)
+
+
+def test_fc_forward_segmax(pkg, dsx, orc, rng):
+    # wide layer: the 128 x 128-tile kernel leaves exact segment maxima, ragged last row block and last column tile included
+    B, k, n = 1000, 96, 33000 + 22
+    X = rng.standard_normal((B, k), dtype=np.float32)
+    W = (rng.standard_normal((k, n), dtype=np.float32) * np.float32(0.2)).astype(np.float32)
+    bias = rng.standard_normal(n, dtype=np.float32)
+    dX, dW, db = dev(pkg, X), dev(pkg, W), dev(pkg, bias)
+    Z = pkg.DeviceArray((B, n), np.float32)
+    Z2 = pkg.DeviceArray((B, n), np.float32)
+    nseg = (n + 63) // 64
+    sm = pkg.DeviceArray.from_numpy(np.full((B, nseg), 7.0, dtype=np.float32))
+    sw = C.c_uint32(99)
+    pkg.check(dsx.dsx_fc_forward_segmax(dX.ptr, k, dW.ptr, 0, db.ptr, Z.ptr, n, B, k, n, 0, None, sm.ptr, C.byref(sw)))
+    pkg.check(dsx.dsx_fc_forward(dX.ptr, k, dW.ptr, 0, db.ptr, Z2.ptr, n, B, k, n, 0, 0, None))
+    assert sw.value == 64
+    z = Z.numpy()
+    assert np.array_equal(z, Z2.numpy())
+    assert np.array_equal(sm.numpy(), segment_maxima(z))
+    # a narrow layer runs the small-tile kernel: no maxima, and it says so
+    n2 = 300
+    Zs = pkg.DeviceArray((B, n2), np.float32)
+    pkg.check(dsx.dsx_fc_forward_segmax(dX.ptr, k, dW.ptr, 0, db.ptr, Zs.ptr, n2, B, k, n2, 0, None, sm.ptr, C.byref(sw)))
+    assert sw.value == 0
+
+
 # ------------------------------------------------------------------------------------------------------------------- KNN
 
 @pytest.mark.parametrize("items,queries,dim,k", [(1003, 9, 24, 10), (50000, 64, 256, 100), (300007, 130, 64, 128)])

@@ -13,9 +13,9 @@ def say(msg):
     print("[case] " + msg, flush=True)
 
 
-def run_and_compare(pkg, dsx, orc, p, position=0, batch=None, filtered=True):
+def run_and_compare(pkg, dsx, orc, p, position=0, batch=None, filtered=True, guided=False):
     from amazon_dsstne_amd.pipeline import DevicePipeline
-    pipe = DevicePipeline(p, dsx)
+    pipe = DevicePipeline(p, dsx, guided=guided)
     pipe.step(position, batch, filtered=filtered)
     keys, idx = pipe.results(batch)
     unit = pipe.output_unit(batch)
@@ -80,3 +80,29 @@ def test_cfg4_large_catalogue_reduced(pkg, dsx, orc, synth):
 def test_nonzero_bias_and_odd_widths(pkg, dsx, orc, synth):
     p = synth.autoencoder("odd-widths", 77, 3001, [70, 33], 45, 17, 2, 1.0, 30, 0.8, (0, 200), bias_std=0.5)
     run_and_compare(pkg, dsx, orc, p, position=45)
+
+
+def test_cfg2_guided_topk_matches_scan_and_oracle(pkg, dsx, orc, synth):
+    # the output layer leaves segment maxima and the top-K reads only the segments that can hold a result: same answers
+    p = synth.config(2)
+    for filtered in (True, False):
+        _, k_scan, i_scan, _ = run_and_compare(pkg, dsx, orc, p, filtered=filtered)
+        pipe, k_gd, i_gd, unit = run_and_compare(pkg, dsx, orc, p, filtered=filtered, guided=True)
+        assert pipe.seg_width.value == 64
+        assert np.array_equal(i_gd, i_scan) and np.array_equal(k_gd.view(np.uint32), k_scan.view(np.uint32))
+        # the maxima themselves: exact maxima of the stored activations
+        sm = pipe.seg_max.numpy()
+        N = unit.shape[1]
+        pad = np.full((unit.shape[0], sm.shape[1] * 64), -np.inf, dtype=np.float32)
+        pad[:, :N] = unit
+        assert np.array_equal(sm, pad.reshape(unit.shape[0], -1, 64).max(axis=2))
+
+
+def test_cfg3_guided_with_saturated_scores(pkg, dsx, orc, synth):
+    # 1024-wide hidden layers saturate many sigmoids at 1.0f: whole segments tie at the bound and the guided kernel has to read
+    # most of the row; indexed, analog filter rows
+    p = synth.autoencoder("cfg3-analog-indexed-b512", 1003, 27278, [1024, 1024], 512, 10, 1, 1.0, 144, 1.0, (5, 2000), analog=True,
+                          indexed=True)
+    _, k_scan, i_scan, _ = run_and_compare(pkg, dsx, orc, p)
+    _, k_gd, i_gd, _ = run_and_compare(pkg, dsx, orc, p, guided=True)
+    assert np.array_equal(i_gd, i_scan) and np.array_equal(k_gd.view(np.uint32), k_scan.view(np.uint32))
