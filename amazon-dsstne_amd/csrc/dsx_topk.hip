@@ -673,11 +673,12 @@ __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kern
 constexpr uint32_t kGuidedSegWidth = 64;
 constexpr uint32_t kGuidedMaxSegs = 2048;
 
-template <bool FILTERED>
+// E: segment maxima per lane (256 * E >= number of segments); the key search costs in proportion.
+template <bool FILTERED, int E>
 __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a)
 {
     using List = WaveTopK<1>;
-    constexpr int E = kGuidedMaxSegs / kTopkThreads;   // maxima per lane
+    static_assert(E * kTopkThreads <= kGuidedMaxSegs, "at most kGuidedMaxSegs segments");
     __shared__ uint64_t sStage[kTopkWaves][List::kStageWords];
     __shared__ uint32_t sPrime[kTopkWaves][32];
     __shared__ uint32_t sListCount;
@@ -1038,10 +1039,15 @@ int topk_guided_run(const float* in, uint32_t width, uint32_t batch, uint32_t k,
     a.values = values;
     a.seg_max = seg_max;
     a.nseg = nseg;
-    if (filtered)
-        hipLaunchKernelGGL(topk_guided_kernel<true>, dim3(batch), dim3(kTopkThreads), lds, ctx().stream, a);
-    else
-        hipLaunchKernelGGL(topk_guided_kernel<false>, dim3(batch), dim3(kTopkThreads), lds, ctx().stream, a);
+#define DSX_GUIDED(F, E) hipLaunchKernelGGL((topk_guided_kernel<F, E>), dim3(batch), dim3(kTopkThreads), lds, ctx().stream, a)
+    if (nseg <= 2 * kTopkThreads) {
+        if (filtered) DSX_GUIDED(true, 2); else DSX_GUIDED(false, 2);
+    } else if (nseg <= 4 * kTopkThreads) {
+        if (filtered) DSX_GUIDED(true, 4); else DSX_GUIDED(false, 4);
+    } else {
+        if (filtered) DSX_GUIDED(true, 8); else DSX_GUIDED(false, 8);
+    }
+#undef DSX_GUIDED
     DSX_LAUNCH_CHECK("topk_guided_kernel");
     return DSX_OK;
 }
