@@ -97,6 +97,16 @@ def network_bench(args, pkg, lib):
     t1 = time.perf_counter()
     ms_step = (t1 - t0) * 1e3 / args.steps
 
+    # The same step when the batch's CSR arrays are handed over as host buffers every time (NNDataSet::LoadSparseData, as the
+    # reference's JNI predict does): never `value`, reported beside it.
+    up_steps = max(5, min(50, args.steps))
+    t0 = time.perf_counter()
+    for _ in range(up_steps):
+        net.load_sparse(p.start, p.end, p.sparse_data, p.sparse_index)
+        step()
+    net.sync()
+    ms_upload = (time.perf_counter() - t0) * 1e3 / up_steps
+
     # The same kernels one at a time on the same shapes (raw C ABI of the kernel library, same stream).
     pipe = DevicePipeline(p, lib)
     pipe.step()
@@ -191,6 +201,8 @@ def network_bench(args, pkg, lib):
         "roofline": roofline,
         "kernels": {n: {k: (round(v, 5) if isinstance(v, float) else v) for k, v in kv.items()} for n, kv in kernels.items()},
         "cpu_baseline": cpu,
+        "with_input_upload": {"ms_per_step": round(ms_upload, 5), "value": round(B / (ms_upload / 1e3), 1), "unit": "samples/s",
+                              "note": "host CSR arrays of the whole dataset copied and uploaded before every step (PCIe-inclusive)"},
     }
     return out
 
