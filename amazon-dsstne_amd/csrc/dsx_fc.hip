@@ -316,6 +316,71 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
     }
 }
 
+// Small problems (a few dozen 64 x 64 tiles, e.g. the 128-wide hidden layers at batch 1024) are bound by the chain of load
+// latencies of a k-loop, not by the matrix cores.  Here a workgroup owns a 32 x 32 tile of Z and its four wavefronts split k
+// four ways: every lane requests all its operands at once, straight from global memory into registers (the X row segment as
+// 128-bit loads, the W column as dwords that coalesce across the 32 lanes of a half wave), one round trip instead of one
+// per k-step; the four partial tiles meet in LDS.  S = k / 4 (32 or 64).
+template <int S, int ACT>
+__global__ __launch_bounds__(kFcThreads) void fc_small_kernel(FcArgs a)
+{
+    constexpr int T = S / 2;   // MFMA steps per wavefront; lane half h supplies k = base + h * T + t at step t
+    __shared__ float sPart[4][16][kWave];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lhi = lane >> 5;
+    const uint32_t col0 = blockIdx.x * 32, row0 = blockIdx.y * 32;
+    const uint32_t kbase = wave * S + lhi * T;
+    const uint32_t row = min(row0 + l32, a.batch - 1), col = min(col0 + l32, a.n - 1);   // out-of-range lanes repeat the edge; never stored
+
+    float av[T], bv[T];
+    const float* xsrc = a.X + (uint64_t)row * a.ldx + kbase;
+#pragma unroll
+    for (int t = 0; t < T; t += 4) {
+        const float4 v = *reinterpret_cast<const float4*>(xsrc + t);
+        av[t] = v.x; av[t + 1] = v.y; av[t + 2] = v.z; av[t + 3] = v.w;
+    }
+    const float* wsrc = a.W + (uint64_t)kbase * a.ldw + col;
+#pragma unroll
+    for (int t = 0; t < T; t++) bv[t] = wsrc[(uint64_t)t * a.ldw];
+    const float bias = a.bias ? a.bias[col] : 0.0f;
+
+    floatx16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+#pragma unroll
+    for (int t = 0; t < T; t++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[t], bv[t], acc, 0, 0, 0);
+
+    // every wavefront publishes its partial tile and finishes four of the sixteen accumulator registers
+#pragma unroll
+    for (int v = 0; v < 16; v++) sPart[wave][v][lane] = acc[v];
+    __syncthreads();
+    if (col0 + l32 >= a.n) return;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int v = wave * 4 + q;
+        const float x = ((sPart[0][v][lane] + sPart[1][v][lane]) + (sPart[2][v][lane] + sPart[3][v][lane])) + bias;
+        const uint32_t r = row0 + 8 * (v / 4) + 4 * lhi + (v % 4);   // v / 4 == wave, v % 4 == q
+        if (r < a.batch) a.Z[(uint64_t)r * a.ldz + col0 + l32] = activate<ACT>(x, a.slope, a.alpha, a.lambda);
+    }
+}
+
+template <int S> static void launch_fc_small(const FcArgs& a)
+{
+    hipStream_t s = ctx().stream;
+    const dim3 grid((a.n + 31) / 32, (a.batch + 31) / 32);
+#define DSX_ACT_CASE(A) case A: hipLaunchKernelGGL((fc_small_kernel<S, A>), grid, dim3(kFcThreads), 0, s, a); break;
+    switch (a.act) {
+        DSX_ACT_CASE(DSX_ACT_SIGMOID)
+        DSX_ACT_CASE(DSX_ACT_TANH)
+        DSX_ACT_CASE(DSX_ACT_RELU)
+        DSX_ACT_CASE(DSX_ACT_LRELU)
+        DSX_ACT_CASE(DSX_ACT_ELU)
+        DSX_ACT_CASE(DSX_ACT_SELU)
+    default: hipLaunchKernelGGL((fc_small_kernel<S, DSX_ACT_LINEAR>), grid, dim3(kFcThreads), 0, s, a); break;
+    }
+#undef DSX_ACT_CASE
+}
+
 template <int MI, int NI, int BK, int XV, int WV, bool TRANS>
 static void launch_fc_act(const FcArgs& a, uint32_t grid)
 {
@@ -384,6 +449,9 @@ int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int trans
             *seg_width = 64;
         }
         launch_fc_shape<2, 2, 16>(a, xv, wv, transposed != 0);
+    } else if (!transposed && !accumulate && xv == 4 && (k == 128 || k == 256) && (uint64_t)batch * n <= (1u << 20)) {
+        if (k == 128) launch_fc_small<32>(a);   // latency bound: all operands in one round trip
+        else launch_fc_small<64>(a);
     } else
         launch_fc_shape<1, 1, 32>(a, xv, wv, transposed != 0);   // few workgroups: deep k-steps, fewer barrier round trips
     DSX_LAUNCH_CHECK("fc_gemm_kernel");

@@ -251,6 +251,23 @@ def test_fc_forward_epilogue(pkg, dsx, orc, rng, act, accumulate):
     assert_close(Z.numpy(), ref, "fc epilogue", rel=1e-4, abs_floor=1e-2)
 
 
+@pytest.mark.parametrize("B,k,n,act", [(1024, 128, 128, 2), (1000, 256, 100, 0), (33, 128, 31, 1), (5, 256, 1, 3), (777, 128, 1000, 12)])
+def test_fc_forward_split_k_small_problems(pkg, dsx, orc, rng, B, k, n, act):
+    # k = 128 / 256 with few output tiles runs the latency-oriented kernel (k split over the four wavefronts); pitched X and Z
+    say("fc_forward split-k B=%d k=%d n=%d act=%d" % (B, k, n, act))
+    X = rng.standard_normal((B, k + 4)).astype(np.float32)
+    W = (rng.standard_normal((k, n)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    dX, dW, db = dev(pkg, X), dev(pkg, W), dev(pkg, bias)
+    Z = pkg.DeviceArray.from_numpy(np.full((B, n + 5), 55.0, dtype=np.float32))
+    params = pkg.ActParams(0.2, 1.5, 1.05)
+    pkg.check(dsx.dsx_fc_forward(dX.ptr, k + 4, dW.ptr, 0, db.ptr, Z.ptr, n + 5, B, k, n, 0, act, C.byref(params)))
+    got = Z.numpy()
+    ref = orc.activation(orc.sgemm_acc(np.ascontiguousarray(X[:, :k]), W, orc.clear_unit([bias], n, B)), act, 0.2, 1.5, 1.05)
+    assert_close(got[:, :n], ref, "split-k fc", rel=1e-4, abs_floor=max(float(np.sqrt(k)) * 0.1, 1e-2))
+    assert np.all(got[:, n:] == 55.0)                             # nothing written past n
+
+
 def test_fc_forward_transposed_and_pitched(pkg, dsx, orc, rng):
     B, k, n = 90, 70, 130
     X = rng.standard_normal((B, k + 6)).astype(np.float32)       # row pitch larger than k
