@@ -26,6 +26,7 @@ struct FcArgs {
     uint32_t tiles_m, tiles_n;
     int accumulate;
     uint32_t act;
+    int fast32;          // every byte offset into X and W fits 32 bits (interior tiles then take the lean load path)
     float* seg_max;      // optional: [batch][nseg] maxima of the activated outputs over 64-column segments
     uint32_t nseg;
     float slope, alpha, lambda;
@@ -209,17 +210,7 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
     };
 
     const uint32_t nk = (a.k + BK - 1) / BK;
-    load_a(0);
-    load_b(0);
-    store_a(0);
-    store_b(0);
-    __syncthreads();
-    for (uint32_t kt = 0; kt < nk; kt++) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) {
-            load_a((kt + 1) * BK);
-            load_b((kt + 1) * BK);
-        }
+    auto multiply = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 2) {
             float av[MI], bv[NI];
@@ -232,11 +223,79 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
 #pragma unroll
                 for (int j = 0; j < NI; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
         }
-        if (kt + 1 < nk) {
-            store_a(buf ^ 1);
-            store_b(buf ^ 1);
+    };
+    // Interior tiles (the vast majority): no bounds checks, and every load is "uniform base + this lane's constant 32-bit byte
+    // offset", so a k-step costs a handful of vector instructions.  That matters more than usual here: fp32 MFMA and ordinary
+    // vector instructions do not overlap on this part (measured), so every VALU instruction in the loop is MFMA time lost.
+    bool lean = false;
+    if constexpr (!TRANS && XV == 4 && (WV == 4 || WV == 2)) {
+        lean = a.fast32 && (row0 + BM <= a.batch) && (col0 + BN <= a.n) && (a.k % BK == 0);
+        if (lean) {
+            uint32_t offA[A_ELEMS / 4], offB[B_ELEMS / WV];
+#pragma unroll
+            for (int p = 0; p < A_ELEMS / 4; p++) {
+                const int idx = tid + p * kFcThreads;
+                offA[p] = ((row0 + idx / (BK / 4)) * a.ldx + (idx % (BK / 4)) * 4) * 4u;
+            }
+#pragma unroll
+            for (int p = 0; p < B_ELEMS / WV; p++) {
+                const int idx = tid + p * kFcThreads;
+                offB[p] = ((uint32_t)(idx / (BN / WV)) * a.ldw + col0 + (idx % (BN / WV)) * WV) * 4u;
+            }
+            auto load_lean = [&](uint32_t k0) __attribute__((always_inline)) {
+                const char* pa = reinterpret_cast<const char*>(a.X) + (uint64_t)k0 * 4;
+                const char* pb = reinterpret_cast<const char*>(a.W) + (uint64_t)k0 * a.ldw * 4;
+#pragma unroll
+                for (int p = 0; p < A_ELEMS / 4; p++) {
+                    const float4 v = *reinterpret_cast<const float4*>(pa + offA[p]);
+                    ra[p * 4 + 0] = v.x; ra[p * 4 + 1] = v.y; ra[p * 4 + 2] = v.z; ra[p * 4 + 3] = v.w;
+                }
+#pragma unroll
+                for (int p = 0; p < B_ELEMS / WV; p++) {
+                    if constexpr (WV == 4) {
+                        const float4 t = *reinterpret_cast<const float4*>(pb + offB[p]);
+                        rb[p * 4 + 0] = t.x; rb[p * 4 + 1] = t.y; rb[p * 4 + 2] = t.z; rb[p * 4 + 3] = t.w;
+                    } else {
+                        const float2 t = *reinterpret_cast<const float2*>(pb + offB[p]);
+                        rb[p * 2 + 0] = t.x; rb[p * 2 + 1] = t.y;
+                    }
+                }
+            };
+            load_lean(0);
+            store_a(0);
+            store_b(0);
+            __syncthreads();
+            for (uint32_t kt = 0; kt < nk; kt++) {
+                const int buf = kt & 1;
+                if (kt + 1 < nk) load_lean((kt + 1) * BK);
+                multiply(buf);
+                if (kt + 1 < nk) {
+                    store_a(buf ^ 1);
+                    store_b(buf ^ 1);
+                }
+                __syncthreads();
+            }
         }
+    }
+    if (!lean) {
+        load_a(0);
+        load_b(0);
+        store_a(0);
+        store_b(0);
         __syncthreads();
+        for (uint32_t kt = 0; kt < nk; kt++) {
+            const int buf = kt & 1;
+            if (kt + 1 < nk) {
+                load_a((kt + 1) * BK);
+                load_b((kt + 1) * BK);
+            }
+            multiply(buf);
+            if (kt + 1 < nk) {
+                store_a(buf ^ 1);
+                store_b(buf ^ 1);
+            }
+            __syncthreads();
+        }
     }
 
     // Epilogue: accumulator register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 block.
@@ -436,6 +495,8 @@ int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int trans
     a.slope = params ? params->slope : 0.01f;
     a.alpha = params ? params->alpha : 1.0f;
     a.lambda = params ? params->lambda : 1.0f;
+    // the lean path's per-lane offsets: (row * ldx + k4) * 4 into X, (kk * ldw + column) * 4 with kk < 32 into a k-slice of W
+    a.fast32 = ((uint64_t)(batch + 128) * ldx * 4 < (1ull << 32)) && ((32ull * ldw + n + 128) * 4 < (1ull << 32));
     const int xv = (((uintptr_t)X % 16) == 0 && (ldx % 4) == 0) ? 4 : 1;
     int wv = 1;
     if (((uintptr_t)W % 16) == 0 && (ldw % 4) == 0) wv = 4;
