@@ -663,7 +663,7 @@ __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kern
     finish_row<R>(list, sStage, a, b, seg, wave, lane);
 }
 
-// Guided top-K (k <= 32): the producer of the scores also left the maximum of every 64-column segment of every row (the
+// Guided top-K (k <= 64): the producer of the scores also left the maximum of every 64-column segment of every row (the
 // dense layer's epilogue has them in registers anyway).  The k-th largest of a row's segment maxima is a score that at least
 // k items reach, so only segments whose maximum reaches it can hold a result: about k of them.  The kernel reads the
 // row's maxima (1/64 of the row), picks that bound with the same key-bit search the scan uses for priming, and then reads
@@ -672,6 +672,7 @@ __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kern
 // right: the survivors go through the same lists as in the scan.
 constexpr uint32_t kGuidedSegWidth = 64;
 constexpr uint32_t kGuidedMaxSegs = 2048;
+constexpr uint32_t kGuidedMaxK = 64;
 
 // E: segment maxima per lane (256 * E >= number of segments); the key search costs in proportion.
 template <bool FILTERED, int E>
@@ -680,7 +681,7 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
     using List = WaveTopK<1>;
     static_assert(E * kTopkThreads <= kGuidedMaxSegs, "at most kGuidedMaxSegs segments");
     __shared__ uint64_t sStage[kTopkWaves][List::kStageWords];
-    __shared__ uint32_t sPrime[kTopkWaves][32];
+    __shared__ uint32_t sPrime[kTopkWaves][kGuidedMaxK];
     __shared__ uint32_t sListCount;
     extern __shared__ uint32_t sDyn[];   // segments to read [nseg] | best listed score per segment [nseg] | bitmap of listed columns
     uint32_t* sList = sDyn;
@@ -710,7 +711,7 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
             mk[e] = (idx < a.nseg) ? score_key(mrow[idx]) : 0u;
         }
     }
-    if (lane < 32) sPrime[wave][lane] = 0;
+    sPrime[wave][lane] = 0;
     if (threadIdx.x == 0) sListCount = 0;
 
     constexpr int kFU = 4;
@@ -782,13 +783,13 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
             published += (uint32_t)__popcll(pm);
         }
         __syncthreads();
-        uint32_t all[2];
+        uint32_t all[4];
 #pragma unroll
-        for (int n = 0; n < 2; n++) {
+        for (int n = 0; n < 4; n++) {
             const uint32_t i = n * kWave + lane;
             all[n] = (i < kTopkWaves * a.k) ? sPrime[i / a.k][i % a.k] : 0u;
         }
-        const uint32_t t = wave_kth_key<2>(all, a.k);
+        const uint32_t t = (a.k <= 32) ? wave_kth_key<2>(reinterpret_cast<const uint32_t(&)[2]>(all), a.k) : wave_kth_key<4>(all, a.k);
         if (t > score_key(-__builtin_inff())) {
             bound = t;
             list.prime(t);
@@ -1012,7 +1013,7 @@ int topk_merge(const uint64_t* partial, uint32_t slots, uint32_t k, float* keys,
     return launch_merge<4>(partial, slots, k, keys, values, batch);
 }
 
-// Guided top-K when it applies (k <= 32, 64-column segments, at most kGuidedMaxSegs of them), the scan otherwise.
+// Guided top-K when it applies (k <= 64, 64-column segments, at most kGuidedMaxSegs of them), the scan otherwise.
 int topk_guided_run(const float* in, uint32_t width, uint32_t batch, uint32_t k, float* keys, uint32_t* values, const float* seg_max,
                     uint32_t seg_width, uint32_t position, const uint32_t* index, const uint64_t* fstart, const uint64_t* fend,
                     const uint32_t* fidx, const float* fmul)
@@ -1021,7 +1022,7 @@ int topk_guided_run(const float* in, uint32_t width, uint32_t batch, uint32_t k,
     const uint32_t nseg = (width + kGuidedSegWidth - 1) / kGuidedSegWidth;
     size_t lds = (size_t)nseg * 4;
     if (filtered) lds += (size_t)nseg * 4 + ((size_t)(width + 31) / 32) * 4;
-    if (!seg_max || seg_width != kGuidedSegWidth || k > 32 || nseg > kGuidedMaxSegs || lds > 40 * 1024)
+    if (!seg_max || seg_width != kGuidedSegWidth || k > kGuidedMaxK || nseg > kGuidedMaxSegs || lds > 40 * 1024)
         return topk_run(in, width, width, batch, k, keys, values, position, index, fstart, fend, fidx, fmul, 0, nullptr, 0, 0, 0);
     TopKArgs a{};
     a.in = in;

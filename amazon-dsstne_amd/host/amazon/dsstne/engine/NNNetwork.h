@@ -62,6 +62,10 @@ public:
     // items listed in the filter dataset (a sparse dataset over the layer's items) by 0, or by the dataset's float values
     // when bUseValues is set — the device-side form of NNRecsGenerator::generateRecs (utils/NNRecsGenerator.cpp:132-150).
     // Passing the input dataset drops the items a sample already has.
+    // The same with the filter as device-resident CSR arrays (row position + b of the arrays filters batch row b; pMul NULL =
+    // every listed unit is multiplied by 0): what NNRecsGenerator::generateRecs does with its SamplesFilter, on the device.
+    void CalculateFilteredTopK(const string& layer, uint32_t k, const uint64_t* pFilterStart, const uint64_t* pFilterEnd,
+                               const uint32_t* pFilterIndex, const NNFloat* pFilterMul, NNFloat* pKey, uint32_t* pValue);
     void CalculateFilteredTopK(const string& layer, uint32_t k, NNDataSetBase* pFilter, GpuBuffer<NNFloat>* pbKey,
                                GpuBuffer<uint32_t>* pbValue, bool bUseValues = false);
     void SetBatch(uint32_t batch);

@@ -340,6 +340,27 @@ void NNNetwork::CalculateFilteredTopK(const string& layer, uint32_t k, NNDataSet
              "NNNetwork::CalculateFilteredTopK");
 }
 
+void NNNetwork::CalculateFilteredTopK(const string& layer, uint32_t k, const uint64_t* pFilterStart, const uint64_t* pFilterEnd,
+                                      const uint32_t* pFilterIndex, const NNFloat* pFilterMul, NNFloat* pKey, uint32_t* pValue)
+{
+    auto it = _mLayer.find(layer);
+    if (it == _mLayer.end() || !it->second->_pbUnit) {
+        printf("NNNetwork::CalculateFilteredTopK: Unknown layer %s or no unit buffer.\n", layer.c_str());
+        return;
+    }
+    NNLayer* pLayer = it->second;
+    if (k > 256 || k > pLayer->_Nx * pLayer->_Ny * pLayer->_Nz) {
+        printf("NNNetwork::CalculateFilteredTopK: k = %u does not fit layer %s (256 at most).\n", k, layer.c_str());
+        return;
+    }
+    uint32_t batch = _batch;
+    if (_position + batch > _examples) batch = _examples - _position;
+    const NNFloat* pSegMax = (pLayer->_segWidth != 0 && pLayer->_pbSegMax) ? pLayer->_pbSegMax->_pDevData : NULL;
+    dsxFatal(dsx_topk_guided(pLayer->_pbUnit->_pDevData, pKey, pValue, batch, pLayer->_localStride, k, pSegMax, pLayer->_segWidth, _position,
+                             NULL, pFilterStart, pFilterEnd, pFilterIndex, pFilterMul),
+             "NNNetwork::CalculateFilteredTopK");
+}
+
 void NNNetwork::SetBatch(uint32_t batch)
 {
     if (batch != _batch) {

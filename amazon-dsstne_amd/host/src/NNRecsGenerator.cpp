@@ -29,22 +29,22 @@ void NNRecsGenerator::generateRecs(NNNetwork* xNetwork, unsigned int xK, const F
     uint32_t x, y, z, w;
     std::tie(x, y, z, w) = pLayer->GetDimensions();
     const uint32_t width = x * y * z * w;
-    NNFloat* pUnit = xNetwork->GetUnitBuffer(recsGenLayerLabel);
     const uint32_t kk = std::min<uint32_t>(xK * TOPK_SCALAR, 256u);
     if (kk > width || (size_t)lBatch * kk > pbKey->_length) {
         printf("NNRecsGenerator::generateRecs: k = %u does not fit layer %s or the result buffers.\n", xK, recsGenLayerLabel.c_str());
         return;
     }
+    // The reference copies the output rows to the host, multiplies the filtered items there, uploads and runs the top-K
+    // (utils/NNRecsGenerator.cpp:138-150); here the filter is applied on the device while the scores are examined.
     SamplesFilter* sf = xFilterSet ? xFilterSet->getSamplesFilter() : NULL;
     if (sf && sf->samples() >= lPosition + lBatch) {
         const uint64_t *fs, *fe;
         const uint32_t* fi;
         const NNFloat* fm;
         sf->deviceArrays(&fs, &fe, &fi, &fm);
-        dsxFatal(dsx_topk_filtered(pUnit, pbKey->_pDevData, pbUIValue->_pDevData, lBatch, width, kk, lPosition, NULL, fs, fe, fi, fm),
-                 "NNRecsGenerator::generateRecs");
+        xNetwork->CalculateFilteredTopK(recsGenLayerLabel, kk, fs, fe, fi, fm, pbKey->_pDevData, pbUIValue->_pDevData);
     } else {
-        dsxFatal(dsx_topk(pUnit, pbKey->_pDevData, pbUIValue->_pDevData, lBatch, width, kk), "NNRecsGenerator::generateRecs");
+        xNetwork->CalculateFilteredTopK(recsGenLayerLabel, kk, NULL, NULL, NULL, NULL, pbKey->_pDevData, pbUIValue->_pDevData);
     }
     pbKey->Download();
     pbUIValue->Download();

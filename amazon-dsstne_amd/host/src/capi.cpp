@@ -269,13 +269,8 @@ int dsstne_topk(dsstne_context* c, const char* layer, uint32_t k, const char* fi
     if (filter_dataset)
         n->CalculateFilteredTopK(layer, k, findDataSet(c, filter_dataset), c->scoreBuf(layer), c->indexBuf(layer));
     else {
-        // the JNI path calls the raw kernel (k up to 256), not NNNetwork::CalculateTopK (k <= 128)
-        NNLayer* l = n->GetLayer(layer);
-        if (!l) return fail("dsstne_topk: unknown layer %s", layer);
-        uint32_t x, y, z, w;
-        std::tie(x, y, z, w) = l->GetDimensions();
-        uint32_t batch = std::min<uint32_t>(n->GetBatch(), n->GetExamples() - n->GetPosition());
-        kCalculateTopK(n->GetUnitBuffer(layer), c->scoreBuf(layer)->_pDevData, c->indexBuf(layer)->_pDevData, batch, x * y * z, k);
+        // like the JNI path, which calls the raw kernel: k up to 256 (NNNetwork::CalculateTopK stops at 128)
+        n->CalculateFilteredTopK(layer, k, NULL, NULL, NULL, NULL, c->scoreBuf(layer)->_pDevData, c->indexBuf(layer)->_pDevData);
     }
     return 0;
     CAPI_CATCH(-1)
@@ -309,6 +304,17 @@ int dsstne_get_units(dsstne_context* c, const char* layer, float* units, size_t 
     if (!p) return fail("dsstne_get_units: layer %s has no unit buffer", layer);
     if (count > c->net()->GetBufferSize(layer)) return fail("dsstne_get_units: %zu values requested, the layer holds %zu", count, (size_t)c->net()->GetBufferSize(layer));
     dsxFatal(dsx_memcpy_d2h(units, p, count * sizeof(float)), "dsstne_get_units");
+    return 0;
+    CAPI_CATCH(-1)
+}
+
+int dsstne_set_units(dsstne_context* c, const char* layer, const float* units, size_t count)
+{
+    CAPI_TRY
+    NNLayer* l = c->net()->GetLayer(layer);
+    if (!l) return fail("dsstne_set_units: unknown layer %s", layer);
+    std::vector<NNFloat> v(units, units + count);
+    if (!const_cast<NNLayer*>(l)->SetUnits(v)) return fail("dsstne_set_units: layer %s refused %zu values", layer, count);
     return 0;
     CAPI_CATCH(-1)
 }

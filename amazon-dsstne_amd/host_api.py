@@ -29,6 +29,7 @@ SIGNATURES = {
     "dsstne_get_topk": ([_vp, _cp, _u32, _u32, _vp, _vp], _int),
     "dsstne_predict": ([_vp, _cp, _u32, _cp, _vp, _vp], _int),
     "dsstne_get_units": ([_vp, _cp, _vp, _sz], _int),
+    "dsstne_set_units": ([_vp, _cp, _vp, _sz], _int),
     "dsstne_sync": ([], _int),
     "dsstne_timer_start": ([], _int),
     "dsstne_timer_stop": ([C.POINTER(_f32)], _int),
@@ -141,6 +142,10 @@ class Network:
         out = np.empty((rows, width), dtype=np.float32)
         _check(self.lib.dsstne_get_units(self.ctx, layer.encode(), out.ctypes.data, out.size))
         return out
+
+    def set_units(self, values, layer="Output"):
+        values = np.ascontiguousarray(values, dtype=np.float32)
+        _check(self.lib.dsstne_set_units(self.ctx, layer.encode(), values.ctypes.data, values.size))
 
     def save(self, path):
         _check(self.lib.dsstne_save_network(self.ctx, path.encode()))

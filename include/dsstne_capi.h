@@ -71,6 +71,8 @@ int dsstne_get_topk(dsstne_context* ctx, const char* layer, uint32_t rows, uint3
 int dsstne_predict(dsstne_context* ctx, const char* layer, uint32_t k, const char* filter_dataset, float* scores, uint32_t* indexes);
 /* NNLayer::GetUnits: the layer's [batch][width] activations. */
 int dsstne_get_units(dsstne_context* ctx, const char* layer, float* units, size_t count);
+/* NNLayer::SetUnits (engine/NNLayer.cpp:318-368 group): overwrites the layer's unit buffer (batch x stride values) from the host. */
+int dsstne_set_units(dsstne_context* ctx, const char* layer, const float* units, size_t count);
 int dsstne_sync(void);
 /* Event timing around calls on the library stream: milliseconds between start and stop. */
 int dsstne_timer_start(void);

@@ -212,7 +212,7 @@ int dsx_topk_filtered(const float* in, float* keys, uint32_t* values, uint32_t b
 /* Top-K (optionally filtered, as dsx_topk_filtered; filter_index == NULL: unfiltered, as dsx_topk) of a score matrix whose
  * producer left segment maxima (dsx_fc_forward_segmax): same results as the scanning calls, but only the segments that can
  * hold a result are read.  seg_max must describe `in` exactly (same batch rows, seg_width 64); with seg_max == NULL,
- * seg_width == 0, k > 32 or more than 2048 segments the call is the scanning one. */
+ * seg_width == 0, k > 64 or more than 2048 segments the call is the scanning one. */
 int dsx_topk_guided(const float* in, float* keys, uint32_t* values, uint32_t batch, uint32_t width, uint32_t k, const float* seg_max,
                     uint32_t seg_width, uint32_t position, const uint32_t* index, const uint64_t* filter_start,
                     const uint64_t* filter_end, const uint32_t* filter_index, const float* filter_mul);

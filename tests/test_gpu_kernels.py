@@ -434,9 +434,9 @@ def run_guided(pkg, dsx, scores, k, seg_max, position=0, index=None, start=None,
 
 
 @pytest.mark.parametrize("batch,width,k", [(16, 27278, 10), (5, 64, 8), (7, 65, 32), (9, 1000, 1), (4, 131072, 32), (3, 40, 32),
-                                           (6, 5000, 64), (2, 200000, 10)])
+                                           (6, 5000, 64), (8, 27278, 50), (5, 5000, 100), (2, 200000, 10)])
 def test_topk_guided_plain(pkg, dsx, orc, rng, batch, width, k):
-    # the last two shapes are outside the guided kernel's range (k > 32, more than 2048 segments): the call scans instead
+    # the last two shapes are outside the guided kernel's range (k > 64, more than 2048 segments): the call scans instead
     say("topk_guided batch=%d width=%d k=%d" % (batch, width, k))
     scores = rng.standard_normal((batch, width), dtype=np.float32)
     keys, idx = run_guided(pkg, dsx, scores, k, segment_maxima(scores))
@@ -461,7 +461,8 @@ def test_topk_guided_ties_nan_and_constant_rows(pkg, dsx, orc, rng):
     assert np.all(keys[4] == np.float32(-999999999999999.0)) and np.all(idx[4] == 0)
 
 
-@pytest.mark.parametrize("batch,width,k,maxnnz", [(32, 1024, 10, 16), (64, 27278, 10, 2000), (8, 70, 32, 60), (16, 27278, 32, 5000)])
+@pytest.mark.parametrize("batch,width,k,maxnnz", [(32, 1024, 10, 16), (64, 27278, 10, 2000), (8, 70, 32, 60), (16, 27278, 32, 5000),
+                                                 (16, 27278, 50, 3000), (4, 200, 64, 150)])
 @pytest.mark.parametrize("with_mul", [False, True])
 def test_topk_guided_filtered(pkg, dsx, orc, rng, batch, width, k, maxnnz, with_mul):
     say("topk_guided filtered batch=%d width=%d k=%d mul=%s" % (batch, width, k, with_mul))

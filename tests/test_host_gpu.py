@@ -68,7 +68,32 @@ def test_network_api_public_constructor_data_runs_analog_kernel(pkg, dsx, orc, s
 
 
 def test_network_api_cfg2_full(pkg, dsx, orc, synth):
+    # output layer of 27,278 units: the forward pass leaves segment maxima and both top-K calls are the guided ones
     host_forward(pkg, dsx, orc, synth.config(2), filtered=True)
+    host_forward(pkg, dsx, orc, synth.config(2), filtered=False)
+
+
+def test_topk_after_units_were_overwritten(pkg, dsx, orc, synth):
+    # the segment maxima of the forward pass must not outlive the units they describe
+    from amazon_dsstne_amd import host_api
+    p = synth.config(2)
+    rng = np.random.default_rng(3)
+    fresh = rng.random((p.batch, p.widths[-1]), dtype=np.float32)
+    net = host_api.Network(p, max_k=p.k)
+    try:
+        net.bind_input()
+        net.predict_batch(0)
+        net.set_units(fresh)
+        net.topk(p.k, filter_dataset=None)
+        keys, idx = net.get_topk(p.batch)
+        net.topk(p.k, filter_dataset="input")
+        fkeys, fidx = net.get_topk(p.batch)
+    finally:
+        net.close()
+    rk, ri = orc.topk(fresh, p.k)
+    assert np.array_equal(idx, ri) and np.array_equal(keys.view(np.uint32), rk.view(np.uint32))
+    rk, ri = orc.topk_filtered(fresh, p.k, 0, None, p.start, p.end, p.sparse_index, None)
+    assert np.array_equal(fidx, ri) and np.array_equal(fkeys.view(np.uint32), rk.view(np.uint32))
 
 
 def test_network_api_positions_and_short_last_batch(pkg, dsx, orc, synth):
