@@ -353,20 +353,21 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
     }
     if constexpr (kCanSegMax) {
         if (want_max) {
-            // Reduce-scatter over the 32 lanes of each half wave: step s pairs the values whose index differs in bit s, the
-            // lane whose own bit s is set keeps the upper one and hands the other over.  31 exchanges later lane l holds
-            // the maximum of value index q = l % 32, i.e. of one of the wave's 64 rows.
+            // Transpose through LDS (the operand tiles are dead by now): lane l wrote its 32 row maxima, and reads back the 32
+            // values that the lanes of its half wave hold for row index q = l % 32.  LDS instructions do not compete with the
+            // matrix cores the way a cross-lane reduction in vector registers would.  Pitch 65 keeps both sides conflict-free.
+            __syncthreads();   // every wavefront is done with sA / sB
+            float* sT = ((wave < 2) ? &sA[0][0][0] : &sB[0][0][0]) + (wave & 1) * (32 * 65);
+            static_assert(sizeof(sA) >= 2 * 32 * 65 * sizeof(float) && sizeof(sB) >= 2 * 32 * 65 * sizeof(float),
+                          "the transposition reuses the operand tiles' LDS, two wavefronts in each");
 #pragma unroll
-            for (int s = 4; s >= 0; s--) {
-                const int half = 1 << s;
-                const bool upper = (l32 >> s) & 1;
+            for (int q = 0; q < 32; q++) sT[q * 65 + lane] = smax[q];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            float m = -__builtin_inff();
 #pragma unroll
-                for (int q = 0; q < half; q++) {
-                    const float keep = upper ? smax[q + half] : smax[q];
-                    const float send = upper ? smax[q] : smax[q + half];
-                    smax[q] = fmaxf(keep, __shfl_xor(send, half, 64));
-                }
-            }
+            for (int t = 0; t < 32; t++) m = fmaxf(m, sT[l32 * 65 + lhi * 32 + t]);
+            smax[0] = m;
             const int q = l32, i = q >> 4, v = q & 15;
             const uint32_t r = row0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * lhi + (v & 3);
             const uint32_t seg = (col0 + wn * 64) / 64;
