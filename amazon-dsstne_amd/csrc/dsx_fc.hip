@@ -356,7 +356,7 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
             // Transpose through LDS (the operand tiles are dead by now): lane l wrote its 32 row maxima, and reads back the 32
             // values that the lanes of its half wave hold for row index q = l % 32.  LDS instructions do not compete with the
             // matrix cores the way a cross-lane reduction in vector registers would.  Pitch 65 keeps both sides conflict-free.
-            __syncthreads();   // every wavefront is done with sA / sB
+            // (the k-loop ended with a barrier: every wavefront is done with sA / sB)
             float* sT = ((wave < 2) ? &sA[0][0][0] : &sB[0][0][0]) + (wave & 1) * (32 * 65);
             static_assert(sizeof(sA) >= 2 * 32 * 65 * sizeof(float) && sizeof(sB) >= 2 * 32 * 65 * sizeof(float),
                           "the transposition reuses the operand tiles' LDS, two wavefronts in each");

@@ -32,9 +32,10 @@ FP32_MFMA_PEAK_TF = 157.3    # MI355X dense fp32 matrix, published
 MEASURED_TRAFFIC = {
     "cfg2-catalogue-27278": {
         "sparse_z_kernel": {"fetch": 15080 * 1024 * 2.0, "write": 512 * 1024 * 1.0},
-        "fc_gemm_kernel[1024x128x128]": {"fetch": 683 * 1024 * 2.0, "write": 512 * 1024 * 1.0},
-        "fc_gemm_kernel[1024x128x27278]": {"fetch": 11370 * 1024 * 2.0, "write": 142900 * 1024 * 1.0},
-        "topk_scan_kernel": {"fetch": 58550 * 1024 * 2.0, "write": 128 * 1024 * 1.0},
+        "fc_small_kernel[1024x128x128]": {"fetch": 1107 * 1024 * 2.0, "write": 512 * 1024 * 1.0},
+        "fc_gemm_kernel[1024x128x27278]": {"fetch": 11470 * 1024 * 2.0, "write": 147200 * 1024 * 1.0},
+        "topk_scan_kernel": {"fetch": 58540 * 1024 * 2.0, "write": 128 * 1024 * 1.0},
+        "topk_guided_kernel": {"fetch": 10610 * 1024 * 2.0, "write": 128 * 1024 * 1.0},
     },
 }
 
@@ -128,15 +129,25 @@ def network_bench(args, pkg, lib):
     kernels["sparse_z_kernel"] = {"bound": "hbm", "ms": ms, "achieved": spmm_bytes / ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                   "algorithmic_bytes": spmm_bytes}
 
+    # the dense layers as the timed step runs them: the last one also leaves segment maxima for the guided top-K
+    gp = DevicePipeline(p, lib, guided=True)
+    gp.step()
+    pkg.check(lib.dsx_sync())
+    last = len(pipe.W) - 1
     for l in range(1, len(pipe.W)):
         kk, n = p.widths[l], p.widths[l + 1]
 
         def k_fc(l=l, kk=kk, n=n):
-            pkg.check(lib.dsx_fc_forward(ptr(pipe.units[l - 1]), kk, ptr(pipe.W[l]), 0, ptr(pipe.b[l]), ptr(pipe.units[l]), n, B, kk, n, 0,
-                                         p.acts[l], params))
+            if l == last:
+                pkg.check(lib.dsx_fc_forward_segmax(ptr(gp.units[l - 1]), kk, ptr(gp.W[l]), 0, ptr(gp.b[l]), ptr(gp.units[l]), n, B, kk, n,
+                                                    p.acts[l], params, ptr(gp.seg_max), C.byref(gp.seg_width)))
+            else:
+                pkg.check(lib.dsx_fc_forward(ptr(pipe.units[l - 1]), kk, ptr(pipe.W[l]), 0, ptr(pipe.b[l]), ptr(pipe.units[l]), n, B, kk, n, 0,
+                                             p.acts[l], params))
         flops = 2.0 * B * kk * n
         ms = time_launches(pkg, lib, k_fc, reps)
-        name = "fc_gemm_kernel[%dx%dx%d]" % (B, kk, n)
+        small = (kk in (128, 256)) and B * n <= (1 << 20)
+        name = "%s[%dx%dx%d]" % ("fc_small_kernel" if small else "fc_gemm_kernel", B, kk, n)
         kernels[name] = {"bound": "mfma", "ms": ms, "achieved": flops / ms / 1e9, "peak": FP32_MFMA_PEAK_TF, "unit": "TFLOP/s",
                          "algorithmic_flops": flops}
 
@@ -146,6 +157,12 @@ def network_bench(args, pkg, lib):
     ms = time_launches(pkg, lib, k_topk, reps)
     kernels["topk_scan_kernel"] = {"bound": "hbm", "ms": ms, "achieved": topk_bytes / ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                    "algorithmic_bytes": topk_bytes}
+    if gp.seg_width.value:
+        # what the timed step runs when the output layer left segment maxima; priced with the scan's algorithmic bytes (it reads
+        # a fraction of them, so the figure can exceed the roofline: it measures the work avoided, not bandwidth)
+        ms = time_launches(pkg, lib, lambda: gp.topk(), reps)
+        kernels["topk_guided_kernel"] = {"bound": "hbm", "ms": ms, "achieved": topk_bytes / ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                         "algorithmic_bytes": topk_bytes, "note": "reads only the segments that can hold a result"}
     for v in kernels.values():
         v["frac"] = v["achieved"] / v["peak"]
 
