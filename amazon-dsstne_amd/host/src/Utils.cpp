@@ -11,6 +11,33 @@
 
 using namespace std;
 
+char* getCmdOption(char** begin, char** end, const string& option)
+{
+    char** it = find(begin, end, option);
+    return (it != end && it + 1 != end) ? *(it + 1) : nullptr;
+}
+
+bool cmdOptionExists(char** begin, char** end, const string& option) { return find(begin, end, option) != end; }
+
+string getRequiredArgValue(int argc, char** argv, string flag, string message, void (*usage)())
+{
+    char* value = getCmdOption(argv, argv + argc, flag);
+    if (!value) {   // missing flag, or a flag without a value after it
+        cout << "Error: Missing required argument: " << flag << ": " << message << endl;
+        if (usage) usage();
+        exit(1);
+    }
+    return string(value);
+}
+
+string getOptionalArgValue(int argc, char** argv, string flag, string defaultValue)
+{
+    char* value = getCmdOption(argv, argv + argc, flag);
+    return value ? string(value) : defaultValue;
+}
+
+bool isArgSet(int argc, char** argv, string flag) { return cmdOptionExists(argv, argv + argc, flag); }
+
 vector<string> split(const string& s, char delim)
 {
     vector<string> out;

@@ -3,11 +3,14 @@
 // tests of tst/unittests.
 #include <cmath>
 #include <fstream>
+#include <map>
+#include <sstream>
 #include <unordered_map>
 
 #include "amazon/dsstne/engine/NNTypes.h"
 #include "amazon/dsstne/knn/KnnExactGpu.h"
 #include "amazon/dsstne/utils/Filters.h"
+#include "amazon/dsstne/utils/NetCDFhelper.h"
 #include "amazon/dsstne/utils/Utils.h"
 #include "NcClassic.h"
 #include "check.h"
@@ -234,6 +237,119 @@ static int writeCdf2(const string& file)
     return 0;
 }
 
+// ---- index files and sample text (the cases of tst/unittests/TestNetCDFhelper.cpp, plus the sample parser) ------------------
+static void testLoadIndex()
+{
+    const std::map<string, unsigned int> valid = {{"110510", 26743}, {"120372", 26744}, {"abc", 7}, {"x y", 0}};
+    auto feed = [&](stringstream& in) {
+        for (const auto& e : valid) in << e.first << "\t" << e.second << "\n";
+    };
+    {   // valid input
+        stringstream in, out;
+        feed(in);
+        unordered_map<string, unsigned int> idx;
+        CHECK(loadIndex(idx, in, out));
+        CHECK(out.str().find("Error") == string::npos);
+        CHECK_EQ(idx.size(), valid.size());
+        for (const auto& e : valid) CHECK(idx.count(e.first) && idx[e.first] == e.second);
+    }
+    {   // a whole entry twice
+        stringstream in, out;
+        feed(in);
+        in << valid.begin()->first << "\t" << valid.begin()->second << "\n";
+        unordered_map<string, unsigned int> idx;
+        CHECK(!loadIndex(idx, in, out));
+        CHECK(out.str().find("Error") != string::npos);
+    }
+    {   // a label twice with another index
+        stringstream in, out;
+        feed(in);
+        in << valid.begin()->first << "\t123\n";
+        unordered_map<string, unsigned int> idx;
+        CHECK(!loadIndex(idx, in, out));
+        CHECK(out.str().find("Error") != string::npos);
+    }
+    for (const char* bad : {"\t123\n", "123\n", "110510\t123\t121017\n"}) {   // no label; no tab; an extra tab
+        stringstream in(bad), out;
+        unordered_map<string, unsigned int> idx;
+        CHECK(!loadIndex(idx, in, out));
+        CHECK(out.str().find("Error") != string::npos);
+    }
+}
+
+static void testParseSamplesAndDatasetFile(const string& dir)
+{
+    unordered_map<string, unsigned int> features = {{"f0", 0}, {"f1", 1}, {"f2", 2}};
+    unordered_map<string, unsigned int> samples;
+    const string text =
+        "s0\tf1,3.5:f2\n"
+        "\n"                      // empty line: ignored
+        "no tab on this line\n"   // malformed: skipped with a warning
+        "s1\tf0,2,9:unknown,1:f2,0.25:\n"   // a third field is ignored (warning), an unknown feature is dropped, an empty tuple is skipped
+        "s2\t\n"                 // a sample without data points
+        "s0\tf0,1.5\n";          // the same sample again: the last line wins
+    {
+        stringstream in(text), out;
+        bool fu = false, su = false;
+        std::map<unsigned int, vector<unsigned int>> sig;
+        std::map<unsigned int, vector<float>> val;
+        CHECK(parseSamples(in, false, features, samples, fu, su, sig, val, out));
+        CHECK(!fu && su);
+        CHECK_EQ(features.size(), 3u);
+        CHECK_EQ(samples.size(), 3u);
+        CHECK(samples["s0"] == 0 && samples["s1"] == 1 && samples["s2"] == 2);
+        CHECK(sig[0] == vector<unsigned int>({0}) && val[0] == vector<float>({1.5f}));
+        CHECK(sig[1] == vector<unsigned int>({0, 2}) && val[1] == vector<float>({2.0f, 0.25f}));
+        CHECK(sig[2].empty());
+        CHECK(out.str().find("Warning") != string::npos);
+    }
+    {   // with feature updates an unknown feature gets the next index
+        stringstream in("s9\tnew,1:f1\n"), out;
+        bool fu = false, su = false;
+        std::map<unsigned int, vector<unsigned int>> sig;
+        std::map<unsigned int, vector<float>> val;
+        unordered_map<string, unsigned int> f2 = features, s2;
+        CHECK(parseSamples(in, true, f2, s2, fu, su, sig, val, out));
+        CHECK(fu && f2["new"] == 3);
+        CHECK(sig[0] == vector<unsigned int>({3, 1}) && val[0] == vector<float>({1.0f, 0.0f}));
+    }
+    // file -> CSR in sample-index order -> dataset file -> read back
+    const string samplesFile = dir + "/samples.txt";
+    {
+        ofstream f(samplesFile);
+        f << "b\tf2,1:f0,1\n" << "a\tf1,7\n";
+    }
+    unordered_map<string, unsigned int> sidx = {{"a", 0}};   // "a" is known: it stays row 0 although it comes second
+    vector<unsigned int> vs, ve, vi;
+    vector<float> vd;
+    stringstream out;
+    CHECK(generateNetCDFIndexes(samplesFile, false, dir + "/features.idx", dir + "/samples.idx", features, sidx, vs, ve, vi, vd, out));
+    CHECK(vs == vector<unsigned int>({0, 1}) && ve == vector<unsigned int>({1, 3}));
+    CHECK(vi == vector<unsigned int>({1, 2, 0}) && vd == vector<float>({7.0f, 1.0f, 1.0f}));
+    CHECK(fileExists(dir + "/samples.idx") && !fileExists(dir + "/features.idx"));   // only the index that changed is exported
+    unordered_map<string, unsigned int> reread;
+    CHECK(loadIndexFromFile(reread, dir + "/samples.idx", out) && reread.size() == 2 && reread["b"] == 1);
+    CHECK_EQ(roundUpMaxIndex(3), 128u);
+    CHECK_EQ(roundUpMaxIndex(128), 128u);
+    CHECK_EQ(roundUpMaxIndex(129), 256u);
+    for (int analog = 0; analog < 2; analog++) {
+        const string nc = dir + (analog ? "/analog.nc" : "/boolean.nc");
+        if (analog) writeNetCDFFile(vs, ve, vi, vd, nc, "gl_input", (unsigned int)features.size());
+        else writeNetCDFFile(vs, ve, vi, nc, "gl_input", (unsigned int)features.size());
+        ncc::Reader r(nc);
+        CHECK_EQ(r.att("datasets").asUInt64(), 1u);
+        CHECK(r.att("name0").asString() == "gl_input");
+        CHECK_EQ(r.att("attributes0").asUInt64(), analog ? (uint64_t)NNDataSetEnums::Sparse : (uint64_t)(NNDataSetEnums::Sparse | NNDataSetEnums::Boolean));
+        CHECK_EQ(r.att("dataType0").asUInt64(), analog ? (uint64_t)NNDataSetEnums::Float : (uint64_t)NNDataSetEnums::UInt);
+        CHECK_EQ(r.att("width0").asUInt64(), 128u);
+        CHECK_EQ(r.dim("examplesDim0"), 2u);
+        vector<uint64_t> s64;
+        r.read<uint64_t>("sparseEnd0", s64);   // stored as 32-bit offsets, widened on reading
+        CHECK(s64 == vector<uint64_t>({1, 3}));
+        CHECK_EQ(r.hasVar("sparseData0"), analog != 0);
+    }
+}
+
 int main(int argc, char** argv)
 {
     if (argc > 2 && string(argv[1]) == "--dump-network") return dumpNetwork(argv[2]);
@@ -244,5 +360,7 @@ int main(int argc, char** argv)
     testFilters(dir);
     testTopKsort();
     testKnnHost(dir);
+    testLoadIndex();
+    testParseSamplesAndDatasetFile(dir);
     return finish("test_host_cpu");
 }

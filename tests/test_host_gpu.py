@@ -139,6 +139,73 @@ def test_native_embedding_example(pkg, dsx, orc, synth, tmp_path):
     assert_topk_parity(keys, idx, ref_keys, ref_idx, ref_unit, "native embedding example")
 
 
+def test_predict_tool_end_to_end(pkg, dsx, orc, synth, tmp_path):
+    """utils/Predict.cpp's flow with the reference's flags: index files + samples text -> dataset file -> network file ->
+    batches of PredictBatch + NNRecsGenerator::generateRecs (top-5K on the device with the samples filter, K written)."""
+    from amazon_dsstne_amd import host_api
+    exe = os.path.join(ROOT, "amazon-dsstne_amd", "predict")
+    if not os.path.exists(exe):
+        pytest.fail("%s is missing: run __graft_entry__.build()" % exe)
+    p = synth.config(1, batches=3)          # 96 samples, batch 32, 1024 items, top-10
+    p.examples -= 7                          # 89 samples: the last batch is short
+    p.unique_examples -= 7
+    p.start, p.end = p.start[:89], p.end[:89]
+    net = host_api.Network(p, dataset="gl_input")
+    netfile = str(tmp_path / "net.nc")
+    net.save(netfile)
+    net.close()
+    N = p.widths[0]
+    with open(tmp_path / "in.idx", "w") as f:
+        for i in range(N):
+            f.write("item%d\t%d\n" % (i, i))
+    with open(tmp_path / "out.idx", "w") as f:
+        for i in reversed(range(N)):       # order of the lines does not matter
+            f.write("item%d\t%d\n" % (i, i))
+    rows = []
+    for r in range(p.examples):
+        cols = p.sparse_index[int(p.start[r]):int(p.end[r])]
+        rows.append("user%d\t" % r + ":".join("item%d,1" % c for c in cols))
+    (tmp_path / "samples.txt").write_text("\n".join(rows) + "\n")
+    # the filter file lists every sample's own items with multiplier 0 (no value given)
+    with open(tmp_path / "filter.txt", "w") as f:
+        for r in range(p.examples):
+            cols = p.sparse_index[int(p.start[r]):int(p.end[r])]
+            f.write("user%d\t" % r + ":".join("item%d" % c for c in cols) + "\n")
+    recs = tmp_path / "recs.txt"
+    r = subprocess.run([exe, "-d", "gl", "-n", netfile, "-r", str(tmp_path / "samples.txt"), "-i", str(tmp_path / "in.idx"), "-o",
+                        str(tmp_path / "out.idx"), "-f", str(tmp_path / "filter.txt"), "-s", str(recs), "-k", str(p.k), "-b", str(p.batch),
+                        "-p", "8.6f"], cwd=str(tmp_path), stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout[-3000:]
+    lines = recs.read_text().splitlines()
+    assert len(lines) == p.examples, r.stdout[-2000:]
+    idx = np.zeros((p.examples, p.k), dtype=np.uint32)
+    keys = np.zeros((p.examples, p.k), dtype=np.float32)
+    for n, line in enumerate(lines):
+        who, cells = line.split("\t")
+        assert who == "user%d" % n
+        cells = [c for c in cells.split(":") if c]
+        assert len(cells) == p.k
+        for j, c in enumerate(cells):
+            name, score = c.split(",")
+            idx[n, j], keys[n, j] = int(name[4:]), float(score)
+    ref_keys = np.zeros_like(keys)
+    ref_idx = np.zeros_like(idx)
+    ref_scores = np.zeros((p.examples, N), dtype=np.float32)
+    for pos in range(0, p.examples, p.batch):
+        rows_here = min(p.batch, p.examples - pos)
+        _, u, _, _ = orc.forward(p, pos, rows_here, filtered=False, want_unit=True, want_topk=False)
+        _, _, k_, i_ = orc.forward(p, pos, rows_here, filtered=True)
+        orc.lib().orc_apply_filter(u.ctypes.data, rows_here, N, 0, pos, None, p.start.ctypes.data, p.end.ctypes.data,
+                                   p.sparse_index.ctypes.data, None)
+        ref_keys[pos:pos + rows_here], ref_idx[pos:pos + rows_here], ref_scores[pos:pos + rows_here] = k_, i_, u
+    mism = idx != ref_idx
+    if mism.any():
+        rws, cls = np.nonzero(mism)
+        gap = np.abs(ref_scores[rws, idx[rws, cls]].astype(np.float64) - ref_keys[rws, cls].astype(np.float64))
+        assert gap.max() < 1e-5
+    assert np.allclose(keys, ref_keys, rtol=1e-4, atol=2e-6)        # printed with six decimals
+
+
 def test_soft_errors_do_not_abort(pkg, dsx, synth, capfd):
     from amazon_dsstne_amd import host_api
     p = synth.config(1)
