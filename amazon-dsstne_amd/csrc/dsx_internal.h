@@ -57,7 +57,7 @@ namespace dsx {
 int topk_run(const float* in, uint32_t pitch, uint32_t width, uint32_t batch, uint32_t k, float* keys, uint32_t* values,
              uint32_t position, const uint32_t* index, const uint64_t* fstart, const uint64_t* fend, const uint32_t* fidx,
              const float* fmul, uint32_t col_offset, uint64_t* partial, uint32_t partial_slots, uint32_t partial_slot0,
-             uint32_t forced_segments);
+             uint32_t forced_segments, uint32_t* row_bound = nullptr);
 int topk_merge(const uint64_t* partial, uint32_t slots, uint32_t k, float* keys, uint32_t* values, uint32_t batch);
 // GEMM building block shared with the KNN search (dsx_fc.hip): Z = X.W (+bias, activation), see dsx_fc_forward.
 int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int transposed, const float* bias, float* Z, uint32_t ldz,

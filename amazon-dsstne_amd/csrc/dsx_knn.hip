@@ -2,8 +2,10 @@
 //
 // The item table is walked in column blocks: each block's scores are produced by the fp32 MFMA GEMM into a scratch
 // matrix that stays far smaller than the full [queries x items] product, the block's per-query top-k is taken straight
-// from it into packed partial lists, and one merge pass at the end combines the blocks.
+// from it into packed partial lists, and one merge pass at the end combines the blocks.  A block's k-th score is a lower
+// bound of the query's final k-th score, so every later block starts with it as its admission threshold.
 #include <algorithm>
+#include <hip/hip_runtime.h>
 #include "dsx_internal.h"
 
 namespace dsx {
@@ -22,6 +24,13 @@ static uint32_t knn_block_columns(uint32_t rows_padded, uint32_t num_queries)
 
 static inline size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 
+// a fill kernel rather than hipMemsetAsync: callers may record the search into a HIP graph
+__global__ __launch_bounds__(256) void knn_clear_kernel(uint32_t* p, uint32_t n)
+{
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
 }  // namespace dsx
 
 using namespace dsx;
@@ -33,7 +42,8 @@ size_t dsx_knn_workspace_bytes(uint32_t rows_padded, uint32_t dim, uint32_t num_
     (void)dim;
     const uint32_t cb = knn_block_columns(rows_padded, num_queries);
     const uint32_t blocks = (rows_padded + cb - 1) / cb;
-    return align256((size_t)num_queries * cb * sizeof(float)) + align256((size_t)num_queries * blocks * k * sizeof(uint64_t));
+    return align256((size_t)num_queries * cb * sizeof(float)) + align256((size_t)num_queries * blocks * k * sizeof(uint64_t)) +
+           align256((size_t)num_queries * sizeof(uint32_t));
 }
 
 int dsx_knn_search(const float* items, uint32_t rows_padded, uint32_t padding, uint32_t dim, const float* queries,
@@ -69,7 +79,9 @@ int dsx_knn_search(const float* items, uint32_t rows_padded, uint32_t padding, u
     const uint32_t blocks = (M + cb - 1) / cb;
     float* block_scores = (float*)workspace;
     uint64_t* partial = (uint64_t*)((char*)workspace + align256((size_t)num_queries * cb * sizeof(float)));
-    (void)blocks_alloc;
+    // per query: key of a score that k items of the blocks done so far reach; later blocks admit nothing below it
+    uint32_t* row_bound = (uint32_t*)((char*)partial + align256((size_t)num_queries * blocks_alloc * k * sizeof(uint64_t)));
+    hipLaunchKernelGGL(knn_clear_kernel, dim3((num_queries + 255) / 256), dim3(256), 0, ctx().stream, row_bound, num_queries);
 
     hipStream_t s = ctx().stream;
     hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
@@ -85,7 +97,7 @@ int dsx_knn_search(const float* items, uint32_t rows_padded, uint32_t padding, u
         if (rc) break;
         if (elapsed_ms) hipEventRecord(ev[1], s);
         rc = topk_run(block_scores, cb, ncols, num_queries, k, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr, c0, partial,
-                      blocks, blk, 1);
+                      blocks, blk, 1, row_bound);
         if (rc) break;
         if (elapsed_ms) {
             hipEventRecord(ev[2], s);

@@ -287,6 +287,8 @@ struct TopKArgs {
     uint64_t* partial;          // [batch][partial_slots][k]
     uint32_t partial_slots;
     uint32_t partial_slot0;     // this launch writes slots partial_slot0 + segment
+    // column blocks of one wide matrix (KNN): key of a score that k earlier columns of the row reach, 0 = none yet; raised here
+    uint32_t* row_bound;        // [batch]
     // guided variant: maxima of the row's 64-column segments, left by the producer of `in`
     const float* seg_max;       // [batch][nseg]
     uint32_t nseg;
@@ -389,6 +391,10 @@ __device__ __forceinline__ void finish_row(WaveTopK<R>& list, uint64_t (*sStage)
         if (word0 != 0 && place0 < a.k) write_slot(place0, word0);
         if (word1 != 0 && place1 < a.k) write_slot(place1, word1);
         for (uint32_t p = total + lane; p < a.k; p += kWave) write_slot(p, 0ull);
+        if (a.row_bound) {   // this block's k-th score bounds the row's final k-th from below
+            if (word0 != 0 && place0 == a.k - 1) atomicMax(&a.row_bound[b], (uint32_t)(word0 >> 32));
+            if (word1 != 0 && place1 == a.k - 1) atomicMax(&a.row_bound[b], (uint32_t)(word1 >> 32));
+        }
         return;
     }
 
@@ -406,6 +412,7 @@ __device__ __forceinline__ void finish_row(WaveTopK<R>& list, uint64_t (*sStage)
     for (int r = 0; r < R; r++) {
         const uint32_t p = r * kWave + lane;
         if (p < a.k) write_slot(p, list.q[r]);
+        if (a.row_bound && p == a.k - 1 && list.q[r] != 0) atomicMax(&a.row_bound[b], (uint32_t)(list.q[r] >> 32));
     }
 }
 
@@ -435,6 +442,10 @@ __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kern
 
     List list;
     list.init(sStage[wave], lane, a.k);
+    if (a.row_bound) {
+        const uint32_t t = a.row_bound[b];   // k columns of earlier blocks of this row reach this score
+        if (t > score_key(-__builtin_inff())) list.prime(t);
+    }
 
     // Software pipeline: the lane's first 2 * CH 16-byte groups are requested before anything else happens (the filter's
     // chain of dependent loads would otherwise sit in front of the scan), and inside the loop two spans are in flight while
@@ -962,7 +973,7 @@ int topk_merge(const uint64_t* partial, uint32_t slots, uint32_t k, float* keys,
 int topk_run(const float* in, uint32_t pitch, uint32_t width, uint32_t batch, uint32_t k, float* keys, uint32_t* values,
              uint32_t position, const uint32_t* index, const uint64_t* fstart, const uint64_t* fend, const uint32_t* fidx,
              const float* fmul, uint32_t col_offset, uint64_t* partial, uint32_t partial_slots, uint32_t partial_slot0,
-             uint32_t forced_segments)
+             uint32_t forced_segments, uint32_t* row_bound)
 {
     const bool filtered = fidx != nullptr;
     TopKArgs a{};
@@ -979,6 +990,7 @@ int topk_run(const float* in, uint32_t pitch, uint32_t width, uint32_t batch, ui
     a.fmul = fmul;
     a.keys = keys;
     a.values = values;
+    a.row_bound = row_bound;
     a.segments = forced_segments ? forced_segments : choose_segments(batch, width, filtered);
     const uint32_t nvec_max = width / 4 + 1;
     const uint32_t gps = (nvec_max + a.segments - 1) / a.segments;
