@@ -3,7 +3,7 @@
 // Sparse Z (the hot one): one 256-lane workgroup per (sample row, column tile).  The row's non-zero column numbers and
 // values are staged in LDS in chunks; the 256 lanes are split into G groups of LPR lanes, a group covers one weight row
 // with VEC consecutive fp32 columns per lane (128-bit gathers when VEC = 4), and the groups walk the non-zeros interleaved
-// (group g takes non-zeros g, g+G, ...), four gathers in flight per lane.  The G partial sums are combined through LDS in
+// (group g takes non-zeros g, g+G, ...), up to sixteen gathers in flight per lane.  The G partial sums are combined through LDS in
 // group order, so the result does not depend on scheduling.  Bias and activation can be applied in the same kernel.
 #include "dsx_device.h"
 #include "dsx_internal.h"

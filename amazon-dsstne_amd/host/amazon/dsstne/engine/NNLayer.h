@@ -47,6 +47,9 @@ private:
     NNFloat _RELUSlope, _ELUAlpha, _SELULambda;
     const Activation _activation;
     const NNFloat _pDropout;
+    const WeightInitialization _weightInit;     // how weights into this layer start when a definition supplies none
+    const NNFloat _weightInitScale;
+    const NNFloat _biasInit;
     bool _bSparse;
     bool _bFastSparse;
     bool _bDirty;

@@ -69,6 +69,7 @@ public:
     void CalculateFilteredTopK(const string& layer, uint32_t k, NNDataSetBase* pFilter, GpuBuffer<NNFloat>* pbKey,
                                GpuBuffer<uint32_t>* pbValue, bool bUseValues = false);
     void SetBatch(uint32_t batch);
+    void Randomize();                           // every connection back to its starting values (engine/NNNetwork.cpp:675-679)
     void SetPosition(uint32_t position);
     void SetShuffleIndices(bool bShuffleIndices);
     void SetCPUValidate(bool bValidate);
@@ -135,5 +136,10 @@ bool SaveNeuralNetworkNetCDF(const NNNetwork& net, const string& fname);
 // Descriptor-level file I/O, usable without a GPU.
 bool LoadNNNetworkDescriptorNetCDF(const string& fname, NNNetworkDescriptor& nd);
 bool SaveNNNetworkDescriptorNetCDF(const string& fname, const NNNetworkDescriptor& nd);
+// Reads a network definition in JSON (engine/NNNetwork.cpp:2792-3760): "N": "auto" layers take their dimensions from the
+// data set of the same name in vDataSet; weights are initialised by each layer's "WeightInit" scheme from the seed given to
+// GpuContext::SetRandomSeed.  Returns NULL after printing a message when the file does not parse or names an unknown key.
+NNNetwork* LoadNeuralNetworkJSON(const string& fname, const uint32_t batch, const vector<NNDataSetBase*>& vDataSet);
+bool LoadNNNetworkDescriptorJSON(const string& fname, NNNetworkDescriptor& nd, const vector<NNDataSetBase*>& vDataSet);
 
 #endif

@@ -45,6 +45,8 @@ private:
              NNFloat maxNorm = 0.0f);
     ~NNWeight();
     NNFloat* GetWeightBuffer() { return _pbWeight ? _pbWeight->_pDevData : NULL; }
+    // Starting values by the output layer's scheme (engine/NNWeight.cpp:500-561); biases start at biasInit.
+    void Randomize();
     uint64_t GetBufferSize() { return _localSize; }
 
 public:

@@ -39,7 +39,8 @@ NNLayer::NNLayer(NNLayerDescriptor& d, uint32_t batch)
     : _name(d._name), _kind(d._kind), _type(d._type), _attributes(d._attributes), _dataSet(d._dataSet), _pDataSet(NULL),
       _vSource(d._vSource), _vSkip(d._vSkip), _Nx(d._Nx), _Ny(d._Ny), _Nz(d._Nz), _Nw(d._Nw), _batch(batch), _localBatch(batch),
       _dimensions(d._dimensions), _RELUSlope(d._RELUSlope), _ELUAlpha(d._ELUAlpha), _SELULambda(d._SELULambda),
-      _activation(d._activation), _pDropout(d._pDropout), _bSparse(d._attributes & NNLayer::Attributes::Sparse), _bFastSparse(false),
+      _activation(d._activation), _pDropout(d._pDropout), _weightInit(d._weightInit), _weightInitScale(d._weightInitScale),
+      _biasInit(d._biasInit), _bSparse(d._attributes & NNLayer::Attributes::Sparse), _bFastSparse(false),
       _bDirty(true), _priority(-1)
 {
     _stride = _Nx * _Ny * _Nz * _Nw;

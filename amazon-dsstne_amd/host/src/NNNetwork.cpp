@@ -86,10 +86,9 @@ NNNetwork::NNNetwork(NNNetworkDescriptor& d, uint32_t batch)
             fatal("NNNetwork::NNNetwork: weight connects unknown layers %s and %s.", wd._inputLayer.c_str(), wd._outputLayer.c_str());
         NNWeight* pWeight = new NNWeight(*in->second, *out->second, wd._bShared, wd._bTransposed, wd._bLocked, wd._norm);
         _vWeight.push_back(pWeight);
-        if (!wd._bShared && wd._vWeight.empty())
-            fatal("NNNetwork::NNNetwork: no weight values supplied between layers %s and %s (random initialisation is a training feature "
-                  "this build does not have).", wd._inputLayer.c_str(), wd._outputLayer.c_str());
-        if (!wd._bShared) {
+        // a definition without values (JSON) starts from the layer's initialisation scheme; shared connections only have biases
+        if (wd._vWeight.empty() || wd._vBias.empty()) pWeight->Randomize();
+        if (!wd._bShared && !wd._vWeight.empty()) {
             if (wd._vWeight.size() < pWeight->_vWeight.size())
                 fatal("NNNetwork::NNNetwork: too few weight values between layers %s and %s.", wd._inputLayer.c_str(), wd._outputLayer.c_str());
             std::copy(wd._vWeight.begin(), wd._vWeight.begin() + pWeight->_vWeight.size(), pWeight->_vWeight.begin());
@@ -132,6 +131,11 @@ NNNetwork::NNNetwork(NNNetworkDescriptor& d, uint32_t batch)
     }
 
     CalculatePropagationOrder();
+}
+
+void NNNetwork::Randomize()
+{
+    for (auto pw : _vWeight) pw->Randomize();
 }
 
 NNNetwork::~NNNetwork()

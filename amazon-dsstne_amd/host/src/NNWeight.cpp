@@ -1,6 +1,7 @@
 // NNWeight.cpp — fully connected weights and biases (reference: engine/NNWeight.cpp:289-479 constructor, 938-1057 setters and
 // getters).  Only the inference state exists: the matrix, the bias vector and their host shadows.
 #include <cinttypes>
+#include <cmath>
 
 #include "amazon/dsstne/engine/NNTypes.h"
 
@@ -44,6 +45,86 @@ NNWeight::NNWeight(NNLayer& inputLayer, NNLayer& outputLayer, bool bShared, bool
 }
 
 NNWeight::~NNWeight() {}
+
+namespace {
+// Counter-based stream: value i of a connection depends only on the process seed, the two layer names and i, so a
+// network gets the same starting weights however its connections are ordered.  (The reference draws from cuRAND's
+// default generator, whose stream is not reproduced here.)
+struct WeightStream {
+    uint64_t key;
+    WeightStream(unsigned long seed, const string& in, const string& out) : key(0x9E3779B97F4A7C15ull ^ (uint64_t)seed)
+    {
+        for (unsigned char c : in) key = (key ^ c) * 0x100000001B3ull;
+        key = (key ^ 0xFFu) * 0x100000001B3ull;
+        for (unsigned char c : out) key = (key ^ c) * 0x100000001B3ull;
+    }
+    uint64_t bits(uint64_t i) const
+    {
+        uint64_t z = key + (i + 1) * 0x9E3779B97F4A7C15ull;
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        return z ^ (z >> 31);
+    }
+    // in (0, 1], like the generator the reference uses
+    float uniform(uint64_t i) const { return (float)((bits(i) >> 40) + 1) * (1.0f / 16777216.0f); }
+    float normal(uint64_t i) const
+    {
+        const uint64_t pair = i >> 1;
+        const float r = sqrtf(-2.0f * logf(uniform(2 * pair))), a = 6.28318530717958647692f * uniform(2 * pair + 1);
+        return (i & 1) ? r * sinf(a) : r * cosf(a);
+    }
+};
+}  // namespace
+
+void NNWeight::Randomize()
+{
+    if (!_bShared) {
+        const WeightStream rng(getGpu()._randomSeed, _inputLayer._name, _outputLayer._name);
+        const NNFloat s = _outputLayer._weightInitScale;
+        const NNFloat nOut = (NNFloat)_outputLayer._stride, nIn = (NNFloat)_inputLayer._stride;
+        NNFloat scale = 0.0f, shift = 0.0f, sigma = 0.0f;
+        bool bNormal = false;
+        switch (_outputLayer._weightInit) {
+        case CaffeXavier:   // uniform in ±s·sqrt(3 / n_out)
+            scale = s * 2.0f * sqrtf(3.0f / nOut);
+            shift = 0.5f * scale;
+            break;
+        case Xavier:        // uniform in ±s·sqrt(6 / (n_out + n_in)) / 2, as the reference scales it
+            scale = s * sqrtf(6.0f / (nOut + nIn));
+            shift = 0.5f * scale;
+            break;
+        case Uniform:       // uniform in ±s
+            scale = 2.0f * s;
+            shift = 0.5f * scale;
+            break;
+        case UnitBall:      // uniform in (0, s]
+            scale = s;
+            break;
+        case Gaussian:      // N(0, s)
+            bNormal = true;
+            sigma = s;
+            break;
+        case SELU:          // N(0, 1 / n_in)
+            bNormal = true;
+            sigma = 1.0f / nIn;
+            break;
+        case Constant:      // the reference's scale-and-shift step computes 0·scale − s here, so every weight is −s
+            shift = s;
+            break;
+        }
+        const uint64_t n = _vWeight.size();
+        if (bNormal) {
+            for (uint64_t i = 0; i < n; i++) _vWeight[i] = sigma * rng.normal(i);
+        } else if (scale != 0.0f) {
+            for (uint64_t i = 0; i < n; i++) _vWeight[i] = rng.uniform(i) * scale - shift;
+        } else {
+            std::fill(_vWeight.begin(), _vWeight.end(), -shift);
+        }
+        _pbWeight->Upload(_vWeight.data());
+    }
+    std::fill(_vBias.begin(), _vBias.end(), _outputLayer._biasInit);
+    _pbBias->Upload(_vBias.data());
+}
 
 bool NNWeight::CopyWeights(const NNWeight* pSrcWeight)
 {

@@ -50,6 +50,17 @@ static NNDataSetBase* makeSparse(const char* name, uint32_t width, uint32_t exam
     return new NNDataSet<T>(examples, unique, (size_t)cap, NNDataSetDimensions(width), indexed != 0, weighted != 0, name);
 }
 
+// Top-K result buffers of in-memory networks: one pair per output layer.
+static void makeResultBuffers(dsstne_context* c)
+{
+    if (c->maxK <= 0) return;
+    vector<const NNLayer*> outs;
+    for (auto it = c->network->GetLayers(NNLayer::Kind::Output, outs); it != outs.end(); ++it) {
+        c->scores[(*it)->GetName()] = new GpuBuffer<NNFloat>((size_t)c->maxK * c->batch);
+        c->indexes[(*it)->GetName()] = new GpuBuffer<uint32_t>((size_t)c->maxK * c->batch);
+    }
+}
+
 extern "C" {
 
 const char* dsstne_last_error(void) { return g_err; }
@@ -112,15 +123,74 @@ dsstne_context* dsstne_create(const char* name, uint32_t batch, int max_k, uint3
     getGpu().SetNeuralNetwork(c->network);
     c->batch = batch;
     c->maxK = max_k;
-    vector<const NNLayer*> outs;
-    for (auto it = c->network->GetLayers(NNLayer::Kind::Output, outs); it != outs.end(); ++it) {
-        if (max_k > 0) {
-            c->scores[(*it)->GetName()] = new GpuBuffer<NNFloat>((size_t)max_k * batch);
-            c->indexes[(*it)->GetName()] = new GpuBuffer<uint32_t>((size_t)max_k * batch);
-        }
-    }
+    makeResultBuffers(c);
     return c;
     CAPI_CATCH(nullptr)
+}
+
+dsstne_context* dsstne_load_definition(const char* definition_file, const char* dataset_file, uint32_t batch, int max_k, uint64_t seed)
+{
+    CAPI_TRY
+    static char arg0[] = "dsstne-capi";
+    char* argv = arg0;
+    getGpu().Startup(1, &argv);
+    getGpu().SetRandomSeed((unsigned long)seed);
+    vector<NNDataSetBase*> vDataSet = LoadNetCDF(dataset_file);
+    if (vDataSet.empty()) {
+        fail("dsstne_load_definition: no data set could be read from %s", dataset_file);
+        getGpu().Shutdown();
+        return nullptr;
+    }
+    NNNetwork* network = LoadNeuralNetworkJSON(definition_file, batch, vDataSet);
+    if (!network) {
+        for (auto d : vDataSet) delete d;
+        getGpu().Shutdown();
+        fail("dsstne_load_definition: %s could not be loaded", definition_file);
+        return nullptr;
+    }
+    dsstne_context* c = new dsstne_context();
+    c->network = network;
+    getGpu().SetNeuralNetwork(network);
+    c->batch = batch;
+    c->maxK = max_k;
+    network->LoadDataSets(vDataSet);
+    for (auto d : vDataSet) c->datasets[d->_name] = d;
+    network->SetPosition(0);
+    makeResultBuffers(c);
+    return c;
+    CAPI_CATCH(nullptr)
+}
+
+int dsstne_get_weights(dsstne_context* c, const char* input_layer, const char* output_layer, float* weights, size_t weight_count,
+                       float* biases, size_t bias_count)
+{
+    CAPI_TRY
+    NNWeight* w = c->net()->GetWeight(input_layer, output_layer);
+    if (!w) return fail("dsstne_get_weights: no connection %s -> %s", input_layer, output_layer);
+    if (weights) {
+        vector<NNFloat> v;
+        if (!w->GetWeights(v) || v.size() > weight_count) return fail("dsstne_get_weights: %zu weights do not fit %zu", v.size(), weight_count);
+        std::copy(v.begin(), v.end(), weights);
+    }
+    if (biases) {
+        vector<NNFloat> v;   // the getters only ever grow the vector they are given
+        if (!w->GetBiases(v) || v.size() > bias_count) return fail("dsstne_get_weights: %zu biases do not fit %zu", v.size(), bias_count);
+        std::copy(v.begin(), v.end(), biases);
+    }
+    return 0;
+    CAPI_CATCH(-1)
+}
+
+int dsstne_set_weights(dsstne_context* c, const char* input_layer, const char* output_layer, const float* weights, size_t weight_count,
+                       const float* biases, size_t bias_count)
+{
+    CAPI_TRY
+    NNWeight* w = c->net()->GetWeight(input_layer, output_layer);
+    if (!w) return fail("dsstne_set_weights: no connection %s -> %s", input_layer, output_layer);
+    if (weights && !w->SetWeights(vector<NNFloat>(weights, weights + weight_count))) return fail("dsstne_set_weights: weights refused");
+    if (biases && !w->SetBiases(vector<NNFloat>(biases, biases + bias_count))) return fail("dsstne_set_weights: biases refused");
+    return 0;
+    CAPI_CATCH(-1)
 }
 
 void dsstne_shutdown(dsstne_context* c)

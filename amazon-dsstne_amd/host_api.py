@@ -37,6 +37,9 @@ SIGNATURES = {
     "dsstne_knn_create": ([_u32, _u32], _vp),
     "dsstne_knn_load": ([_vp, _vp, _u32, _u32, C.POINTER(_cp)], _int),
     "dsstne_knn_load_file": ([_vp, _cp, C.c_char, C.c_char], _int),
+    "dsstne_load_definition": ([_cp, _cp, _u32, _int, C.c_uint64], _vp),
+    "dsstne_get_weights": ([_vp, _cp, _cp, _vp, C.c_size_t, _vp, C.c_size_t], _int),
+    "dsstne_set_weights": ([_vp, _cp, _cp, _vp, C.c_size_t, _vp, C.c_size_t], _int),
     "dsstne_knn_search": ([_vp, _u32, _vp, _u32, _vp, _vp], _int),
     "dsstne_knn_elapsed": ([_vp, C.POINTER(_f32), C.POINTER(_f32)], _int),
     "dsstne_knn_destroy": ([_vp], None),
@@ -136,8 +139,8 @@ class Network:
         _check(self.lib.dsstne_get_topk(self.ctx, layer.encode(), rows, k, scores.ctypes.data, idx.ctypes.data))
         return scores, idx
 
-    def units(self, layer="Output", rows=None):
-        width = self.p.widths[-1] if layer == "Output" else None
+    def units(self, layer="Output", rows=None, width=None):
+        width = width or self.p.widths[-1]
         rows = rows or self.p.batch
         out = np.empty((rows, width), dtype=np.float32)
         _check(self.lib.dsstne_get_units(self.ctx, layer.encode(), out.ctypes.data, out.size))
@@ -150,6 +153,20 @@ class Network:
     def save(self, path):
         _check(self.lib.dsstne_save_network(self.ctx, path.encode()))
 
+    def get_weights(self, input_layer, output_layer, rows, cols, biases=None):
+        """Weights [rows = input width][cols = output width] and the connection's biases (`biases` of them, default cols).
+        A tied connection has no matrix of its own (NNWeight::GetWeights hands back nothing): ask with rows = cols = 0."""
+        w = np.empty((rows, cols), dtype=np.float32)
+        b = np.empty(biases or cols, dtype=np.float32)
+        _check(self.lib.dsstne_get_weights(self.ctx, input_layer.encode(), output_layer.encode(), w.ctypes.data, w.size, b.ctypes.data, b.size))
+        return w, b
+
+    def set_weights(self, input_layer, output_layer, weights=None, biases=None):
+        w = None if weights is None else np.ascontiguousarray(weights, dtype=np.float32)
+        b = None if biases is None else np.ascontiguousarray(biases, dtype=np.float32)
+        _check(self.lib.dsstne_set_weights(self.ctx, input_layer.encode(), output_layer.encode(), None if w is None else w.ctypes.data,
+                                           0 if w is None else w.size, None if b is None else b.ctypes.data, 0 if b is None else b.size))
+
     def sync(self):
         _check(self.lib.dsstne_sync())
 
@@ -157,3 +174,21 @@ class Network:
         if self.ctx:
             self.lib.dsstne_shutdown(self.ctx)
             self.ctx = None
+
+
+class DefinedNetwork(Network):
+    """A network built from a JSON definition file and a dataset file (the training tool's start-up: LoadNetCDF,
+    LoadNeuralNetworkJSON, LoadDataSets); weights start from the definition's initialisation schemes and `seed`."""
+
+    def __init__(self, definition_file, dataset_file, batch, max_k, seed=12134, k=None):
+        self.lib = load_host_library()
+        self.dataset = None
+
+        class _Shape:
+            pass
+        self.p = _Shape()
+        self.p.batch, self.p.k, self.p.widths = batch, (k or max_k), [None]
+        self.max_k = max_k
+        self.ctx = self.lib.dsstne_load_definition(definition_file.encode(), dataset_file.encode(), batch, max_k, seed)
+        if not self.ctx:
+            raise DsxError("dsstne_load_definition failed: %s" % self.lib.dsstne_last_error().decode())

@@ -34,6 +34,19 @@ dsstne_context* dsstne_create(const char* name, uint32_t batch, int max_k, uint3
                               const uint32_t* weight_in, const uint32_t* weight_out, const float* const* weights,
                               const float* const* biases);
 
+/* The training tool's start-up (utils/Train.cpp:119-133) up to the first prediction: LoadNetCDF(dataset_file), then
+ * LoadNeuralNetworkJSON(definition_file, batch, datasets) (engine/NNNetwork.cpp:2792-3760: "N": "auto" layers are sized by
+ * the data set they name), then LoadDataSets.  Weights start from each layer's "WeightInit" scheme and `seed`
+ * (GpuContext::SetRandomSeed); the context owns the data sets.  NULL + dsstne_last_error() on failure. */
+dsstne_context* dsstne_load_definition(const char* definition_file, const char* dataset_file, uint32_t batch, int max_k, uint64_t seed);
+
+/* Weights and biases of the connection input_layer -> output_layer (NNWeight::GetWeights/GetBiases/SetWeights/SetBiases,
+ * engine/NNWeight.cpp:938-1057): weights [width(in)][width(out)] fp32 row-major, biases [width(out)].  A NULL array is skipped. */
+int dsstne_get_weights(dsstne_context* ctx, const char* input_layer, const char* output_layer, float* weights, size_t weight_count,
+                       float* biases, size_t bias_count);
+int dsstne_set_weights(dsstne_context* ctx, const char* input_layer, const char* output_layer, const float* weights, size_t weight_count,
+                       const float* biases, size_t bias_count);
+
 /* Dsstne.shutdown: deletes the network, the datasets created by dsstne_load_datasets and the device context. */
 void dsstne_shutdown(dsstne_context* ctx);
 

@@ -12,6 +12,7 @@
 #include "amazon/dsstne/utils/Filters.h"
 #include "amazon/dsstne/utils/NetCDFhelper.h"
 #include "amazon/dsstne/utils/Utils.h"
+#include "Json.h"
 #include "NcClassic.h"
 #include "check.h"
 
@@ -350,11 +351,185 @@ static void testParseSamplesAndDatasetFile(const string& dir)
     }
 }
 
+
+static void testJsonReader()
+{
+    json::Value v;
+    string err;
+    CHECK(json::parse("{ \"a\" : [1, 2.5e1, -3], // note\n \"b\" : { \"c\" : \"x\\n\\u00e9\\\"\" }, /* c */ \"d\" : true, \"e\" : null, \"f\" : false }", v, err));
+    CHECK(v.isObject() && v.members().size() == 5);
+    CHECK(v.members()[0].first == "a" && v.members()[4].first == "f");   // file order is kept
+    const json::Value* a = v.find("a");
+    CHECK(a && a->isArray() && a->size() == 3);
+    CHECK_EQ((*a)[1].asDouble(), 25.0);
+    CHECK_EQ((*a)[2].asInt(), (int64_t)-3);
+    CHECK(v.find("b")->find("c")->asString() == "x\n\xc3\xa9\"");
+    CHECK(v.find("d")->asBool() && !v.find("f")->asBool() && v.find("e")->isNull());
+    CHECK(v.find("zzz") == nullptr);
+    CHECK_EQ(v.find("d")->size(), (size_t)1);            // a scalar reads as an array of one
+    CHECK(&(*v.find("d"))[0] == v.find("d"));
+    bool threw = false;
+    try { v.find("a")->asString(); } catch (std::runtime_error&) { threw = true; }
+    CHECK(threw);
+    CHECK(json::parse("[]", v, err) && v.isArray() && v.size() == 0);
+    CHECK(json::parse(" 7 ", v, err) && v.asInt() == 7);
+    for (const char* bad : {"{", "{\"a\" 1}", "[1,]", "{\"a\":1,}", "\"abc", "tru", "{\"a\":1} x", "/* open", "[1 2]", "{'a':1}", ""}) {
+        err.clear();
+        CHECK(!json::parse(bad, v, err));
+        CHECK(err.find("line ") == 0);
+    }
+    CHECK(!json::parse("{\n\n  \"a\" : ?\n}", v, err) && err.find("line 3, column 9") == 0);
+    CHECK(json::lower("ReLU Max") == "relu max");
+}
+
+static const NNWeightDescriptor* findWeight(const NNNetworkDescriptor& nd, const string& in, const string& out)
+{
+    for (auto& w : nd._vWeightDescriptor)
+        if (w._inputLayer == in && w._outputLayer == out) return &w;
+    return nullptr;
+}
+
+static void testNetworkDefinitions(const string& dir, const string& golden)
+{
+    const vector<NNDataSetBase*> none;
+    {   // data file of the reference's tests: tst/test_data/validate_L2_LRelu_02.json
+        NNNetworkDescriptor nd;
+        CHECK(LoadNNNetworkDescriptorJSON(golden + "/validate_L2_LRelu_02.json", nd, none));
+        CHECK(nd._name == "L2 1d regression");
+        CHECK_EQ((int)nd._kind, (int)NNNetwork::Kind::FeedForward);
+        CHECK_EQ((int)nd._errorFunction, (int)ErrorFunction::L2);
+        CHECK(!nd._bShuffleIndices);
+        CHECK_EQ(nd._vLayerDescriptor.size(), (size_t)3);
+        const NNLayerDescriptor& in = nd._vLayerDescriptor[0];
+        const NNLayerDescriptor& hid = nd._vLayerDescriptor[1];
+        const NNLayerDescriptor& out = nd._vLayerDescriptor[2];
+        CHECK(in._name == "Input" && in._kind == NNLayer::Kind::Input && in._Nx == 2 && in._dataSet == "input");
+        CHECK(in._attributes == NNLayer::Attributes::Sparse);
+        CHECK(hid._name == "Hidden" && hid._kind == NNLayer::Kind::Hidden && hid._activation == Activation::LeakyRectifiedLinear);
+        CHECK_EQ(hid._RELUSlope, 0.5f);
+        CHECK(hid._vSource == vector<string>({"Input"}));
+        CHECK(out._kind == NNLayer::Kind::Output && out._activation == Activation::Linear && out._dataSet == "output");
+        CHECK(out._vSource == vector<string>({"Input"}));      // the output reads the input, not the hidden layer
+        CHECK_EQ(nd._vWeightDescriptor.size(), (size_t)2);
+        CHECK(findWeight(nd, "Input", "Hidden") && findWeight(nd, "Input", "Output") && !findWeight(nd, "Hidden", "Output"));
+        CHECK(nd._vWeightDescriptor[0]._vWeight.empty() && !nd._vWeightDescriptor[0]._bShared);
+        // layers without a slope of their own take the network's (default 0.0... is stored, never NaN)
+        CHECK(!std::isnan(out._RELUSlope) && !std::isnan(out._ELUAlpha) && !std::isnan(out._SELULambda));
+    }
+    {   // the MovieLens sample definition sizes two layers from data sets, which are not there
+        NNNetworkDescriptor nd;
+        CHECK(!LoadNNNetworkDescriptorJSON(golden + "/movielens_config.json", nd, none));
+    }
+    {
+        NNNetworkDescriptor nd;
+        CHECK(LoadNNNetworkDescriptorJSON(golden + "/tied_autoencoder.json", nd, none));
+        CHECK(nd._name == "tied autoencoder" && nd._kind == NNNetwork::Kind::AutoEncoder && nd._errorFunction == ErrorFunction::CrossEntropy);
+        CHECK(nd._bShuffleIndices);
+        CHECK_EQ(nd._RELUSlope, 0.125f);
+        CHECK_EQ(nd._ELUAlpha, 1.5f);
+        CHECK_EQ(nd._decay, 0.25f);
+        CHECK_EQ(nd._deltaBoost_one, 30.0f);
+        CHECK_EQ(nd._deltaBoost_zero, 2.0f);
+        CHECK_EQ(nd._LRN_k, 3.0f);
+        CHECK_EQ(nd._LRN_n, 7u);
+        CHECK_EQ(nd._LRN_alpha, 0.5f);
+        CHECK_EQ(nd._LRN_beta, 0.25f);
+        CHECK_EQ(nd._maxout_k, 4u);
+        CHECK_EQ(nd._vLayerDescriptor.size(), (size_t)5);
+        const auto& L = nd._vLayerDescriptor;
+        CHECK(L[0]._name == "Input0" && L[0]._kind == NNLayer::Kind::Input && L[0]._Nx == 96 && (L[0]._attributes & NNLayer::Attributes::Sparse));
+        CHECK(L[1]._name == "Enc" && L[1]._kind == NNLayer::Kind::Hidden && L[1]._vSource == vector<string>({"Input0"}));
+        CHECK(L[1]._weightInit == Gaussian && L[1]._weightInitScale == 0.01f && L[1]._biasInit == 0.5f);
+        CHECK_EQ(L[1]._RELUSlope, 0.125f);                       // network default
+        CHECK(L[2]._activation == Activation::ExponentialLinear && L[2]._ELUAlpha == 0.75f && L[2]._pDropout == 0.5f);
+        CHECK(L[2]._vSkip == vector<string>({"Enc"}) && L[2]._dimensions == 1 && L[2]._Nx == 32);
+        CHECK(L[2]._weightInit == Constant);
+        CHECK(L[3]._kind == NNLayer::Kind::Hidden && L[3]._vSource == vector<string>({"Input0", "Enc"}) && L[3]._weightNorm == 2.0f);
+        CHECK_EQ(L[3]._ELUAlpha, 1.5f);
+        CHECK(L[4]._kind == NNLayer::Kind::Output && L[4]._name == "Out" && L[4]._dataSet == "out");
+        CHECK_EQ(nd._vWeightDescriptor.size(), (size_t)6);
+        const NNWeightDescriptor* tied = findWeight(nd, "Mid", "Out");
+        CHECK(tied && tied->_bShared && tied->_bTransposed && tied->_sourceInputLayer == "Input0" && tied->_sourceOutputLayer == "Enc");
+        const NNWeightDescriptor* side = findWeight(nd, "Side", "Out");
+        CHECK(side && !side->_bShared);
+        CHECK(findWeight(nd, "Enc", "Side") && findWeight(nd, "Enc", "Side")->_norm == 2.0f);
+        // the descriptor survives the binary network format (weights stay empty)
+        NNNetworkDescriptor back;
+        CHECK(SaveNNNetworkDescriptorNetCDF(dir + "/tied.nc", nd) && LoadNNNetworkDescriptorNetCDF(dir + "/tied.nc", back));
+        CHECK(back._vLayerDescriptor.size() == 5 && back._vLayerDescriptor[2]._vSkip == vector<string>({"Enc"}));
+        CHECK(back._vWeightDescriptor.size() == 6 && back._vWeightDescriptor[4]._bTransposed);
+    }
+    // what the loader refuses, one definition each
+    struct Case { const char* what; const char* text; };
+    const Case refused[] = {
+        {"old version", "{\"Version\": 0.5, \"Layers\": [{\"N\": 2}, {\"N\": 2}]}"},
+        {"unknown network key", "{\"Layers\": [{\"N\": 2}, {\"N\": 2}], \"Colour\": 1}"},
+        {"unknown network kind", "{\"Kind\": \"Recurrent\", \"Layers\": [{\"N\": 2}, {\"N\": 2}]}"},
+        {"unknown error function", "{\"ErrorFunction\": \"L3\", \"Layers\": [{\"N\": 2}, {\"N\": 2}]}"},
+        {"unknown layer key", "{\"Layers\": [{\"N\": 2}, {\"N\": 2, \"Colour\": 1}]}"},
+        {"activation on an input layer", "{\"Layers\": [{\"N\": 2, \"Activation\": \"Relu\"}, {\"N\": 2}]}"},
+        {"data set on a hidden layer", "{\"Layers\": [{\"N\": 2}, {\"N\": 2, \"DataSet\": \"x\"}, {\"N\": 2}]}"},
+        {"source on an input layer", "{\"Layers\": [{\"N\": 2, \"Source\": \"x\"}, {\"N\": 2}]}"},
+        {"auto on a hidden layer", "{\"Layers\": [{\"N\": 2}, {\"N\": \"auto\"}, {\"N\": 2}]}"},
+        {"auto without its data set", "{\"Layers\": [{\"N\": \"auto\", \"DataSet\": \"nowhere\"}, {\"N\": 2}]}"},
+        {"duplicate layer name", "{\"Layers\": [{\"Name\": \"a\", \"N\": 2}, {\"Name\": \"a\", \"N\": 2}]}"},
+        {"five dimensions", "{\"Layers\": [{\"N\": [1, 2, 3, 4, 5]}, {\"N\": 2}]}"},
+        {"unknown activation", "{\"Layers\": [{\"N\": 2}, {\"N\": 2, \"Activation\": \"Swish\"}]}"},
+        {"unknown layer kind", "{\"Layers\": [{\"N\": 2}, {\"N\": 2, \"Kind\": \"Middle\"}]}"},
+        {"unknown layer type", "{\"Layers\": [{\"N\": 2}, {\"N\": 2, \"Type\": \"Dense\"}]}"},
+        {"unknown weight scheme", "{\"Layers\": [{\"N\": 2}, {\"N\": 2, \"WeightInit\": {\"Scheme\": \"He\"}}]}"},
+        {"unknown weight init field", "{\"Layers\": [{\"N\": 2}, {\"N\": 2, \"WeightInit\": {\"Gain\": 1}}]}"},
+        {"unknown shared weight field", "{\"Layers\": [{\"N\": 2}, {\"N\": 2}, {\"N\": 2, \"SharedWeights\": {\"Transpose\": true}}]}"},
+        {"shared weight without its source", "{\"Layers\": [{\"N\": 2}, {\"N\": 2}, {\"N\": 2, \"SharedWeights\": {\"InputLayer\": \"nope\"}}]}"},
+        {"unknown penalty parameter", "{\"SparsenessPenalty\": {\"q\": 1}, \"Layers\": [{\"N\": 2}, {\"N\": 2}]}"},
+        {"not JSON", "{\"Layers\": [{\"N\": 2}, {\"N\": 2}]"},
+    };
+    for (auto& c : refused) {
+        const string f = dir + "/refused.json";
+        { ofstream o(f); o << c.text; }
+        NNNetworkDescriptor nd;
+        if (LoadNNNetworkDescriptorJSON(f, nd, none)) {
+            printf("FAILED: definition with %s was accepted\n", c.what);
+            CHECK(false);
+        } else
+            CHECK(true);
+    }
+    {   // defaults: kinds by position, names by kind and position, Sigmoid, Xavier, chain of sources, multi-dimensional N
+        const string f = dir + "/defaults.json";
+        { ofstream o(f); o << "{\"Layers\": [{\"N\": [4, 3, 2]}, {\"N\": 5}, {\"N\": 6, \"Sparse\": false}], \"Denoising\": {\"p\": 0.25},"
+                              " \"SparsenessPenalty\": {\"p\": 0.1, \"beta\": 0.5}}"; }
+        NNNetworkDescriptor nd;
+        CHECK(LoadNNNetworkDescriptorJSON(f, nd, none));
+        const auto& L = nd._vLayerDescriptor;
+        CHECK(L.size() == 3 && L[0]._name == "Input0" && L[1]._name == "Hidden1" && L[2]._name == "Output2");
+        CHECK(L[0]._Nx == 4 && L[0]._Ny == 3 && L[0]._Nz == 2 && L[0]._dimensions == 3);
+        CHECK(L[1]._activation == Activation::Sigmoid && L[1]._weightInit == Xavier && L[1]._vSource == vector<string>({"Input0"}));
+        CHECK(L[2]._vSource == vector<string>({"Hidden1"}) && L[2]._attributes == NNLayer::Attributes::None);
+        CHECK(nd._bDenoising && nd._bSparsenessPenalty);
+        CHECK(!(L[0]._attributes & NNLayer::Attributes::Denoising));   // only sparse input layers are denoised
+        CHECK_EQ(nd._vWeightDescriptor.size(), (size_t)2);
+    }
+    {   // a single layer object instead of an array, a convolutional entry with a kernel (parsed, not built)
+        const string f = dir + "/conv.json";
+        { ofstream o(f); o << "{\"Layers\": [{\"N\": [8, 8, 3]}, {\"Type\": \"Convolutional\", \"N\": 16, \"Kernel\": [3, 3], \"KernelStride\": 2},"
+                              " {\"Type\": \"Pooling\", \"Function\": \"Max\", \"Kernel\": [2, 2]}, {\"N\": 10, \"Activation\": \"SoftMax\"}]}"; }
+        NNNetworkDescriptor nd;
+        CHECK(LoadNNNetworkDescriptorJSON(f, nd, none));
+        const auto& L = nd._vLayerDescriptor;
+        CHECK(L[1]._type == NNLayer::Type::Convolutional && L[1]._kernelX == 3 && L[1]._kernelY == 3 && L[1]._kernelDimensions == 2);
+        CHECK(L[1]._kernelStrideX == 2 && L[1]._kernelStrideY == 1 && !L[1]._bDimensionsProvided);
+        CHECK(L[2]._type == NNLayer::Type::Pooling && L[2]._poolingFunction == PoolingFunction::Max);
+        CHECK_EQ(nd._vWeightDescriptor.size(), (size_t)2);       // pooling layers have no weights
+        CHECK(L[3]._activation == Activation::SoftMax);
+    }
+}
+
 int main(int argc, char** argv)
 {
     if (argc > 2 && string(argv[1]) == "--dump-network") return dumpNetwork(argv[2]);
     if (argc > 2 && string(argv[1]) == "--write-cdf2") return writeCdf2(argv[2]);
     const string dir = argc > 1 ? argv[1] : "/tmp";
+    const string golden = argc > 2 ? argv[2] : "tests/golden/ldl";
     testDimensions();
     testNetworkFileRoundTrip(dir);
     testFilters(dir);
@@ -362,5 +537,7 @@ int main(int argc, char** argv)
     testKnnHost(dir);
     testLoadIndex();
     testParseSamplesAndDatasetFile(dir);
+    testJsonReader();
+    testNetworkDefinitions(dir, golden);
     return finish("test_host_cpu");
 }

@@ -19,7 +19,7 @@ def need_exe():
 
 def test_cpp_host_unit_tests(tmp_path):
     need_exe()
-    r = subprocess.run([EXE, str(tmp_path)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    r = subprocess.run([EXE, str(tmp_path), os.path.join(ROOT, "tests", "golden", "ldl")], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
     assert r.returncode == 0, r.stdout[-3000:]
     assert "0 failed" in r.stdout
 
