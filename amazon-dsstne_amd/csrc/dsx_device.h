@@ -43,6 +43,21 @@ __device__ __forceinline__ float activate_rt(float x, uint32_t act, float slope,
     }
 }
 
+// Unsigned key with the order of the scores (NaN patterns land above +inf or below -inf; callers keep NaN out).
+__device__ __forceinline__ uint32_t score_key(float key)
+{
+    key += 0.0f;   // -0.0 -> +0.0 so that both zeros tie and fall back to the column order
+    uint32_t u = __float_as_uint(key);
+    u ^= (uint32_t)((int32_t)u >> 31) | 0x80000000u;
+    return u;
+}
+
+__device__ __forceinline__ float key_score(uint32_t u)
+{
+    u ^= ((u >> 31) - 1u) | 0x80000000u;
+    return __uint_as_float(u);
+}
+
 // CalculateActivation (engine/NNLayer.cpp:1646-1683) runs a kernel only for sigmoid, tanh, ReLU, leaky ReLU, ELU, SELU and
 // softmax; every other ordinal leaves the unit buffer as it is.  Softmax is a row operation with its own kernel.
 inline bool is_elementwise_activation(uint32_t act) { return act != DSX_ACT_SOFTMAX; }

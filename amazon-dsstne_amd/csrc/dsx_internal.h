@@ -63,4 +63,10 @@ int topk_merge(const uint64_t* partial, uint32_t slots, uint32_t k, float* keys,
 int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int transposed, const float* bias, float* Z, uint32_t ldz,
            uint32_t batch, uint32_t k, uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params,
            float* seg_max = nullptr, uint32_t* seg_width = nullptr);
+// Candidate mode of the same kernel (exact KNN): scores are compared with row_bound[row] and the survivors appended to
+// cand[row][cand_cap] as packed words; nothing else is written.  knn_refresh folds a row's candidates into its best list.
+int fc_candidates_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, uint32_t batch, uint32_t k, uint32_t n,
+                      uint32_t col_offset, const uint32_t* row_bound, uint64_t* cand, uint32_t* cand_count, uint32_t cand_cap,
+                      uint32_t* overflow);
+int knn_refresh(uint64_t* best, const uint64_t* cand, uint32_t* cand_count, uint32_t cap, uint32_t k, uint32_t* row_bound, uint32_t batch);
 }  // namespace dsx

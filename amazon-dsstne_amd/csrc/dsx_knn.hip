@@ -1,9 +1,15 @@
 // dsx_knn.hip — device part of the exact KNN search: scores = queries . items^T, then the k best items per query.
 //
-// The item table is walked in column blocks: each block's scores are produced by the fp32 MFMA GEMM into a scratch
-// matrix that stays far smaller than the full [queries x items] product, the block's per-query top-k is taken straight
-// from it into packed partial lists, and one merge pass at the end combines the blocks.  A block's k-th score is a lower
-// bound of the query's final k-th score, so every later block starts with it as its admission threshold.
+// The first column block of the item table goes through the fp32 MFMA GEMM into a scratch score matrix and the scanning
+// top-K; its k-th score per query is a lower bound of the query's final k-th score.  From there on the score matrix is never
+// written: the same GEMM kernel runs in candidate mode, where a tile is only compared with the rows' bounds and the few
+// scores that reach them are appended to per-query candidate lists.  After every column range (each four times as wide as
+// everything before it, so that a range leaves about 4 k candidates per query) a small kernel folds the candidates into
+// the query's best list and raises its bound.  Results are exact for any input: a list that fills up (items sorted by
+// score, say) raises a flag that the host reads at the end, and the search is then redone block by block — GEMM into the
+// scratch matrix, scanning top-K into packed partial lists with the running bound, one merge — which is also the path
+// taken while the stream is being captured into a graph (no host read-back there) and for operands that are not 16-byte
+// aligned.
 #include <algorithm>
 #include <hip/hip_runtime.h>
 #include "dsx_internal.h"
@@ -13,10 +19,14 @@ namespace dsx {
 static void* g_knn_ws = nullptr;
 static size_t g_knn_ws_bytes = 0;
 
+static uint32_t g_knn_block_columns = 0;   // 0: sized by the rule below
+static int g_knn_last_path = 0;            // how the last search ran: DSX_KNN_PATH_*
+
 static uint32_t knn_block_columns(uint32_t rows_padded, uint32_t num_queries)
 {
     // about 1 GiB of scores per block, a multiple of 1024 columns
     uint64_t cols = ((uint64_t)1 << 30) / ((uint64_t)std::max(1u, num_queries) * sizeof(float));
+    if (g_knn_block_columns) cols = g_knn_block_columns;
     cols = std::max<uint64_t>(1024, cols / 1024 * 1024);
     cols = std::min<uint64_t>(cols, ((uint64_t)rows_padded + 1023) / 1024 * 1024);
     return (uint32_t)cols;
@@ -31,19 +41,143 @@ __global__ __launch_bounds__(256) void knn_clear_kernel(uint32_t* p, uint32_t n)
     if (i < n) p[i] = 0;
 }
 
+constexpr uint32_t kCandCap = 4096;   // candidate words per query and column range
+
+struct KnnWorkspace {
+    float* block_scores;
+    uint64_t* partial;      // block path: [queries][blocks][k]; candidate path: [queries][k], the best lists
+    uint32_t* row_bound;    // [queries] key of a score that k items seen so far reach; later columns admit nothing below it
+    uint32_t* cand_count;   // [queries]
+    uint32_t* overflow;     // [1] (+ padding)
+    uint64_t* cand;         // [queries][kCandCap]
+    size_t bytes;
+};
+
+static KnnWorkspace knn_layout(void* base, uint32_t rows_padded, uint32_t num_queries, uint32_t k)
+{
+    const uint32_t cb = knn_block_columns(rows_padded, num_queries);
+    const uint32_t blocks = (rows_padded + cb - 1) / cb;
+    KnnWorkspace w;
+    char* p = (char*)base;
+    w.block_scores = (float*)p;
+    p += align256((size_t)num_queries * cb * sizeof(float));
+    w.partial = (uint64_t*)p;
+    p += align256((size_t)num_queries * blocks * k * sizeof(uint64_t));
+    w.row_bound = (uint32_t*)p;             // row_bound, cand_count and overflow are cleared together
+    w.cand_count = w.row_bound + num_queries;
+    w.overflow = w.cand_count + num_queries;
+    p += align256(((size_t)2 * num_queries + 64) * sizeof(uint32_t));
+    w.cand = (uint64_t*)p;
+    p += align256((size_t)num_queries * kCandCap * sizeof(uint64_t));
+    w.bytes = (size_t)(p - (char*)base);
+    return w;
+}
+
+struct KnnTimer {
+    hipEvent_t ev[2] = {nullptr, nullptr};
+    bool on = false;
+    float gemm = 0.0f, topk = 0.0f;
+    void start(hipStream_t s) { if (on) hipEventRecord(ev[0], s); }
+    void stop(hipStream_t s, float& into)
+    {
+        if (!on) return;
+        hipEventRecord(ev[1], s);
+        hipEventSynchronize(ev[1]);
+        float ms = 0.0f;
+        hipEventElapsedTime(&ms, ev[0], ev[1]);
+        into += ms;
+    }
+};
+
+// Block by block through the scratch score matrix; exact for any input, usable under stream capture.
+static int knn_search_blocks(const KnnWorkspace& w, const float* items, uint32_t rows_padded, uint32_t M, uint32_t dim, const float* queries,
+                             uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, KnnTimer& t)
+{
+    hipStream_t s = ctx().stream;
+    const uint32_t cb = knn_block_columns(rows_padded, num_queries);
+    const uint32_t blocks = (M + cb - 1) / cb;
+    hipLaunchKernelGGL(knn_clear_kernel, dim3((num_queries + 255) / 256), dim3(256), 0, s, w.row_bound, num_queries);
+    for (uint32_t blk = 0; blk < blocks; blk++) {
+        const uint32_t c0 = blk * cb;
+        const uint32_t ncols = std::min(cb, M - c0);
+        t.start(s);
+        int rc = fc_run(queries, dim, items + c0, rows_padded, 0, nullptr, w.block_scores, cb, num_queries, dim, ncols, 0, DSX_ACT_LINEAR, nullptr);
+        if (rc) return rc;
+        t.stop(s, t.gemm);
+        t.start(s);
+        rc = topk_run(w.block_scores, cb, ncols, num_queries, k, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr, c0,
+                      w.partial, blocks, blk, 1, w.row_bound);
+        if (rc) return rc;
+        t.stop(s, t.topk);
+    }
+    t.start(s);
+    int rc = topk_merge(w.partial, blocks, k, scores, indexes, num_queries);
+    t.stop(s, t.topk);
+    return rc;
+}
+
+// First block as above, the rest in candidate mode.  *overflowed tells the caller to redo the search block by block.
+static int knn_search_candidates(const KnnWorkspace& w, const float* items, uint32_t rows_padded, uint32_t M, uint32_t dim,
+                                 const float* queries, uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, KnnTimer& t,
+                                 bool* overflowed)
+{
+    hipStream_t s = ctx().stream;
+    const uint32_t cb = knn_block_columns(rows_padded, num_queries);
+    const uint32_t clear_words = 2 * num_queries + 64;
+    hipLaunchKernelGGL(knn_clear_kernel, dim3((clear_words + 255) / 256), dim3(256), 0, s, w.row_bound, clear_words);
+    uint32_t done = std::min(cb, M);
+    t.start(s);
+    int rc = fc_run(queries, dim, items, rows_padded, 0, nullptr, w.block_scores, cb, num_queries, dim, done, 0, DSX_ACT_LINEAR, nullptr);
+    if (rc) return rc;
+    t.stop(s, t.gemm);
+    t.start(s);
+    rc = topk_run(w.block_scores, cb, done, num_queries, k, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr, 0, w.partial, 1, 0,
+                  1, w.row_bound);
+    if (rc) return rc;
+    t.stop(s, t.topk);
+    while (done < M) {
+        // a multiple of the tile width keeps every range's first column 16-byte aligned
+        const uint32_t ncols = (uint32_t)std::min<uint64_t>((uint64_t)M - done, (uint64_t)done * 4 / 128 * 128);
+        t.start(s);
+        rc = fc_candidates_run(queries, dim, items + done, rows_padded, num_queries, dim, ncols, done, w.row_bound, w.cand, w.cand_count,
+                               kCandCap, w.overflow);
+        if (rc) return rc;
+        t.stop(s, t.gemm);
+        t.start(s);
+        rc = knn_refresh(w.partial, w.cand, w.cand_count, kCandCap, k, w.row_bound, num_queries);
+        if (rc) return rc;
+        t.stop(s, t.topk);
+        done += ncols;
+    }
+    t.start(s);
+    rc = topk_merge(w.partial, 1, k, scores, indexes, num_queries);
+    if (rc) return rc;
+    t.stop(s, t.topk);
+    uint32_t flag = 0;
+    DSX_HIP(hipMemcpyAsync(&flag, w.overflow, sizeof(flag), hipMemcpyDeviceToHost, s));
+    DSX_HIP(hipStreamSynchronize(s));
+    *overflowed = flag != 0;
+    return DSX_OK;
+}
+
 }  // namespace dsx
 
 using namespace dsx;
 
 extern "C" {
 
+int dsx_knn_set_block_columns(uint32_t columns)
+{
+    g_knn_block_columns = columns;
+    return DSX_OK;
+}
+
+int dsx_knn_last_search_path(void) { return g_knn_last_path; }
+
 size_t dsx_knn_workspace_bytes(uint32_t rows_padded, uint32_t dim, uint32_t num_queries, uint32_t k)
 {
     (void)dim;
-    const uint32_t cb = knn_block_columns(rows_padded, num_queries);
-    const uint32_t blocks = (rows_padded + cb - 1) / cb;
-    return align256((size_t)num_queries * cb * sizeof(float)) + align256((size_t)num_queries * blocks * k * sizeof(uint64_t)) +
-           align256((size_t)num_queries * sizeof(uint32_t));
+    return knn_layout(nullptr, rows_padded, num_queries, k).bytes;
 }
 
 int dsx_knn_search(const float* items, uint32_t rows_padded, uint32_t padding, uint32_t dim, const float* queries,
@@ -59,6 +193,7 @@ int dsx_knn_search(const float* items, uint32_t rows_padded, uint32_t padding, u
     const size_t need = dsx_knn_workspace_bytes(rows_padded, dim, num_queries, k);
     if (workspace) {
         DSX_CHECK_ARG(workspace_bytes >= need, "dsx_knn_search: workspace of %zu bytes, %zu needed", workspace_bytes, need);
+        DSX_CHECK_ARG(((uintptr_t)workspace % 256) == 0, "dsx_knn_search: workspace is not 256-byte aligned");
     } else {
         if (g_knn_ws_bytes < need) {
             if (g_knn_ws) {
@@ -73,57 +208,27 @@ int dsx_knn_search(const float* items, uint32_t rows_padded, uint32_t padding, u
         }
         workspace = g_knn_ws;
     }
+    const KnnWorkspace w = knn_layout(workspace, rows_padded, num_queries, k);
     const uint32_t M = rows_padded - padding;
-    const uint32_t cb = knn_block_columns(rows_padded, num_queries);
-    const uint32_t blocks_alloc = (rows_padded + cb - 1) / cb;
-    const uint32_t blocks = (M + cb - 1) / cb;
-    float* block_scores = (float*)workspace;
-    uint64_t* partial = (uint64_t*)((char*)workspace + align256((size_t)num_queries * cb * sizeof(float)));
-    // per query: key of a score that k items of the blocks done so far reach; later blocks admit nothing below it
-    uint32_t* row_bound = (uint32_t*)((char*)partial + align256((size_t)num_queries * blocks_alloc * k * sizeof(uint64_t)));
-    hipLaunchKernelGGL(knn_clear_kernel, dim3((num_queries + 255) / 256), dim3(256), 0, ctx().stream, row_bound, num_queries);
-
     hipStream_t s = ctx().stream;
-    hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
-    float t_gemm = 0.0f, t_topk = 0.0f;
-    if (elapsed_ms)
-        for (auto& e : ev) DSX_HIP(hipEventCreate(&e));
-    int rc = DSX_OK;
-    for (uint32_t blk = 0; blk < blocks && rc == DSX_OK; blk++) {
-        const uint32_t c0 = blk * cb;
-        const uint32_t ncols = std::min(cb, M - c0);
-        if (elapsed_ms) hipEventRecord(ev[0], s);
-        rc = fc_run(queries, dim, items + c0, rows_padded, 0, nullptr, block_scores, cb, num_queries, dim, ncols, 0, DSX_ACT_LINEAR, nullptr);
-        if (rc) break;
-        if (elapsed_ms) hipEventRecord(ev[1], s);
-        rc = topk_run(block_scores, cb, ncols, num_queries, k, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr, c0, partial,
-                      blocks, blk, 1, row_bound);
-        if (rc) break;
-        if (elapsed_ms) {
-            hipEventRecord(ev[2], s);
-            hipEventSynchronize(ev[2]);
-            float a = 0, b = 0;
-            hipEventElapsedTime(&a, ev[0], ev[1]);
-            hipEventElapsedTime(&b, ev[1], ev[2]);
-            t_gemm += a;
-            t_topk += b;
-        }
-    }
-    if (rc == DSX_OK) {
-        if (elapsed_ms) hipEventRecord(ev[0], s);
-        rc = topk_merge(partial, blocks, k, scores, indexes, num_queries);
-        if (elapsed_ms && rc == DSX_OK) {
-            hipEventRecord(ev[1], s);
-            hipEventSynchronize(ev[1]);
-            float a = 0;
-            hipEventElapsedTime(&a, ev[0], ev[1]);
-            t_topk += a;
-        }
-    }
+    KnnTimer t;
     if (elapsed_ms) {
-        for (auto& e : ev) hipEventDestroy(e);
-        elapsed_ms[0] = t_gemm;
-        elapsed_ms[1] = t_topk;
+        t.on = true;
+        for (auto& e : t.ev) DSX_HIP(hipEventCreate(&e));
+    }
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    hipStreamIsCapturing(s, &capturing);
+    const bool aligned = ((uintptr_t)items % 16) == 0 && ((uintptr_t)queries % 16) == 0 && (rows_padded % 4) == 0 && (dim % 4) == 0;
+    const bool candidates = aligned && capturing == hipStreamCaptureStatusNone && M > knn_block_columns(rows_padded, num_queries);
+    int rc = DSX_OK;
+    bool redo = !candidates;
+    if (candidates) rc = knn_search_candidates(w, items, rows_padded, M, dim, queries, num_queries, k, scores, indexes, t, &redo);
+    g_knn_last_path = !candidates ? DSX_KNN_PATH_BLOCKS : (redo ? DSX_KNN_PATH_CANDIDATES_REDONE : DSX_KNN_PATH_CANDIDATES);
+    if (rc == DSX_OK && redo) rc = knn_search_blocks(w, items, rows_padded, M, dim, queries, num_queries, k, scores, indexes, t);
+    if (elapsed_ms) {
+        for (auto& e : t.ev) hipEventDestroy(e);
+        elapsed_ms[0] = t.gemm;
+        elapsed_ms[1] = t.topk;
     }
     return rc;
 }

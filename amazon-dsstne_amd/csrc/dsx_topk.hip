@@ -28,21 +28,6 @@ constexpr int kTopkThreads = 256;
 constexpr int kTopkWaves = kTopkThreads / kWave;
 constexpr uint32_t kMaxBitmapBits = 256 * 1024;   // 32 KiB of LDS per workgroup
 
-// Unsigned key with the order of the scores (NaN patterns land above +inf or below -inf; callers keep NaN out).
-__device__ __forceinline__ uint32_t score_key(float key)
-{
-    key += 0.0f;   // -0.0 -> +0.0 so that both zeros tie and fall back to the column order
-    uint32_t u = __float_as_uint(key);
-    u ^= (uint32_t)((int32_t)u >> 31) | 0x80000000u;
-    return u;
-}
-
-__device__ __forceinline__ float key_score(uint32_t u)
-{
-    u ^= ((u >> 31) - 1u) | 0x80000000u;
-    return __uint_as_float(u);
-}
-
 __device__ __forceinline__ uint64_t pack_score(float key, uint32_t col)
 {
     return ((uint64_t)score_key(key) << 32) | (uint32_t)~col;
@@ -1023,6 +1008,55 @@ int topk_merge(const uint64_t* partial, uint32_t slots, uint32_t k, float* keys,
     if (k <= 64) return launch_merge<1>(partial, slots, k, keys, values, batch);
     if (k <= 128) return launch_merge<2>(partial, slots, k, keys, values, batch);
     return launch_merge<4>(partial, slots, k, keys, values, batch);
+}
+
+// Exact KNN with candidate lists: merges a row's running best list (k packed words, best first) with the candidates the last
+// column range left behind, writes the best k back, raises the row's bound to their k-th key and empties the candidate
+// list.  One wavefront per row.
+template <int R>
+__global__ __launch_bounds__(kWave) void knn_refresh_kernel(uint64_t* best, const uint64_t* cand, uint32_t* cand_count, uint32_t cap,
+                                                            uint32_t k, uint32_t* row_bound)
+{
+    using List = WaveTopK<R>;
+    __shared__ uint64_t sStage[List::kStageWords];
+    const uint32_t b = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    List list;
+    list.init(sStage, lane, k);
+    uint64_t* mine = best + (uint64_t)b * k;
+    for (uint32_t p0 = 0; p0 < k; p0 += kWave) {
+        const uint32_t p = p0 + lane;
+        const uint64_t word = (p < k) ? mine[p] : 0ull;
+        list.offer(word != 0, word);
+    }
+    const uint32_t n = min(cand_count[b], cap);
+    const uint64_t* src = cand + (uint64_t)b * cap;
+    for (uint32_t p0 = 0; p0 < n; p0 += kWave) {
+        const uint32_t p = p0 + lane;
+        const uint64_t word = (p < n) ? src[p] : 0ull;
+        list.offer(word != 0, word);
+    }
+    list.finish();
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const uint32_t p = r * kWave + lane;
+        if (p < k) mine[p] = list.q[r];
+        if (p == k - 1 && list.q[r] != 0) row_bound[b] = max(row_bound[b], (uint32_t)(list.q[r] >> 32));
+    }
+    if (lane == 0) cand_count[b] = 0;
+}
+
+int knn_refresh(uint64_t* best, const uint64_t* cand, uint32_t* cand_count, uint32_t cap, uint32_t k, uint32_t* row_bound, uint32_t batch)
+{
+    hipStream_t s = ctx().stream;
+    if (k <= 64)
+        hipLaunchKernelGGL((knn_refresh_kernel<1>), dim3(batch), dim3(kWave), 0, s, best, cand, cand_count, cap, k, row_bound);
+    else if (k <= 128)
+        hipLaunchKernelGGL((knn_refresh_kernel<2>), dim3(batch), dim3(kWave), 0, s, best, cand, cand_count, cap, k, row_bound);
+    else
+        hipLaunchKernelGGL((knn_refresh_kernel<4>), dim3(batch), dim3(kWave), 0, s, best, cand, cand_count, cap, k, row_bound);
+    DSX_LAUNCH_CHECK("knn_refresh_kernel");
+    return DSX_OK;
 }
 
 // Guided top-K when it applies (k <= 64, 64-column segments, at most kGuidedMaxSegs of them), the scan otherwise.

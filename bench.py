@@ -250,7 +250,8 @@ def knn_bench(args, pkg, lib):
     flops = 2.0 * Q * D * (rows - pad)
     roofline = {"kernel": "fc_gemm_kernel (knn scores)", "bound": "mfma", "achieved": round(flops / el[0] / 1e9, 3), "peak": FP32_MFMA_PEAK_TF,
                 "unit": "TFLOP/s", "frac": round(flops / el[0] / 1e9 / FP32_MFMA_PEAK_TF, 4), "traffic": None, "avg_launch_ms": round(el[0], 4),
-                "topk_ms": round(el[1], 4)}
+                "topk_ms": round(el[1], 4),
+                "path": {0: "blocks", 1: "candidate lists", 2: "candidate lists, redone block by block"}[lib.dsx_knn_last_search_path()]}
     cpu = None
     if args.cpu_seconds > 0:
         orc = entry.load_oracle()

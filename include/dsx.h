@@ -221,13 +221,24 @@ int dsx_topk_guided(const float* in, float* keys, uint32_t* values, uint32_t bat
 /* Device part of KnnExactGpu::search (knn/KnnExactGpu.cu:99-148): scores = queries . items^T (cublasSgemmEx) followed by
  * the padded top-K.  items is column-major [rows_padded x dim] as KnnData::load builds it (knn/KnnData.cpp:197-207),
  * i.e. items[d * rows_padded + m]; queries is row-major [num_queries x dim]; the score matrix is produced in column
- * blocks inside the call and never stored whole.  workspace (device, workspace_bytes) may be NULL: the library then
+ * blocks inside the call and never stored whole: the first block goes through a scratch matrix and the scanning top-K,
+ * later column ranges only append the scores that reach a query's running k-th score to candidate lists (exact; if a list
+ * fills up the call notices at its end and repeats the search block by block).  The call returns when the results are
+ * complete on the device.  workspace (device, 256-byte aligned, workspace_bytes) may be NULL: the library then
  * allocates what it needs for the call.  elapsed_ms (optional, 2 floats) receives the GEMM and top-K times like
  * KnnData::elapsedSgemm / elapsedTopK. */
 int dsx_knn_search(const float* items, uint32_t rows_padded, uint32_t padding, uint32_t dim, const float* queries,
                    uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, void* workspace, size_t workspace_bytes,
                    float* elapsed_ms);
 size_t dsx_knn_workspace_bytes(uint32_t rows_padded, uint32_t dim, uint32_t num_queries, uint32_t k);
+/* No counterpart in the reference: width of the first column block (rounded down to a multiple of 1024, at least 1024;
+ * 0 restores the default of about 1 GiB of scores).  Workspace sizes depend on it: set it before asking for them. */
+int dsx_knn_set_block_columns(uint32_t columns);
+/* No counterpart in the reference: how the last dsx_knn_search of this process ran. */
+#define DSX_KNN_PATH_BLOCKS 0             /* every column block through the scratch score matrix and the scanning top-K */
+#define DSX_KNN_PATH_CANDIDATES 1         /* first block as above, then candidate lists */
+#define DSX_KNN_PATH_CANDIDATES_REDONE 2  /* a candidate list filled up: repeated block by block */
+int dsx_knn_last_search_path(void);
 
 #ifdef __cplusplus
 }

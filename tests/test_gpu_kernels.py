@@ -540,3 +540,98 @@ def test_knn_search(pkg, dsx, orc, synth, items, queries, dim, k):
         assert np.abs(full[r, got_i[r, c]] - full[r, ref_i[r, c]]).max() < 1e-5
     assert_close(got_s, np.take_along_axis(full, got_i.astype(np.int64), axis=1), "knn scores", rel=1e-4, abs_floor=0.05)
     assert el[0] > 0 and el[1] > 0
+
+
+def knn_case(pkg, dsx, orc, items_m, queries_m, k, pad_value=50.0):
+    """Runs dsx_knn_search on row-major items/queries and returns (scores, indexes, oracle scores, oracle indexes, times)."""
+    items, dim = items_m.shape
+    queries = queries_m.shape[0]
+    rows = (items + 7) // 8 * 8
+    pad = rows - items
+    cm = np.full((dim, rows), pad_value, dtype=np.float32)
+    cm[:, :items] = items_m.T
+    dI, dQ = dev(pkg, cm), dev(pkg, queries_m)
+    scores = pkg.DeviceArray((queries, k), np.float32)
+    idx = pkg.DeviceArray((queries, k), np.uint32)
+    el = (C.c_float * 2)()
+    pkg.check(dsx.dsx_knn_search(dI.ptr, rows, pad, dim, dQ.ptr, queries, k, scores.ptr, idx.ptr, None, 0, el))
+    ref_s, ref_i = orc.knn_search(cm, rows, pad, dim, queries_m, k)
+    return scores.numpy(), idx.numpy(), ref_s, ref_i, el
+
+
+@pytest.fixture
+def small_knn_blocks(dsx):
+    """First column block of 1,024 items, so that searches of a few ten thousand items run the candidate ranges
+    (1,024 scanned, then 4,096, 20,480, ... compared with the queries' bounds)."""
+    dsx.dsx_knn_set_block_columns(1024)
+    yield
+    dsx.dsx_knn_set_block_columns(0)
+
+
+@pytest.mark.parametrize("items,queries,dim,k", [(30011, 70, 64, 100), (9000, 130, 256, 10), (26000, 33, 32, 200), (1500, 5, 16, 64)])
+def test_knn_search_candidate_ranges(pkg, dsx, orc, synth, small_knn_blocks, items, queries, dim, k):
+    say("knn candidate ranges items=%d queries=%d dim=%d k=%d" % (items, queries, dim, k))
+    p = synth.knn_config(seed=5, items=items, queries=queries, dim=dim, k=k)
+    got_s, got_i, ref_s, ref_i, _ = knn_case(pkg, dsx, orc, p.items, p.queries, k)
+    assert dsx.dsx_knn_last_search_path() == 1       # candidate lists, none of them full
+    full = p.queries.astype(np.float64) @ p.items.astype(np.float64).T
+    assert got_i.max() < items
+    mism = got_i != ref_i
+    if mism.any():
+        r, c = np.nonzero(mism)
+        assert np.abs(full[r, got_i[r, c]] - full[r, ref_i[r, c]]).max() < 1e-5
+    assert_close(got_s, np.take_along_axis(full, got_i.astype(np.int64), axis=1), "knn scores", rel=1e-4, abs_floor=0.05)
+    assert (np.diff(got_s, axis=1) <= 0).all()
+
+
+def test_knn_search_candidate_ranges_exact_ties(pkg, dsx, orc, rng, small_knn_blocks):
+    """Small integer vectors: every score is an exactly representable integer whatever the order of the sum, thousands of
+    items tie, and the result must be the oracle's bit for bit (score descending, then the lower item number)."""
+    items, queries, dim, k = 21000, 40, 16, 100
+    it = rng.integers(-2, 3, size=(items, dim)).astype(np.float32)
+    q = rng.integers(-2, 3, size=(queries, dim)).astype(np.float32)
+    got_s, got_i, ref_s, ref_i, _ = knn_case(pkg, dsx, orc, it, q, k)
+    assert dsx.dsx_knn_last_search_path() == 1
+    assert np.array_equal(got_s, ref_s)
+    assert np.array_equal(got_i, ref_i)
+    q[3] = 0.0                                       # every item ties at 0 for this query: its candidate list fills up
+    got_s, got_i, ref_s, ref_i, _ = knn_case(pkg, dsx, orc, it, q, k)
+    assert dsx.dsx_knn_last_search_path() == 2
+    assert np.array_equal(got_s, ref_s)
+    assert np.array_equal(got_i, ref_i)
+    assert np.array_equal(got_i[3], np.arange(k, dtype=np.uint32))
+
+
+def test_knn_search_full_candidate_list_falls_back(pkg, dsx, orc, rng, small_knn_blocks):
+    """Items sorted by rising score for some queries: every later item beats the bound, the candidate lists (4,096 words per
+    query and range) fill up, and the search is redone block by block.  The result is exact all the same."""
+    items, queries, dim, k = 40000, 12, 8, 50
+    direction = rng.standard_normal(dim).astype(np.float32)
+    direction /= np.linalg.norm(direction)
+    scale = np.linspace(0.001, 1.0, items, dtype=np.float32)
+    it = (scale[:, None] * direction[None, :]).astype(np.float32)
+    it += (rng.standard_normal((items, dim)) * 1e-4).astype(np.float32)
+    q = rng.standard_normal((queries, dim)).astype(np.float32)
+    q[0] = direction                                 # scores rise with the item number
+    q[1] = -direction                                # and fall: the first block already holds the answer
+    got_s, got_i, ref_s, ref_i, _ = knn_case(pkg, dsx, orc, it, q, k)
+    assert dsx.dsx_knn_last_search_path() == 2
+    full = q.astype(np.float64) @ it.astype(np.float64).T
+    mism = got_i != ref_i
+    if mism.any():
+        r, c = np.nonzero(mism)
+        assert np.abs(full[r, got_i[r, c]] - full[r, ref_i[r, c]]).max() < 1e-5
+    assert_close(got_s, np.take_along_axis(full, got_i.astype(np.int64), axis=1), "knn scores", rel=1e-4, abs_floor=0.05)
+    assert got_i[0].min() >= items - 2 * k and got_i[1].max() < 2 * k
+
+
+def test_knn_search_unaligned_dim_takes_block_path(pkg, dsx, orc, synth, small_knn_blocks):
+    p = synth.knn_config(seed=9, items=5000, queries=17, dim=30, k=20)      # 30 floats per row: no 128-bit loads
+    got_s, got_i, ref_s, ref_i, _ = knn_case(pkg, dsx, orc, p.items, p.queries, 20)
+    assert dsx.dsx_knn_last_search_path() == 0
+    full = p.queries.astype(np.float64) @ p.items.astype(np.float64).T
+    mism = got_i != ref_i
+    if mism.any():
+        r, c = np.nonzero(mism)
+        assert np.abs(full[r, got_i[r, c]] - full[r, ref_i[r, c]]).max() < 1e-5
+    assert_close(got_s, np.take_along_axis(full, got_i.astype(np.int64), axis=1), "knn scores", rel=1e-4, abs_floor=0.05)
