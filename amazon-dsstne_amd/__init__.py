@@ -81,10 +81,14 @@ SIGNATURES = {
     "dsx_topk_guided": [_vp, _vp, _vp, _u32, _u32, _u32, _vp, _u32, _u32, _vp, _vp, _vp, _vp, _vp],
     "dsx_knn_search": [_vp, _u32, _u32, _u32, _vp, _u32, _u32, _vp, _vp, _vp, _sz, C.POINTER(_f32)],
     "dsx_knn_set_block_columns": [_u32],
+    "dsx_knn_f16_convert_items": [_vp, _u32, _u32, _u32, _vp],
+    "dsx_knn_search_f16": [_vp, _u32, _u32, _u32, _vp, _u32, _u32, _vp, _vp, _vp, _sz, C.POINTER(_f32)],
     "dsx_knn_last_search_path": [],
 }
-SPECIAL_RESTYPES = {"dsx_last_error": C.c_char_p, "dsx_stream": C.c_void_p, "dsx_knn_workspace_bytes": C.c_size_t}
-SPECIAL_ARGTYPES = {"dsx_last_error": [], "dsx_stream": [], "dsx_knn_workspace_bytes": [_u32, _u32, _u32, _u32]}
+SPECIAL_RESTYPES = {"dsx_last_error": C.c_char_p, "dsx_stream": C.c_void_p, "dsx_knn_workspace_bytes": C.c_size_t,
+                    "dsx_knn_workspace_bytes_f16": C.c_size_t, "dsx_knn_f16_table_bytes": C.c_size_t}
+SPECIAL_ARGTYPES = {"dsx_last_error": [], "dsx_stream": [], "dsx_knn_workspace_bytes": [_u32, _u32, _u32, _u32],
+                    "dsx_knn_workspace_bytes_f16": [_u32, _u32, _u32, _u32], "dsx_knn_f16_table_bytes": [_u32, _u32]}
 
 _lib = None
 

@@ -11,8 +11,6 @@
 
 namespace dsx {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-
 constexpr int kFcThreads = 256;
 constexpr int kXcds = 8;
 
@@ -30,15 +28,7 @@ struct FcArgs {
     float* seg_max;      // optional: [batch][nseg] maxima of the activated outputs over 64-column segments
     uint32_t nseg;
     float slope, alpha, lambda;
-    // Candidate mode (exact nearest-neighbour search): Z is not written.  A score whose key reaches row_bound[row] is appended
-    // as a packed word (key << 32 | ~(col_offset + column)) to the row's list cand[row][cand_cap]; cand_count[row] counts the
-    // appends, and *overflow is set when a list is full.
-    const uint32_t* row_bound;
-    uint64_t* cand;
-    uint32_t* cand_count;
-    uint32_t cand_cap;
-    uint32_t col_offset;
-    uint32_t* overflow;
+    CandArgs cand;       // candidate mode (template flag CAND): Z is not written, see candidate_epilogue
 };
 
 // MI, NI: 32x32 MFMA blocks per wavefront in M and N.  XV / WV: vector width (floats) of the global loads of X / W.
@@ -307,57 +297,10 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
         }
     }
 
-    // Candidate mode: the tile is only compared with the rows' admission bounds.  A bound is the key of a score that k items
-    // seen earlier reach, so almost every tile ends after MI * NI * 16 compares per lane; the few survivors are appended to
-    // their rows' lists with one atomic each.  The bounds of the tile's rows are staged in LDS as floats (the operand tiles
-    // are dead by now), four consecutive rows per 128-bit read; a NaN score fails "x < bound" and is sorted out by its key.
     if constexpr (CAND) {
-        float* sBound = &sA[0][0][0];
         static_assert(sizeof(sA) >= BM * sizeof(float), "the bounds reuse the X tile's LDS");
-        if (tid < BM) {
-            const uint32_t r = row0 + tid;
-            sBound[tid] = (r < a.batch) ? key_score(a.row_bound[r]) : __builtin_inff();
-        }
-        __syncthreads();
-        float bf[MI][4][4];
-        bool any = false;
-#pragma unroll
-        for (int i = 0; i < MI; i++)
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const float4 t = *reinterpret_cast<const float4*>(&sBound[wm * 32 * MI + i * 32 + 8 * g + 4 * lhi]);
-                bf[i][g][0] = t.x; bf[i][g][1] = t.y; bf[i][g][2] = t.z; bf[i][g][3] = t.w;
-            }
-#pragma unroll
-        for (int i = 0; i < MI; i++)
-#pragma unroll
-            for (int j = 0; j < NI; j++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) any |= !(acc[i][j][v] < bf[i][v / 4][v % 4]);
-        if (any) {
-#pragma unroll
-            for (int j = 0; j < NI; j++) {
-                const uint32_t c = col0 + wn * 32 * NI + j * 32 + l32;
-                if (c >= a.n) continue;
-#pragma unroll
-                for (int i = 0; i < MI; i++) {
-#pragma unroll
-                    for (int v = 0; v < 16; v++) {
-                        const float x = acc[i][j][v];
-                        if (x < bf[i][v / 4][v % 4]) continue;
-                        const uint32_t r = row0 + wm * 32 * MI + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
-                        if (r >= a.batch) continue;
-                        const uint32_t key = score_key(x);
-                        if (key < a.row_bound[r]) continue;
-                        const uint32_t pos = atomicAdd(&a.cand_count[r], 1u);
-                        if (pos < a.cand_cap)
-                            a.cand[(uint64_t)r * a.cand_cap + pos] = ((uint64_t)key << 32) | (uint32_t)~(a.col_offset + c);
-                        else
-                            *a.overflow = 1u;
-                    }
-                }
-            }
-        }
+        // (the k-loop ended with a barrier: every wavefront is done with sA)
+        candidate_epilogue<MI, NI>(acc, &sA[0][0][0], a.cand, row0, col0, a.batch, a.n, tid, wm, wn, l32, lhi);
         return;
     }
 
@@ -586,8 +529,7 @@ int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int trans
 // Scores of queries[batch][k] against n columns of W, compared with the rows' bounds instead of stored (FcArgs, candidate
 // mode).  The caller guarantees 16-byte aligned operands with pitches that are multiples of four floats.
 int fc_candidates_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, uint32_t batch, uint32_t k, uint32_t n,
-                      uint32_t col_offset, const uint32_t* row_bound, uint64_t* cand, uint32_t* cand_count, uint32_t cand_cap,
-                      uint32_t* overflow)
+                      const CandArgs& cand)
 {
     FcArgs a{};
     a.X = X; a.W = W;
@@ -595,12 +537,7 @@ int fc_candidates_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw
     a.batch = batch; a.k = k; a.n = n;
     a.act = DSX_ACT_LINEAR;
     a.fast32 = ((uint64_t)(batch + 128) * ldx * 4 < (1ull << 32)) && ((32ull * ldw + n + 128) * 4 < (1ull << 32));
-    a.row_bound = row_bound;
     a.cand = cand;
-    a.cand_count = cand_count;
-    a.cand_cap = cand_cap;
-    a.col_offset = col_offset;
-    a.overflow = overflow;
     a.tiles_m = (batch + 127) / 128;
     a.tiles_n = (n + 127) / 128;
     const uint32_t total = a.tiles_m * a.tiles_n;

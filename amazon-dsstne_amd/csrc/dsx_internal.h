@@ -63,10 +63,18 @@ int topk_merge(const uint64_t* partial, uint32_t slots, uint32_t k, float* keys,
 int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int transposed, const float* bias, float* Z, uint32_t ldz,
            uint32_t batch, uint32_t k, uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params,
            float* seg_max = nullptr, uint32_t* seg_width = nullptr);
-// Candidate mode of the same kernel (exact KNN): scores are compared with row_bound[row] and the survivors appended to
-// cand[row][cand_cap] as packed words; nothing else is written.  knn_refresh folds a row's candidates into its best list.
+// Candidate mode of the same kernel (exact KNN): scores are compared with the rows' bounds and the survivors appended to
+// per-row lists as packed words (CandArgs); nothing else is written.  knn_refresh folds a row's candidates into its best
+// list.  The caller guarantees 16-byte aligned operands with pitches that are multiples of four floats.
+struct CandArgs;
 int fc_candidates_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, uint32_t batch, uint32_t k, uint32_t n,
-                      uint32_t col_offset, const uint32_t* row_bound, uint64_t* cand, uint32_t* cand_count, uint32_t cand_cap,
-                      uint32_t* overflow);
+                      const CandArgs& cand);
+// fp16 storage of the KNN operands (dsx_knn_f16.hip): padded row-major layout, conversion, and the score kernel in store mode
+// (cand == NULL: Z[batch][ldz]) or candidate mode.
+uint32_t knn_f16_ld(uint32_t dim);
+uint64_t knn_f16_rows(uint64_t rows);
+int knn_to_f16(const float* src, bool colmajor, uint64_t src_ld, uint32_t rows_valid, uint32_t dim, void* dst, uint32_t rows_out);
+int knn_f16_scores_run(const void* queries16, const void* items16, uint32_t ld, uint32_t batch, uint32_t n, float* Z, uint32_t ldz,
+                       const CandArgs* cand);
 int knn_refresh(uint64_t* best, const uint64_t* cand, uint32_t* cand_count, uint32_t cap, uint32_t k, uint32_t* row_bound, uint32_t batch);
 }  // namespace dsx

@@ -9,9 +9,11 @@
 // score, say) raises a flag that the host reads at the end, and the search is then redone block by block — GEMM into the
 // scratch matrix, scanning top-K into packed partial lists with the running bound, one merge — which is also the path
 // taken while the stream is being captured into a graph (no host read-back there) and for operands that are not 16-byte
-// aligned.
+// aligned.  With fp16 storage (dsx_knn_search_f16) the scores come from the f16 MFMA kernel of dsx_knn_f16.hip instead, through
+// the same three steps.
 #include <algorithm>
 #include <hip/hip_runtime.h>
+#include "dsx_device.h"
 #include "dsx_internal.h"
 
 namespace dsx {
@@ -50,10 +52,11 @@ struct KnnWorkspace {
     uint32_t* cand_count;   // [queries]
     uint32_t* overflow;     // [1] (+ padding)
     uint64_t* cand;         // [queries][kCandCap]
+    void* queries16;        // fp16 storage only: the query batch, [queries rounded up to 128][ld] halves
     size_t bytes;
 };
 
-static KnnWorkspace knn_layout(void* base, uint32_t rows_padded, uint32_t num_queries, uint32_t k)
+static KnnWorkspace knn_layout(void* base, uint32_t rows_padded, uint32_t num_queries, uint32_t k, bool f16 = false, uint32_t dim = 0)
 {
     const uint32_t cb = knn_block_columns(rows_padded, num_queries);
     const uint32_t blocks = (rows_padded + cb - 1) / cb;
@@ -69,9 +72,32 @@ static KnnWorkspace knn_layout(void* base, uint32_t rows_padded, uint32_t num_qu
     p += align256(((size_t)2 * num_queries + 64) * sizeof(uint32_t));
     w.cand = (uint64_t*)p;
     p += align256((size_t)num_queries * kCandCap * sizeof(uint64_t));
+    w.queries16 = p;
+    if (f16) p += align256((size_t)knn_f16_rows(num_queries) * knn_f16_ld(dim) * 2);
     w.bytes = (size_t)(p - (char*)base);
     return w;
 }
+
+// Where the scores of a column range come from: the fp32 table through fc_gemm_kernel, or the fp16 table through knn_f16_kernel.
+struct KnnOperands {
+    bool f16 = false;
+    const float* items = nullptr;       // fp32: column-major [dim][rows_padded]
+    const float* queries = nullptr;     // fp32: [queries][dim]
+    const char* items16 = nullptr;      // fp16: [rows rounded up to 128][ld]
+    const void* queries16 = nullptr;
+    uint32_t rows_padded = 0, dim = 0, ld16 = 0;
+
+    int into_matrix(uint32_t c0, uint32_t ncols, uint32_t num_queries, float* Z, uint32_t ldz) const
+    {
+        if (f16) return knn_f16_scores_run(queries16, items16 + (uint64_t)c0 * ld16 * 2, ld16, num_queries, ncols, Z, ldz, nullptr);
+        return fc_run(queries, dim, items + c0, rows_padded, 0, nullptr, Z, ldz, num_queries, dim, ncols, 0, DSX_ACT_LINEAR, nullptr);
+    }
+    int into_candidates(uint32_t c0, uint32_t ncols, uint32_t num_queries, const CandArgs& cand) const
+    {
+        if (f16) return knn_f16_scores_run(queries16, items16 + (uint64_t)c0 * ld16 * 2, ld16, num_queries, ncols, nullptr, 0, &cand);
+        return fc_candidates_run(queries, dim, items + c0, rows_padded, num_queries, dim, ncols, cand);
+    }
+};
 
 struct KnnTimer {
     hipEvent_t ev[2] = {nullptr, nullptr};
@@ -90,18 +116,18 @@ struct KnnTimer {
 };
 
 // Block by block through the scratch score matrix; exact for any input, usable under stream capture.
-static int knn_search_blocks(const KnnWorkspace& w, const float* items, uint32_t rows_padded, uint32_t M, uint32_t dim, const float* queries,
-                             uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, KnnTimer& t)
+static int knn_search_blocks(const KnnWorkspace& w, const KnnOperands& op, uint32_t M, uint32_t num_queries, uint32_t k, float* scores,
+                             uint32_t* indexes, KnnTimer& t)
 {
     hipStream_t s = ctx().stream;
-    const uint32_t cb = knn_block_columns(rows_padded, num_queries);
+    const uint32_t cb = knn_block_columns(op.rows_padded, num_queries);
     const uint32_t blocks = (M + cb - 1) / cb;
     hipLaunchKernelGGL(knn_clear_kernel, dim3((num_queries + 255) / 256), dim3(256), 0, s, w.row_bound, num_queries);
     for (uint32_t blk = 0; blk < blocks; blk++) {
         const uint32_t c0 = blk * cb;
         const uint32_t ncols = std::min(cb, M - c0);
         t.start(s);
-        int rc = fc_run(queries, dim, items + c0, rows_padded, 0, nullptr, w.block_scores, cb, num_queries, dim, ncols, 0, DSX_ACT_LINEAR, nullptr);
+        int rc = op.into_matrix(c0, ncols, num_queries, w.block_scores, cb);
         if (rc) return rc;
         t.stop(s, t.gemm);
         t.start(s);
@@ -117,17 +143,16 @@ static int knn_search_blocks(const KnnWorkspace& w, const float* items, uint32_t
 }
 
 // First block as above, the rest in candidate mode.  *overflowed tells the caller to redo the search block by block.
-static int knn_search_candidates(const KnnWorkspace& w, const float* items, uint32_t rows_padded, uint32_t M, uint32_t dim,
-                                 const float* queries, uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, KnnTimer& t,
-                                 bool* overflowed)
+static int knn_search_candidates(const KnnWorkspace& w, const KnnOperands& op, uint32_t M, uint32_t num_queries, uint32_t k, float* scores,
+                                 uint32_t* indexes, KnnTimer& t, bool* overflowed)
 {
     hipStream_t s = ctx().stream;
-    const uint32_t cb = knn_block_columns(rows_padded, num_queries);
+    const uint32_t cb = knn_block_columns(op.rows_padded, num_queries);
     const uint32_t clear_words = 2 * num_queries + 64;
     hipLaunchKernelGGL(knn_clear_kernel, dim3((clear_words + 255) / 256), dim3(256), 0, s, w.row_bound, clear_words);
     uint32_t done = std::min(cb, M);
     t.start(s);
-    int rc = fc_run(queries, dim, items, rows_padded, 0, nullptr, w.block_scores, cb, num_queries, dim, done, 0, DSX_ACT_LINEAR, nullptr);
+    int rc = op.into_matrix(0, done, num_queries, w.block_scores, cb);
     if (rc) return rc;
     t.stop(s, t.gemm);
     t.start(s);
@@ -139,8 +164,8 @@ static int knn_search_candidates(const KnnWorkspace& w, const float* items, uint
         // a multiple of the tile width keeps every range's first column 16-byte aligned
         const uint32_t ncols = (uint32_t)std::min<uint64_t>((uint64_t)M - done, (uint64_t)done * 4 / 128 * 128);
         t.start(s);
-        rc = fc_candidates_run(queries, dim, items + done, rows_padded, num_queries, dim, ncols, done, w.row_bound, w.cand, w.cand_count,
-                               kCandCap, w.overflow);
+        const CandArgs cand{w.row_bound, w.cand, w.cand_count, kCandCap, done, w.overflow};
+        rc = op.into_candidates(done, ncols, num_queries, cand);
         if (rc) return rc;
         t.stop(s, t.gemm);
         t.start(s);
@@ -180,17 +205,29 @@ size_t dsx_knn_workspace_bytes(uint32_t rows_padded, uint32_t dim, uint32_t num_
     return knn_layout(nullptr, rows_padded, num_queries, k).bytes;
 }
 
-int dsx_knn_search(const float* items, uint32_t rows_padded, uint32_t padding, uint32_t dim, const float* queries,
-                   uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, void* workspace, size_t workspace_bytes,
-                   float* elapsed_ms)
+size_t dsx_knn_workspace_bytes_f16(uint32_t rows_padded, uint32_t dim, uint32_t num_queries, uint32_t k)
+{
+    return knn_layout(nullptr, rows_padded, num_queries, k, true, dim).bytes;
+}
+
+size_t dsx_knn_f16_table_bytes(uint32_t rows_padded, uint32_t dim) { return (size_t)knn_f16_rows(rows_padded) * knn_f16_ld(dim) * 2; }
+
+int dsx_knn_f16_convert_items(const float* items, uint32_t rows_padded, uint32_t padding, uint32_t dim, void* items_f16)
 {
     DSX_REQUIRE_INIT();
-    DSX_CHECK_ARG(items && queries && scores && indexes, "dsx_knn_search: null device pointer");
-    DSX_CHECK_ARG(padding < rows_padded, "dsx_knn_search: padding %u leaves no item of %u", padding, rows_padded);
-    DSX_CHECK_ARG(dim > 0, "dsx_knn_search: dim is 0");
-    DSX_CHECK_ARG(k >= 1 && k <= 256, "dsx_knn_search: k = %u is outside 1..256", k);
-    if (num_queries == 0) return DSX_OK;
-    const size_t need = dsx_knn_workspace_bytes(rows_padded, dim, num_queries, k);
+    DSX_CHECK_ARG(items && items_f16, "dsx_knn_f16_convert_items: null device pointer");
+    DSX_CHECK_ARG(padding < rows_padded && dim > 0, "dsx_knn_f16_convert_items: rows_padded %u, padding %u, dim %u", rows_padded, padding, dim);
+    DSX_CHECK_ARG(((uintptr_t)items_f16 % 16) == 0, "dsx_knn_f16_convert_items: the fp16 table is not 16-byte aligned");
+    return knn_to_f16(items, true, rows_padded, rows_padded - padding, dim, items_f16, (uint32_t)knn_f16_rows(rows_padded));
+}
+
+}  // extern "C"
+
+// Both precisions: workspace, the two paths, timing.
+static int knn_search_common(KnnOperands& op, uint32_t padding, uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, void* workspace,
+                             size_t workspace_bytes, float* elapsed_ms, bool aligned, const float* queries_f32)
+{
+    const size_t need = knn_layout(nullptr, op.rows_padded, num_queries, k, op.f16, op.dim).bytes;
     if (workspace) {
         DSX_CHECK_ARG(workspace_bytes >= need, "dsx_knn_search: workspace of %zu bytes, %zu needed", workspace_bytes, need);
         DSX_CHECK_ARG(((uintptr_t)workspace % 256) == 0, "dsx_knn_search: workspace is not 256-byte aligned");
@@ -208,29 +245,75 @@ int dsx_knn_search(const float* items, uint32_t rows_padded, uint32_t padding, u
         }
         workspace = g_knn_ws;
     }
-    const KnnWorkspace w = knn_layout(workspace, rows_padded, num_queries, k);
-    const uint32_t M = rows_padded - padding;
+    const KnnWorkspace w = knn_layout(workspace, op.rows_padded, num_queries, k, op.f16, op.dim);
+    const uint32_t M = op.rows_padded - padding;
     hipStream_t s = ctx().stream;
     KnnTimer t;
     if (elapsed_ms) {
         t.on = true;
         for (auto& e : t.ev) DSX_HIP(hipEventCreate(&e));
     }
+    int rc = DSX_OK;
+    if (op.f16) {   // the query batch in the table's format (knn/KnnExactGpu.cu:108-116); counted as GEMM time like the copy it replaces
+        t.start(s);
+        rc = knn_to_f16(queries_f32, false, op.dim, num_queries, op.dim, w.queries16, (uint32_t)knn_f16_rows(num_queries));
+        t.stop(s, t.gemm);
+        op.queries16 = w.queries16;
+    }
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     hipStreamIsCapturing(s, &capturing);
-    const bool aligned = ((uintptr_t)items % 16) == 0 && ((uintptr_t)queries % 16) == 0 && (rows_padded % 4) == 0 && (dim % 4) == 0;
-    const bool candidates = aligned && capturing == hipStreamCaptureStatusNone && M > knn_block_columns(rows_padded, num_queries);
-    int rc = DSX_OK;
+    const bool candidates = aligned && capturing == hipStreamCaptureStatusNone && M > knn_block_columns(op.rows_padded, num_queries);
     bool redo = !candidates;
-    if (candidates) rc = knn_search_candidates(w, items, rows_padded, M, dim, queries, num_queries, k, scores, indexes, t, &redo);
+    if (rc == DSX_OK && candidates) rc = knn_search_candidates(w, op, M, num_queries, k, scores, indexes, t, &redo);
     g_knn_last_path = !candidates ? DSX_KNN_PATH_BLOCKS : (redo ? DSX_KNN_PATH_CANDIDATES_REDONE : DSX_KNN_PATH_CANDIDATES);
-    if (rc == DSX_OK && redo) rc = knn_search_blocks(w, items, rows_padded, M, dim, queries, num_queries, k, scores, indexes, t);
+    if (rc == DSX_OK && redo) rc = knn_search_blocks(w, op, M, num_queries, k, scores, indexes, t);
     if (elapsed_ms) {
         for (auto& e : t.ev) hipEventDestroy(e);
         elapsed_ms[0] = t.gemm;
         elapsed_ms[1] = t.topk;
     }
     return rc;
+}
+
+extern "C" {
+
+int dsx_knn_search(const float* items, uint32_t rows_padded, uint32_t padding, uint32_t dim, const float* queries,
+                   uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, void* workspace, size_t workspace_bytes,
+                   float* elapsed_ms)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(items && queries && scores && indexes, "dsx_knn_search: null device pointer");
+    DSX_CHECK_ARG(padding < rows_padded, "dsx_knn_search: padding %u leaves no item of %u", padding, rows_padded);
+    DSX_CHECK_ARG(dim > 0, "dsx_knn_search: dim is 0");
+    DSX_CHECK_ARG(k >= 1 && k <= 256, "dsx_knn_search: k = %u is outside 1..256", k);
+    if (num_queries == 0) return DSX_OK;
+    KnnOperands op;
+    op.items = items;
+    op.queries = queries;
+    op.rows_padded = rows_padded;
+    op.dim = dim;
+    const bool aligned = ((uintptr_t)items % 16) == 0 && ((uintptr_t)queries % 16) == 0 && (rows_padded % 4) == 0 && (dim % 4) == 0;
+    return knn_search_common(op, padding, num_queries, k, scores, indexes, workspace, workspace_bytes, elapsed_ms, aligned, nullptr);
+}
+
+int dsx_knn_search_f16(const void* items_f16, uint32_t rows_padded, uint32_t padding, uint32_t dim, const float* queries,
+                       uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, void* workspace, size_t workspace_bytes,
+                       float* elapsed_ms)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(items_f16 && queries && scores && indexes, "dsx_knn_search_f16: null device pointer");
+    DSX_CHECK_ARG(((uintptr_t)items_f16 % 16) == 0, "dsx_knn_search_f16: the fp16 table is not 16-byte aligned");
+    DSX_CHECK_ARG(padding < rows_padded, "dsx_knn_search_f16: padding %u leaves no item of %u", padding, rows_padded);
+    DSX_CHECK_ARG(dim > 0, "dsx_knn_search_f16: dim is 0");
+    DSX_CHECK_ARG(k >= 1 && k <= 256, "dsx_knn_search_f16: k = %u is outside 1..256", k);
+    if (num_queries == 0) return DSX_OK;
+    KnnOperands op;
+    op.f16 = true;
+    op.items16 = (const char*)items_f16;
+    op.rows_padded = rows_padded;
+    op.dim = dim;
+    op.ld16 = knn_f16_ld(dim);
+    return knn_search_common(op, padding, num_queries, k, scores, indexes, workspace, workspace_bytes, elapsed_ms, true, queries);
 }
 
 }  // extern "C"

@@ -1,0 +1,200 @@
+// dsx_knn_f16.hip — scores of the exact KNN search with items and queries stored as fp16 (the reference's DataType::FP16:
+// knn/KnnData.cpp:209-216 converts the table with kFloatToHalf, knn/KnnExactGpu.cu:108-116 converts every query batch, and
+// cublasSgemmEx multiplies fp16 operands into fp32 scores).
+//
+// Storage is this library's own: both operands row-major with the vector's components contiguous ([item][ld] and
+// [query][ld] halves, ld = dim rounded up to 32, zero filled; rows rounded up to the 128 of a tile, zero filled), which is
+// what v_mfma_f32_32x32x16_f16 wants — a lane's operand is 8 consecutive components of one row, one 128-bit read — and
+// leaves the k-loop without any bounds check.  A 256-lane workgroup (2 x 2 wavefronts) owns a 128 x 128 tile of scores;
+// 32 components of both operands per step are staged in LDS (double buffered, rows padded to 80 bytes so that the 128-bit
+// reads of 8 lanes cover all banks once).  Products of fp16 values are exact in fp32 and the sums are fp32, as in the
+// reference's GEMM.  Epilogues: plain store (first column block) or candidate lists (everything after it).
+#include "dsx_device.h"
+#include "dsx_internal.h"
+
+namespace dsx {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+
+constexpr int kF16Threads = 256;
+constexpr int kF16Xcds = 8;
+
+struct KnnF16Args {
+    const _Float16* A;      // queries [rows rounded up to 128][ld]
+    const _Float16* B;      // items of this column range [columns rounded up to 128][ld]
+    uint32_t ld;            // halves per row, a multiple of 32
+    uint32_t batch, n;      // valid rows of A, valid columns (items) of this range
+    uint32_t tiles_m, tiles_n;
+    float* Z;               // store mode: scores [batch][ldz]
+    uint32_t ldz;
+    CandArgs cand;          // candidate mode
+};
+
+template <bool CAND>
+__global__ __launch_bounds__(kF16Threads, 3) void knn_f16_kernel(KnnF16Args a)
+{
+    constexpr int BM = 128, BN = 128, BK = 32, PITCH = BK + 8;   // halves; 80-byte rows
+    __shared__ __attribute__((aligned(16))) _Float16 sA[2][BM][PITCH];
+    __shared__ __attribute__((aligned(16))) _Float16 sB[2][BN][PITCH];
+
+    const uint32_t total = a.tiles_m * a.tiles_n;
+    uint32_t wg = blockIdx.x;
+    {
+        const uint32_t per_xcd = (total + kF16Xcds - 1) / kF16Xcds;
+        const uint32_t xcd = wg % kF16Xcds, local = wg / kF16Xcds;
+        wg = xcd * per_xcd + local;
+        if (local >= per_xcd || wg >= total) return;
+    }
+    const uint32_t tm = wg % a.tiles_m, tn = wg / a.tiles_m;
+    const uint32_t row0 = tm * BM, col0 = tn * BN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    // staging: a tile step is 128 rows x 64 bytes per operand = 512 chunks of 16 bytes, two per lane and operand
+    const int srow = tid >> 2, spart = tid & 3;
+    const uint4* gA0 = reinterpret_cast<const uint4*>(a.A + (uint64_t)(row0 + srow) * a.ld) + spart;
+    const uint4* gA1 = reinterpret_cast<const uint4*>(a.A + (uint64_t)(row0 + srow + 64) * a.ld) + spart;
+    const uint4* gB0 = reinterpret_cast<const uint4*>(a.B + (uint64_t)(col0 + srow) * a.ld) + spart;
+    const uint4* gB1 = reinterpret_cast<const uint4*>(a.B + (uint64_t)(col0 + srow + 64) * a.ld) + spart;
+    uint4 ra0, ra1, rb0, rb1;
+    auto load = [&](uint32_t kt) __attribute__((always_inline)) {
+        const uint32_t o = kt * (BK / 8);   // in 16-byte chunks
+        ra0 = gA0[o]; ra1 = gA1[o]; rb0 = gB0[o]; rb1 = gB1[o];
+    };
+    auto store = [&](int buf) __attribute__((always_inline)) {
+        *reinterpret_cast<uint4*>(&sA[buf][srow][spart * 8]) = ra0;
+        *reinterpret_cast<uint4*>(&sA[buf][srow + 64][spart * 8]) = ra1;
+        *reinterpret_cast<uint4*>(&sB[buf][srow][spart * 8]) = rb0;
+        *reinterpret_cast<uint4*>(&sB[buf][srow + 64][spart * 8]) = rb1;
+    };
+    auto multiply = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ks++) {
+            half8 av[2], bv[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) av[i] = *reinterpret_cast<const half8*>(&sA[buf][wm * 64 + i * 32 + l32][ks * 16 + lhi * 8]);
+#pragma unroll
+            for (int j = 0; j < 2; j++) bv[j] = *reinterpret_cast<const half8*>(&sB[buf][wn * 64 + j * 32 + l32][ks * 16 + lhi * 8]);
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[j], acc[i][j], 0, 0, 0);
+        }
+    };
+
+    const uint32_t nk = a.ld / BK;
+    load(0);
+    store(0);
+    __syncthreads();
+    for (uint32_t kt = 0; kt < nk; kt++) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) load(kt + 1);
+        multiply(buf);
+        if (kt + 1 < nk) store(buf ^ 1);
+        __syncthreads();
+    }
+
+    if constexpr (CAND) {
+        static_assert(sizeof(sA) >= BM * sizeof(float), "the bounds reuse the query tile's LDS");
+        candidate_epilogue<2, 2>(acc, reinterpret_cast<float*>(&sA[0][0][0]), a.cand, row0, col0, a.batch, a.n, tid, wm, wn, l32, lhi);
+    } else {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const uint32_t c = col0 + wn * 64 + j * 32 + l32;
+            if (c >= a.n) continue;
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const uint32_t r = row0 + wm * 64 + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
+                    if (r < a.batch) a.Z[(uint64_t)r * a.ldz + c] = acc[i][j][v];
+                }
+        }
+    }
+}
+
+// fp32 -> fp16, round to nearest even (__float2half), into the padded row-major layout.  src is either column-major
+// (items: src[d * src_ld + row]) or row-major (queries: src[row * src_ld + d]); rows >= rows_valid and components >= dim
+// become zero.  One lane per 8 output halves.
+template <bool COLMAJOR>
+__global__ __launch_bounds__(256) void knn_to_f16_kernel(const float* src, uint64_t src_ld, uint32_t rows_valid, uint32_t dim, _Float16* dst,
+                                                         uint32_t rows_out, uint32_t ld)
+{
+    const uint64_t chunk = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    const uint32_t per_row = ld / 8;
+    uint32_t row, part;
+    if constexpr (COLMAJOR) {
+        // consecutive lanes take consecutive rows of one 8-component group: the reads of a component are then contiguous
+        const uint64_t rows64 = rows_out;
+        part = (uint32_t)(chunk / rows64);
+        row = (uint32_t)(chunk % rows64);
+        if (part >= per_row) return;
+    } else {
+        row = (uint32_t)(chunk / per_row);
+        part = (uint32_t)(chunk % per_row);
+        if (row >= rows_out) return;
+    }
+    half8 h;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const uint32_t d = part * 8 + e;
+        float x = 0.0f;
+        if (row < rows_valid && d < dim) x = COLMAJOR ? src[(uint64_t)d * src_ld + row] : src[(uint64_t)row * src_ld + d];
+        h[e] = (_Float16)x;
+    }
+    *reinterpret_cast<half8*>(dst + (uint64_t)row * ld + part * 8) = h;
+}
+
+uint32_t knn_f16_ld(uint32_t dim) { return (dim + 31) / 32 * 32; }
+uint64_t knn_f16_rows(uint64_t rows) { return (rows + 127) / 128 * 128; }
+
+int knn_to_f16(const float* src, bool colmajor, uint64_t src_ld, uint32_t rows_valid, uint32_t dim, void* dst, uint32_t rows_out)
+{
+    const uint32_t ld = knn_f16_ld(dim);
+    const uint64_t chunks = (uint64_t)rows_out * (ld / 8);
+    const uint32_t grid = (uint32_t)((chunks + 255) / 256);
+    if (colmajor)
+        hipLaunchKernelGGL((knn_to_f16_kernel<true>), dim3(grid), dim3(256), 0, ctx().stream, src, src_ld, rows_valid, dim, (_Float16*)dst, rows_out, ld);
+    else
+        hipLaunchKernelGGL((knn_to_f16_kernel<false>), dim3(grid), dim3(256), 0, ctx().stream, src, src_ld, rows_valid, dim, (_Float16*)dst, rows_out, ld);
+    DSX_LAUNCH_CHECK("knn_to_f16_kernel");
+    return DSX_OK;
+}
+
+// Scores of `batch` queries against `n` items starting at items16 (both in the padded fp16 layout): stored into Z[batch][ldz]
+// when cand == NULL, compared with the queries' bounds otherwise.
+int knn_f16_scores_run(const void* queries16, const void* items16, uint32_t ld, uint32_t batch, uint32_t n, float* Z, uint32_t ldz,
+                       const CandArgs* cand)
+{
+    KnnF16Args a{};
+    a.A = (const _Float16*)queries16;
+    a.B = (const _Float16*)items16;
+    a.ld = ld;
+    a.batch = batch;
+    a.n = n;
+    a.Z = Z;
+    a.ldz = ldz;
+    a.tiles_m = (batch + 127) / 128;
+    a.tiles_n = (n + 127) / 128;
+    const uint32_t total = a.tiles_m * a.tiles_n;
+    const uint32_t grid = ((total + kF16Xcds - 1) / kF16Xcds) * kF16Xcds;
+    if (cand) {
+        a.cand = *cand;
+        hipLaunchKernelGGL((knn_f16_kernel<true>), dim3(grid), dim3(kF16Threads), 0, ctx().stream, a);
+    } else {
+        hipLaunchKernelGGL((knn_f16_kernel<false>), dim3(grid), dim3(kF16Threads), 0, ctx().stream, a);
+    }
+    DSX_LAUNCH_CHECK("knn_f16_kernel");
+    return DSX_OK;
+}
+
+}  // namespace dsx

@@ -252,6 +252,25 @@ def knn_bench(args, pkg, lib):
                 "unit": "TFLOP/s", "frac": round(flops / el[0] / 1e9 / FP32_MFMA_PEAK_TF, 4), "traffic": None, "avg_launch_ms": round(el[0], 4),
                 "topk_ms": round(el[1], 4),
                 "path": {0: "blocks", 1: "candidate lists", 2: "candidate lists, redone block by block"}[lib.dsx_knn_last_search_path()]}
+    # the same search with fp16 storage of items and queries (the reference's DataType::FP16): reported beside the fp32 figure
+    table = pkg.DeviceArray((lib.dsx_knn_f16_table_bytes(rows, D),), np.uint8, lib)
+    pkg.check(lib.dsx_knn_f16_convert_items(dI.ptr, rows, pad, D, table.ptr))
+
+    def step16(timing=None):
+        pkg.check(lib.dsx_knn_search_f16(table.ptr, rows, pad, D, dQ.ptr, Q, K, scores.ptr, idx.ptr, None, 0, timing))
+    for _ in range(max(1, args.warmup)):
+        step16()
+    pkg.check(lib.dsx_sync())
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step16()
+    pkg.check(lib.dsx_sync())
+    ms16 = (time.perf_counter() - t0) * 1e3 / args.steps
+    step16(el)
+    f16 = {"ms_per_step": round(ms16, 4), "value": round(Q / (ms16 / 1e3), 1), "unit": "queries/s", "dtype": "f16 operands, f32 sums",
+           "kernel": "knn_f16_kernel", "bound": "mfma", "achieved": round(flops / el[0] / 1e9, 3), "peak": 2500.0, "unit_roofline": "TFLOP/s",
+           "frac": round(flops / el[0] / 1e9 / 2500.0, 4), "scores_ms": round(el[0], 4), "topk_ms": round(el[1], 4),
+           "path": {0: "blocks", 1: "candidate lists", 2: "candidate lists, redone block by block"}[lib.dsx_knn_last_search_path()]}
     cpu = None
     if args.cpu_seconds > 0:
         orc = entry.load_oracle()
@@ -267,7 +286,7 @@ def knn_bench(args, pkg, lib):
             "unit": "queries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
             "config": {"workload": p.name, "queries": Q, "dim": D, "items": rows - pad, "top_k": K}, "roofline": roofline,
-            "cpu_baseline": cpu}
+            "cpu_baseline": cpu, "f16_storage": f16}
 
 
 def main():

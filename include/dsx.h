@@ -231,6 +231,18 @@ int dsx_knn_search(const float* items, uint32_t rows_padded, uint32_t padding, u
                    uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, void* workspace, size_t workspace_bytes,
                    float* elapsed_ms);
 size_t dsx_knn_workspace_bytes(uint32_t rows_padded, uint32_t dim, uint32_t num_queries, uint32_t k);
+/* fp16 storage (astdl::knn::DataType::FP16).  The reference converts the column-major table once (KnnData::load,
+ * knn/KnnData.cpp:209-216, kFloatToHalf of knn/MathUtil.cu:33-81: round to nearest even) and every query batch before the
+ * GEMM (knn/KnnExactGpu.cu:108-116), multiplies fp16 operands and keeps fp32 scores.  Same arithmetic here; the fp16 table's
+ * layout is this library's own: dsx_knn_f16_convert_items turns the fp32 column-major device table (as dsx_knn_search takes
+ * it) into it, items_f16 (device, 16-byte aligned) holding dsx_knn_f16_table_bytes(rows_padded, dim) bytes; the fp32 table
+ * can be freed afterwards.  dsx_knn_search_f16 takes fp32 queries like dsx_knn_search and converts them in its workspace. */
+size_t dsx_knn_f16_table_bytes(uint32_t rows_padded, uint32_t dim);
+int dsx_knn_f16_convert_items(const float* items, uint32_t rows_padded, uint32_t padding, uint32_t dim, void* items_f16);
+int dsx_knn_search_f16(const void* items_f16, uint32_t rows_padded, uint32_t padding, uint32_t dim, const float* queries,
+                       uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, void* workspace, size_t workspace_bytes,
+                       float* elapsed_ms);
+size_t dsx_knn_workspace_bytes_f16(uint32_t rows_padded, uint32_t dim, uint32_t num_queries, uint32_t k);
 /* No counterpart in the reference: width of the first column block (rounded down to a multiple of 1024, at least 1024;
  * 0 restores the default of about 1 GiB of scores).  Workspace sizes depend on it: set it before asking for them. */
 int dsx_knn_set_block_columns(uint32_t columns);

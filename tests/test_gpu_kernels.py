@@ -635,3 +635,83 @@ def test_knn_search_unaligned_dim_takes_block_path(pkg, dsx, orc, synth, small_k
         r, c = np.nonzero(mism)
         assert np.abs(full[r, got_i[r, c]] - full[r, ref_i[r, c]]).max() < 1e-5
     assert_close(got_s, np.take_along_axis(full, got_i.astype(np.int64), axis=1), "knn scores", rel=1e-4, abs_floor=0.05)
+
+
+def knn_case_f16(pkg, dsx, orc, items_m, queries_m, k):
+    """fp16 storage: the fp32 column-major table is converted on the device, queries inside the search.  The oracle gets the
+    same operands rounded to fp16 (numpy rounds to nearest even like __float2half) and multiplies them in fp32."""
+    items, dim = items_m.shape
+    queries = queries_m.shape[0]
+    rows = (items + 7) // 8 * 8
+    pad = rows - items
+    cm = np.full((dim, rows), 50.0, dtype=np.float32)
+    cm[:, :items] = items_m.T
+    dI, dQ = dev(pkg, cm), dev(pkg, queries_m)
+    table = pkg.DeviceArray((dsx.dsx_knn_f16_table_bytes(rows, dim),), np.uint8)
+    pkg.check(dsx.dsx_knn_f16_convert_items(dI.ptr, rows, pad, dim, table.ptr))
+    scores = pkg.DeviceArray((queries, k), np.float32)
+    idx = pkg.DeviceArray((queries, k), np.uint32)
+    el = (C.c_float * 2)()
+    pkg.check(dsx.dsx_knn_search_f16(table.ptr, rows, pad, dim, dQ.ptr, queries, k, scores.ptr, idx.ptr, None, 0, el))
+    it16 = items_m.astype(np.float16).astype(np.float32)
+    q16 = queries_m.astype(np.float16).astype(np.float32)
+    cm16 = np.zeros((dim, rows), dtype=np.float32)
+    cm16[:, :items] = it16.T
+    ref_s, ref_i = orc.knn_search(cm16, rows, pad, dim, q16, k)
+    return scores.numpy(), idx.numpy(), ref_s, ref_i, it16, q16, table
+
+
+@pytest.mark.parametrize("items,queries,dim,k,blocks", [(1003, 9, 24, 10, 0), (50000, 64, 256, 100, 0), (30011, 70, 64, 100, 1024),
+                                                          (9000, 130, 250, 10, 1024), (26000, 33, 32, 200, 1024)])
+def test_knn_search_f16(pkg, dsx, orc, synth, items, queries, dim, k, blocks):
+    say("knn fp16 items=%d queries=%d dim=%d k=%d first block=%d" % (items, queries, dim, k, blocks))
+    p = synth.knn_config(seed=21, items=items, queries=queries, dim=dim, k=k)
+    dsx.dsx_knn_set_block_columns(blocks)
+    try:
+        got_s, got_i, ref_s, ref_i, it16, q16, _ = knn_case_f16(pkg, dsx, orc, p.items, p.queries, k)
+        assert dsx.dsx_knn_last_search_path() == (1 if blocks else 0)
+    finally:
+        dsx.dsx_knn_set_block_columns(0)
+    full = q16.astype(np.float64) @ it16.astype(np.float64).T
+    assert got_i.max() < items
+    mism = got_i != ref_i
+    if mism.any():
+        r, c = np.nonzero(mism)
+        assert np.abs(full[r, got_i[r, c]] - full[r, ref_i[r, c]]).max() < 1e-5
+    assert_close(got_s, np.take_along_axis(full, got_i.astype(np.int64), axis=1), "knn fp16 scores", rel=1e-4, abs_floor=0.05)
+    assert (np.diff(got_s, axis=1) <= 0).all()
+
+
+def test_knn_f16_table_layout_and_rounding(pkg, dsx, rng):
+    """The converted table: item-major rows of ld = dim rounded up to 32 halves, rows rounded up to 128, values rounded to
+    nearest even, padding rows and components zero."""
+    items, dim = 1003, 24
+    rows = (items + 7) // 8 * 8
+    it = (rng.standard_normal((items, dim)) * 3).astype(np.float32)
+    it[0, :4] = [65504.0, 1e-8, -0.0, 2049.0]          # largest half, flushes towards zero (a subnormal half or 0), -0, a tie (-> 2048)
+    cm = np.full((dim, rows), 7.0, dtype=np.float32)
+    cm[:, :items] = it.T
+    table = pkg.DeviceArray((dsx.dsx_knn_f16_table_bytes(rows, dim),), np.uint8)
+    pkg.check(dsx.dsx_knn_f16_convert_items(dev(pkg, cm).ptr, rows, rows - items, dim, table.ptr))
+    t = table.numpy().view(np.float16).reshape(-1, 32)
+    assert t.shape[0] == 1024
+    assert np.array_equal(t[:items, :dim].view(np.uint16), it.astype(np.float16).view(np.uint16))
+    assert (t[items:] == 0).all() and (t[:, dim:] == 0).all()
+
+
+def test_knn_search_f16_exact_ties_and_full_lists(pkg, dsx, orc, rng):
+    """Small integers are exact in fp16 too: bit-identical to the oracle, including the query whose candidates all tie."""
+    items, queries, dim, k = 21000, 40, 16, 100
+    it = rng.integers(-2, 3, size=(items, dim)).astype(np.float32)
+    q = rng.integers(-2, 3, size=(queries, dim)).astype(np.float32)
+    dsx.dsx_knn_set_block_columns(1024)
+    try:
+        got_s, got_i, ref_s, ref_i, _, _, _ = knn_case_f16(pkg, dsx, orc, it, q, k)
+        assert dsx.dsx_knn_last_search_path() == 1
+        assert np.array_equal(got_s, ref_s) and np.array_equal(got_i, ref_i)
+        q[3] = 0.0
+        got_s, got_i, ref_s, ref_i, _, _, _ = knn_case_f16(pkg, dsx, orc, it, q, k)
+        assert dsx.dsx_knn_last_search_path() == 2
+        assert np.array_equal(got_s, ref_s) and np.array_equal(got_i, ref_i)
+    finally:
+        dsx.dsx_knn_set_block_columns(0)
