@@ -170,7 +170,6 @@ KnnData::KnnData(int numGpus, int batchSize, int maxK, DataType dataType)
         msg << "This build searches on exactly one GPU (the whole item table lives in one device's HBM). Required " << numGpus;
         throw std::runtime_error(msg.str());
     }
-    if (dataType != DataType::FP32) throw std::runtime_error("Only fp32 item storage is available in this build");
     if (maxK < 1 || maxK > 256) throw std::invalid_argument("maxK must be in 1..256");
     check(dsx_init(0), "KnnData");
     fprintf(stderr, "INFO: Initializing KnnData with numGpus = %d, batchSize = %d, maxK = %d, dataType = %s\n", numGpus, batchSize, maxK,
@@ -203,15 +202,30 @@ void KnnData::load(int device, DataReader* dataReader)
     freeMatrix(hResultScores[device]);
     freeMatrix(hResultIndexes[device]);
     freeMatrix(dWorkspaces[device]);
-    dCollectionPartitions[device] = allocateMatrixOnDevice(rows, columns, sizeof(float));
-    check(dsx_memcpy_h2d(dCollectionPartitions[device].data, hTmpData, hTmp.getSizeInBytes()), "KnnData::load");
+    if (dataType == DataType::FP16) {
+        // knn/KnnData.cpp:209-216: the table is kept as halves (round to nearest even); the fp32 copy only lives until it is
+        // converted.  The fp16 table has this library's padded item-major layout, so its Matrix describes the logical shape
+        // (rows x columns of 2-byte elements) over an allocation of dsx_knn_f16_table_bytes.
+        Matrix dTmp = allocateMatrixOnDevice(rows, columns, sizeof(float));
+        check(dsx_memcpy_h2d(dTmp.data, hTmpData, hTmp.getSizeInBytes()), "KnnData::load");
+        void* table = nullptr;
+        check(dsx_malloc(&table, dsx_knn_f16_table_bytes(rows, (uint32_t)columns)), "KnnData::load");
+        dCollectionPartitions[device] = Matrix(table, rows, columns, 2, MemoryType::Device);
+        check(dsx_knn_f16_convert_items((const float*)dTmp.data, rows, rows - actualRows, (uint32_t)columns, table), "KnnData::load");
+        check(dsx_sync(), "KnnData::load");
+        freeMatrix(dTmp);
+    } else {
+        dCollectionPartitions[device] = allocateMatrixOnDevice(rows, columns, sizeof(float));
+        check(dsx_memcpy_h2d(dCollectionPartitions[device].data, hTmpData, hTmp.getSizeInBytes()), "KnnData::load");
+    }
     freeMatrix(hTmp);
     dInputBatches[device] = allocateMatrixOnDevice(batchSize, columns, sizeof(float));
     dResultScores[device] = allocateMatrixOnDevice(batchSize, maxK, sizeof(float));
     dResultIndexes[device] = allocateMatrixOnDevice(batchSize, maxK, sizeof(uint32_t));
     hResultScores[device] = allocateMatrixOnHost(batchSize, maxK, sizeof(float));
     hResultIndexes[device] = allocateMatrixOnHost(batchSize, maxK, sizeof(uint32_t));
-    const size_t ws = dsx_knn_workspace_bytes(rows, columns, batchSize, maxK);
+    const size_t ws = dataType == DataType::FP16 ? dsx_knn_workspace_bytes_f16(rows, columns, batchSize, maxK)
+                                                 : dsx_knn_workspace_bytes(rows, columns, batchSize, maxK);
     dWorkspaces[device] = allocateMatrixOnDevice(1, 1, ws);
     dsx_device_info info;
     check(dsx_get_device_info(&info), "KnnData::load");
@@ -286,10 +300,16 @@ void KnnExactGpu::search(int k, const float* inputs, int size, std::string* keys
 
     check(dsx_memcpy_h2d(dIn.data, inputs, (size_t)size * D * sizeof(float)), "KnnExactGpu::search");
     float elapsed[2] = {0, 0};
-    check(dsx_knn_search((const float*)items.data, items.numRows, data->collectionRowsPadded[device], (uint32_t)D, (const float*)dIn.data,
-                         (uint32_t)size, (uint32_t)maxK, dScores, dIndexes, data->dWorkspaces[device].data,
-                         data->dWorkspaces[device].elementSize, elapsed),
-          "KnnExactGpu::search");
+    if (data->dataType == DataType::FP16)
+        check(dsx_knn_search_f16(items.data, items.numRows, data->collectionRowsPadded[device], (uint32_t)D, (const float*)dIn.data,
+                                 (uint32_t)size, (uint32_t)maxK, dScores, dIndexes, data->dWorkspaces[device].data,
+                                 data->dWorkspaces[device].elementSize, elapsed),
+              "KnnExactGpu::search");
+    else
+        check(dsx_knn_search((const float*)items.data, items.numRows, data->collectionRowsPadded[device], (uint32_t)D, (const float*)dIn.data,
+                             (uint32_t)size, (uint32_t)maxK, dScores, dIndexes, data->dWorkspaces[device].data,
+                             data->dWorkspaces[device].elementSize, elapsed),
+              "KnnExactGpu::search");
     data->elapsedSgemm[device] = elapsed[0];
     data->elapsedTopK[device] = elapsed[1];
     check(dsx_memcpy_d2h(hScores, dScores, (size_t)size * maxK * sizeof(float)), "KnnExactGpu::search");

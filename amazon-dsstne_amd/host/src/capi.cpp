@@ -401,11 +401,13 @@ struct dsstne_knn {
     bool numericKeys = true;
 };
 
-dsstne_knn* dsstne_knn_create(uint32_t batch, uint32_t max_k)
+dsstne_knn* dsstne_knn_create(uint32_t batch, uint32_t max_k) { return dsstne_knn_create_typed(batch, max_k, "fp32"); }
+
+dsstne_knn* dsstne_knn_create_typed(uint32_t batch, uint32_t max_k, const char* data_type)
 {
     CAPI_TRY
     dsstne_knn* k = new dsstne_knn();
-    k->data = new astdl::knn::KnnData(1, (int)batch, (int)max_k, astdl::knn::DataType::FP32);
+    k->data = new astdl::knn::KnnData(1, (int)batch, (int)max_k, astdl::knn::getDataTypeFromString(data_type ? data_type : "fp32"));
     k->knn = new astdl::knn::KnnExactGpu(k->data);
     return k;
     CAPI_CATCH(nullptr)

@@ -40,6 +40,7 @@ SIGNATURES = {
     "dsstne_load_definition": ([_cp, _cp, _u32, _int, C.c_uint64], _vp),
     "dsstne_get_weights": ([_vp, _cp, _cp, _vp, C.c_size_t, _vp, C.c_size_t], _int),
     "dsstne_set_weights": ([_vp, _cp, _cp, _vp, C.c_size_t, _vp, C.c_size_t], _int),
+    "dsstne_knn_create_typed": ([_u32, _u32, _cp], _vp),
     "dsstne_knn_search": ([_vp, _u32, _vp, _u32, _vp, _vp], _int),
     "dsstne_knn_elapsed": ([_vp, C.POINTER(_f32), C.POINTER(_f32)], _int),
     "dsstne_knn_destroy": ([_vp], None),

@@ -277,3 +277,36 @@ def test_knn_api(pkg, dsx, orc, synth, tmp_path):
         assert i2[:, 0].tolist() == [0, 1, 2, 3, 4] and np.allclose(s2[:, 0], 1.0, atol=1e-5)
     finally:
         lib.dsstne_knn_destroy(knn)
+
+
+def test_knn_api_fp16_storage(pkg, dsx, orc, synth):
+    """KnnData(…, DataType::FP16) + KnnExactGpu::search: table and queries rounded to fp16, fp32 scores (knn/KnnData.cpp:209-216,
+    knn/KnnExactGpu.cu:108-116); a partial batch (size < batchSize) as the JNI passes it."""
+    from amazon_dsstne_amd import host_api
+    lib = host_api.load_host_library()
+    p = synth.knn_config(seed=6, items=12345, queries=21, dim=40, k=16)
+    assert not lib.dsstne_knn_create_typed(64, 32, b"fp8")
+    assert b"Unknown DataType" in lib.dsstne_last_error()
+    knn = lib.dsstne_knn_create_typed(64, 32, b"fp16")
+    assert knn, lib.dsstne_last_error()
+    try:
+        items = np.ascontiguousarray(p.items)
+        assert lib.dsstne_knn_load(knn, items.ctypes.data, items.shape[0], items.shape[1], None) == 0, lib.dsstne_last_error()
+        scores = np.empty((21, 16), dtype=np.float32)
+        idx = np.empty((21, 16), dtype=np.uint32)
+        q = np.ascontiguousarray(p.queries)
+        assert lib.dsstne_knn_search(knn, 16, q.ctypes.data, 21, scores.ctypes.data, idx.ctypes.data) == 0, lib.dsstne_last_error()
+        it16 = p.items.astype(np.float16).astype(np.float64)
+        q16 = p.queries.astype(np.float16).astype(np.float64)
+        full = q16 @ it16.T
+        order = np.argsort(-full, axis=1, kind="stable")[:, :16]
+        mism = idx != order
+        if mism.any():
+            r, c = np.nonzero(mism)
+            assert np.abs(full[r, idx[r, c]] - full[r, order[r, c]]).max() < 1e-5
+        assert_close(scores, np.take_along_axis(full, idx.astype(np.int64), axis=1), "knn fp16 scores", rel=1e-4, abs_floor=0.05)
+        # the rounding is visible: against the unrounded operands the scores are off by more than fp32 summation explains
+        exact = p.queries.astype(np.float64) @ p.items.astype(np.float64).T
+        assert np.abs(scores - np.take_along_axis(exact, idx.astype(np.int64), axis=1)).max() > 1e-5
+    finally:
+        lib.dsstne_knn_destroy(knn)
