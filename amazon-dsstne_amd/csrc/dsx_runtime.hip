@@ -31,6 +31,31 @@ static std::map<void*, size_t> g_host_allocs;
 
 using namespace dsx;
 
+// Uploads of up to kUploadSlotBytes go through a ring of pinned staging buffers: the caller's bytes are copied into a slot,
+// the DMA is queued on the library's stream and the call returns — the source may be reused at once (as after the blocking
+// cudaMemcpy of GpuBuffer::Upload), and everything queued later on the stream sees the data.  A batch's CSR arrays (four
+// uploads, engine/NNTypes.cpp:583-778) then cost four host copies instead of four round trips.  A slot is reused only after
+// its own copy has finished.
+constexpr int kUploadSlots = 8;
+constexpr size_t kUploadSlotBytes = (size_t)4 << 20;
+static char* g_upload_host[kUploadSlots] = {};
+static hipEvent_t g_upload_done[kUploadSlots] = {};
+static bool g_upload_busy[kUploadSlots] = {};
+static int g_upload_next = 0;
+
+static void upload_ring_release()
+{
+    for (int i = 0; i < kUploadSlots; i++) {
+        if (g_upload_host[i]) hipHostFree(g_upload_host[i]);
+        if (g_upload_done[i]) hipEventDestroy(g_upload_done[i]);
+        g_upload_host[i] = nullptr;
+        g_upload_done[i] = nullptr;
+        g_upload_busy[i] = false;
+    }
+    g_upload_next = 0;
+}
+
+
 extern "C" {
 
 const char* dsx_last_error(void) { return g_error; }
@@ -72,6 +97,7 @@ int dsx_shutdown(void)
     if (!c.initialized) return DSX_OK;
     if (--c.users > 0) return DSX_OK;
     hipStreamSynchronize(c.stream);
+    upload_ring_release();
     {
         std::lock_guard<std::mutex> lock(g_alloc_mutex);
         for (auto& kv : g_device_allocs) hipFree(kv.first);
@@ -202,8 +228,23 @@ int dsx_memcpy_h2d(void* dst, const void* src, size_t bytes)
     DSX_REQUIRE_INIT();
     if (bytes == 0) return DSX_OK;
     DSX_CHECK_ARG(dst && src, "dsx_memcpy_h2d: null pointer");
-    DSX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx().stream));
-    DSX_HIP(hipStreamSynchronize(ctx().stream));   // blocking like cudaMemcpy in GpuBuffer::Upload: src may be pageable
+    if (bytes > kUploadSlotBytes) {
+        DSX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx().stream));
+        DSX_HIP(hipStreamSynchronize(ctx().stream));   // src may be pageable: wait until it has been read
+        return DSX_OK;
+    }
+    std::lock_guard<std::mutex> lock(g_alloc_mutex);
+    const int slot = g_upload_next;
+    g_upload_next = (g_upload_next + 1) % kUploadSlots;
+    if (!g_upload_host[slot]) {
+        DSX_HIP(hipHostMalloc((void**)&g_upload_host[slot], kUploadSlotBytes, hipHostMallocDefault));
+        DSX_HIP(hipEventCreateWithFlags(&g_upload_done[slot], hipEventDisableTiming));
+    }
+    if (g_upload_busy[slot]) DSX_HIP(hipEventSynchronize(g_upload_done[slot]));
+    memcpy(g_upload_host[slot], src, bytes);
+    DSX_HIP(hipMemcpyAsync(dst, g_upload_host[slot], bytes, hipMemcpyHostToDevice, ctx().stream));
+    DSX_HIP(hipEventRecord(g_upload_done[slot], ctx().stream));
+    g_upload_busy[slot] = true;
     return DSX_OK;
 }
 

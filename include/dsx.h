@@ -109,7 +109,9 @@ int dsx_malloc_host(void** host_ptr, size_t bytes);
 int dsx_free(void* device_ptr);
 int dsx_free_host(void* host_ptr);
 int dsx_memset(void* device_ptr, int value, size_t bytes);
-int dsx_memcpy_h2d(void* device_dst, const void* host_src, size_t bytes);   /* GpuBuffer::Upload   */
+/* GpuBuffer::Upload.  host_src may be reused as soon as the call returns; the copy itself is ordered on the library's stream
+ * before everything queued later (uploads of up to 4 MiB are staged in pinned memory and not waited for). */
+int dsx_memcpy_h2d(void* device_dst, const void* host_src, size_t bytes);
 int dsx_memcpy_d2h(void* host_dst, const void* device_src, size_t bytes);   /* GpuBuffer::Download */
 int dsx_memcpy_d2d(void* device_dst, const void* device_src, size_t bytes); /* GpuBuffer::Copy     */
 int dsx_sync(void);
