@@ -72,24 +72,38 @@ struct CandArgs {
     uint32_t* overflow;
 };
 
-// Epilogue of a 2 x 2 wavefront workgroup whose wavefront (wm, wn) holds MI x NI accumulators of 32 x 32 (register v of lane l:
-// row 8*(v/4) + 4*(l/32) + v%4, column l%32): the tile is only compared with the rows' admission bounds.  A bound is the key
-// of a score that k items seen earlier reach, so almost every tile ends after MI * NI * 16 compares per lane; the few
-// survivors are appended to their rows' lists with one atomic each.  The bounds of the tile's 64*MI rows are staged in LDS
-// (sBound, free for use by now) as floats, four consecutive rows per 128-bit read; a NaN score fails "x < bound" and is
-// sorted out by its key.  Every lane of the workgroup must call this.
-template <int MI, int NI>
-__device__ __forceinline__ void candidate_epilogue(const floatx16 (&acc)[MI][NI], float* sBound, const CandArgs& c, uint32_t row0,
-                                                   uint32_t col0, uint32_t batch, uint32_t n, int tid, int wm, int wn, int l32, int lhi)
+// The epilogue below needs the admission bounds of the tile's rows.  Lane t < 32*MI*WM asks for row t's bound here, at the start
+// of the kernel: asked for in the epilogue, the load's latency would sit at the end of every tile.
+template <int MI, int WM = 2>
+__device__ __forceinline__ uint32_t candidate_bound_prefetch(const CandArgs& c, uint32_t row0, uint32_t batch, int tid)
 {
-    constexpr int BM = 64 * MI;
-    if (tid < BM) {
-        const uint32_t r = row0 + tid;
-        sBound[tid] = (r < batch) ? key_score(c.row_bound[r]) : __builtin_inff();
-    }
+    uint32_t key = 0xffffffffu;   // rows beyond the batch admit nothing
+    if (tid < 32 * MI * WM && row0 + tid < batch) key = c.row_bound[row0 + tid];
+    return key;
+}
+
+// Epilogue of a workgroup of WM x WN wavefronts whose wavefront (wm, wn) holds MI x NI accumulators of 32 x 32 (register v of
+// lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32): the tile is only compared with the rows' admission bounds.  A bound is the key
+// of a score that k items seen earlier reach, so a lane usually ends after its MI * NI * 16 compares.  The bounds of the
+// tile's 32*MI*WM rows are staged in LDS as floats (`lds`: kCandLdsBytes of workgroup memory that is free by now), four
+// consecutive rows per 128-bit read; "not (x < bound)" also lets NaN scores and a few scores whose key is below the bound's
+// through, which the merge of the lists sorts out.  A wavefront with survivors first gathers them in a list in LDS and
+// then appends the whole list to the rows' global lists, one atomic per survivor but all of them in flight together: asked
+// for one by one, each atomic's round trip (thousands of cycles) would be waited for separately.
+// bound_key is what candidate_bound_prefetch returned to this lane.  Every lane of the workgroup must call this.
+constexpr int kCandWaveList = 256;   // survivors a wavefront gathers before it appends them
+template <int MI, int WM = 2, int WN = 2> constexpr int kCandLdsBytes = 32 * MI * WM * 4 + WM * WN * kCandWaveList * 12;
+
+template <int MI, int NI, int WM = 2, int WN = 2>
+__device__ __forceinline__ void candidate_epilogue(const floatx16 (&acc)[MI][NI], float* lds, const CandArgs& c, uint32_t bound_key,
+                                                   uint32_t row0, uint32_t col0, uint32_t batch, uint32_t n, int tid, int wm, int wn, int l32,
+                                                   int lhi)
+{
+    constexpr int BM = 32 * MI * WM;   // at most as many rows as the workgroup has lanes
+    float* sBound = lds;
+    if (tid < BM) sBound[tid] = (row0 + tid < batch) ? key_score(bound_key) : __builtin_inff();
     __syncthreads();
     float bf[MI][4][4];
-    bool any = false;
 #pragma unroll
     for (int i = 0; i < MI; i++)
 #pragma unroll
@@ -97,35 +111,71 @@ __device__ __forceinline__ void candidate_epilogue(const floatx16 (&acc)[MI][NI]
             const float4 t = *reinterpret_cast<const float4*>(&sBound[wm * 32 * MI + i * 32 + 8 * g + 4 * lhi]);
             bf[i][g][0] = t.x; bf[i][g][1] = t.y; bf[i][g][2] = t.z; bf[i][g][3] = t.w;
         }
+    // one compare per score, its wavefront-wide result (a scalar register pair) gathered per 32 x 32 block: nothing else
+    // happens for a block without survivors
+    uint64_t block_mask[MI][NI];
+    uint64_t any_mask = 0;
 #pragma unroll
     for (int i = 0; i < MI; i++)
 #pragma unroll
-        for (int j = 0; j < NI; j++)
+        for (int j = 0; j < NI; j++) {
+            uint64_t m = 0;
 #pragma unroll
-            for (int v = 0; v < 16; v++) any |= !(acc[i][j][v] < bf[i][v / 4][v % 4]);
-    if (!any) return;
+            for (int v = 0; v < 16; v++) m |= __builtin_amdgcn_ballot_w64(!(acc[i][j][v] < bf[i][v / 4][v % 4]));
+            block_mask[i][j] = m;
+            any_mask |= m;
+        }
+    if (any_mask == 0) return;   // nothing among this wavefront's scores
+
+    const int wave = tid >> 6, lane = tid & 63;
+    uint64_t* sWord = reinterpret_cast<uint64_t*>(lds + BM) + wave * kCandWaveList;
+    uint32_t* sRow = reinterpret_cast<uint32_t*>(reinterpret_cast<uint64_t*>(lds + BM) + WM * WN * kCandWaveList) + wave * kCandWaveList;
+    uint32_t listed = 0;   // wavefront-uniform
+    auto append_all = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        for (uint32_t e = lane; e < listed; e += 64) {
+            const uint32_t r = sRow[e];
+            const uint64_t word = sWord[e];
+            if (r == 0xffffffffu) continue;
+            const uint32_t pos = atomicAdd(&c.cand_count[r], 1u);
+            if (pos < c.cand_cap)
+                c.cand[(uint64_t)r * c.cand_cap + pos] = word;
+            else
+                *c.overflow = 1u;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        listed = 0;
+    };
 #pragma unroll
     for (int j = 0; j < NI; j++) {
         const uint32_t col = col0 + wn * 32 * NI + j * 32 + l32;
-        if (col >= n) continue;
+        const bool col_ok = col < n;   // columns beyond the range hold sums over zero padding, which a bound <= 0 would let through
+        const uint64_t col_mask = __builtin_amdgcn_ballot_w64(col_ok);
 #pragma unroll
         for (int i = 0; i < MI; i++) {
+            if ((block_mask[i][j] & col_mask) == 0) continue;
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const float x = acc[i][j][v];
-                if (x < bf[i][v / 4][v % 4]) continue;
+                float x = acc[i][j][v];
+                asm volatile("" : "+v"(x));   // compared afresh: results kept from the pass above would cost more than they save
+                const uint64_t mask = __builtin_amdgcn_ballot_w64(!(x < bf[i][v / 4][v % 4]) && col_ok);
+                if (mask == 0) continue;
+                const bool cand = (mask >> lane) & 1;
                 const uint32_t r = row0 + wm * 32 * MI + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
-                if (r >= batch) continue;
-                const uint32_t key = score_key(x);
-                if (key < c.row_bound[r]) continue;
-                const uint32_t pos = atomicAdd(&c.cand_count[r], 1u);
-                if (pos < c.cand_cap)
-                    c.cand[(uint64_t)r * c.cand_cap + pos] = ((uint64_t)key << 32) | (uint32_t)~(c.col_offset + col);
-                else
-                    *c.overflow = 1u;
+                const uint32_t count = (uint32_t)__builtin_popcountll(mask);
+                if (listed + count > (uint32_t)kCandWaveList) append_all();
+                if (cand) {
+                    const uint32_t slot = listed + __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+                    sWord[slot] = ((uint64_t)score_key(x) << 32) | (uint32_t)~(c.col_offset + col);
+                    sRow[slot] = (r < batch) ? r : 0xffffffffu;   // (rows beyond the batch have an infinite bound: never taken)
+                }
+                listed += count;
             }
         }
     }
+    append_all();
 }
 
 // CalculateActivation (engine/NNLayer.cpp:1646-1683) runs a kernel only for sigmoid, tanh, ReLU, leaky ReLU, ELU, SELU and

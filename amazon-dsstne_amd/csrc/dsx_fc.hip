@@ -68,6 +68,8 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
     float ra[A_ELEMS], rb[B_ELEMS];
+    uint32_t bound_key = 0;
+    if constexpr (CAND) bound_key = candidate_bound_prefetch<MI>(a.cand, row0, a.batch, tid);
 
     // X tile: element (i, kk) of the tile is X[row0 + i][k0 + kk]; lanes walk k fastest.
     auto load_a = [&](uint32_t k0) {
@@ -261,6 +263,7 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
                 }
             };
             load_lean(0);
+            if constexpr (CAND) asm volatile("" ::"v"(bound_key));   // the bound's load is issued up here, not moved down to its use
             store_a(0);
             store_b(0);
             __syncthreads();
@@ -279,6 +282,7 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
     if (!lean) {
         load_a(0);
         load_b(0);
+        if constexpr (CAND) asm volatile("" ::"v"(bound_key));
         store_a(0);
         store_b(0);
         __syncthreads();
@@ -298,9 +302,9 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
     }
 
     if constexpr (CAND) {
-        static_assert(sizeof(sA) >= BM * sizeof(float), "the bounds reuse the X tile's LDS");
+        static_assert(sizeof(sA) >= kCandLdsBytes<MI>, "the epilogue reuses the X tile's LDS");
         // (the k-loop ended with a barrier: every wavefront is done with sA)
-        candidate_epilogue<MI, NI>(acc, &sA[0][0][0], a.cand, row0, col0, a.batch, a.n, tid, wm, wn, l32, lhi);
+        candidate_epilogue<MI, NI>(acc, &sA[0][0][0], a.cand, bound_key, row0, col0, a.batch, a.n, tid, wm, wn, l32, lhi);
         return;
     }
 

@@ -52,7 +52,7 @@ struct KnnWorkspace {
     uint32_t* cand_count;   // [queries]
     uint32_t* overflow;     // [1] (+ padding)
     uint64_t* cand;         // [queries][kCandCap]
-    void* queries16;        // fp16 storage only: the query batch, [queries rounded up to 128][ld] halves
+    void* queries16;        // fp16 storage only: the query batch, [queries rounded up to 256][ld] halves
     size_t bytes;
 };
 
@@ -83,7 +83,7 @@ struct KnnOperands {
     bool f16 = false;
     const float* items = nullptr;       // fp32: column-major [dim][rows_padded]
     const float* queries = nullptr;     // fp32: [queries][dim]
-    const char* items16 = nullptr;      // fp16: [rows rounded up to 128][ld]
+    const char* items16 = nullptr;      // fp16: [rows rounded up to 256][ld]
     const void* queries16 = nullptr;
     uint32_t rows_padded = 0, dim = 0, ld16 = 0;
 

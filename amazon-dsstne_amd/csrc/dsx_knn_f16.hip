@@ -3,7 +3,7 @@
 // cublasSgemmEx multiplies fp16 operands into fp32 scores).
 //
 // Storage is this library's own: both operands row-major with the vector's components contiguous ([item][ld] and
-// [query][ld] halves, ld = dim rounded up to 32, zero filled; rows rounded up to the 128 of a tile, zero filled), which is
+// [query][ld] halves, ld = dim rounded up to 64, zero filled; rows rounded up to 256, the tallest tile, zero filled), which is
 // what v_mfma_f32_32x32x16_f16 wants — a lane's operand is 8 consecutive components of one row, one 128-bit read — and
 // leaves the k-loop without any bounds check.  A 256-lane workgroup (2 x 2 wavefronts) owns a 128 x 128 tile of scores;
 // 32 components of both operands per step are staged in LDS (double buffered, rows padded to 80 bytes so that the 128-bit
@@ -16,13 +16,12 @@ namespace dsx {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 
-constexpr int kF16Threads = 256;
 constexpr int kF16Xcds = 8;
 
 struct KnnF16Args {
-    const _Float16* A;      // queries [rows rounded up to 128][ld]
-    const _Float16* B;      // items of this column range [columns rounded up to 128][ld]
-    uint32_t ld;            // halves per row, a multiple of 32
+    const _Float16* A;      // queries [rows rounded up to 256][ld]
+    const _Float16* B;      // items of this column range [columns rounded up to 256][ld]
+    uint32_t ld;            // halves per row, a multiple of 64
     uint32_t batch, n;      // valid rows of A, valid columns (items) of this range
     uint32_t tiles_m, tiles_n;
     float* Z;               // store mode: scores [batch][ldz]
@@ -30,10 +29,16 @@ struct KnnF16Args {
     CandArgs cand;          // candidate mode
 };
 
-template <bool CAND>
-__global__ __launch_bounds__(kF16Threads, 3) void knn_f16_kernel(KnnF16Args a)
+// MI x NI accumulator blocks of 32 x 32 per wavefront, WM x WN wavefronts per workgroup: a (32*MI*WM) x (32*NI*WN) tile, with
+// as many rows and columns as half the workgroup's lanes (two 16-byte chunks per lane, operand and step).  WPE: wavefronts
+// per SIMD the register budget is sized for.
+template <int MI, int NI, int WM, int WN, int WPE, bool CAND>
+__global__ __launch_bounds__(64 * WM * WN) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void knn_f16_kernel(KnnF16Args a)
 {
-    constexpr int BM = 128, BN = 128, BK = 32, PITCH = BK + 8;   // halves; 80-byte rows
+    constexpr int THREADS = 64 * WM * WN;
+    constexpr int BM = 32 * MI * WM, BN = 32 * NI * WN, BK = 32, PITCH = BK + 8;   // halves; 80-byte rows
+    constexpr int RS = THREADS / 4;                                                // rows between a lane's two chunks
+    static_assert(BM == THREADS / 2 && BN == THREADS / 2, "two chunks per lane, operand and step");
     __shared__ __attribute__((aligned(16))) _Float16 sA[2][BM][PITCH];
     __shared__ __attribute__((aligned(16))) _Float16 sB[2][BN][PITCH];
 
@@ -48,74 +53,92 @@ __global__ __launch_bounds__(kF16Threads, 3) void knn_f16_kernel(KnnF16Args a)
     const uint32_t tm = wg % a.tiles_m, tn = wg / a.tiles_m;
     const uint32_t row0 = tm * BM, col0 = tn * BN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
     const int l32 = lane & 31, lhi = lane >> 5;
 
-    floatx16 acc[2][2];
+    floatx16 acc[MI][NI];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < NI; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    // staging: a tile step is 128 rows x 64 bytes per operand = 512 chunks of 16 bytes, two per lane and operand
+    // A step of a tile is 64 bytes per row = four chunks of 16 bytes; lane t takes chunk t % 4 of rows t / 4 and t / 4 + RS of
+    // both operands.  The loads of the next two steps are in flight in registers (two stages of named registers — 128-bit
+    // values reached through arrays or references from inside lambdas would live in scratch memory); the step that is due
+    // next is written to the LDS double buffer while the current one is multiplied.
     const int srow = tid >> 2, spart = tid & 3;
-    const uint4* gA0 = reinterpret_cast<const uint4*>(a.A + (uint64_t)(row0 + srow) * a.ld) + spart;
-    const uint4* gA1 = reinterpret_cast<const uint4*>(a.A + (uint64_t)(row0 + srow + 64) * a.ld) + spart;
-    const uint4* gB0 = reinterpret_cast<const uint4*>(a.B + (uint64_t)(col0 + srow) * a.ld) + spart;
-    const uint4* gB1 = reinterpret_cast<const uint4*>(a.B + (uint64_t)(col0 + srow + 64) * a.ld) + spart;
-    uint4 ra0, ra1, rb0, rb1;
-    auto load = [&](uint32_t kt) __attribute__((always_inline)) {
-        const uint32_t o = kt * (BK / 8);   // in 16-byte chunks
-        ra0 = gA0[o]; ra1 = gA1[o]; rb0 = gB0[o]; rb1 = gB1[o];
-    };
-    auto store = [&](int buf) __attribute__((always_inline)) {
-        *reinterpret_cast<uint4*>(&sA[buf][srow][spart * 8]) = ra0;
-        *reinterpret_cast<uint4*>(&sA[buf][srow + 64][spart * 8]) = ra1;
-        *reinterpret_cast<uint4*>(&sB[buf][srow][spart * 8]) = rb0;
-        *reinterpret_cast<uint4*>(&sB[buf][srow + 64][spart * 8]) = rb1;
-    };
+    const uint4* gA = reinterpret_cast<const uint4*>(a.A + (uint64_t)(row0 + srow) * a.ld) + spart;
+    const uint4* gB = reinterpret_cast<const uint4*>(a.B + (uint64_t)(col0 + srow) * a.ld) + spart;
+    const uint32_t rstep = RS * (a.ld / 8);   // chunks between a lane's two rows
+    const uint32_t nk = a.ld / BK;            // a multiple of 2
+#define F16_LOAD(S, KT)                                                                                                  \
+    do {                                                                                                                 \
+        const uint32_t o_ = min((uint32_t)(KT), nk - 1) * (BK / 8); /* past the end: the last step again, never used */  \
+        S##a0 = gA[o_];                                                                                                  \
+        S##a1 = gA[o_ + rstep];                                                                                          \
+        S##b0 = gB[o_];                                                                                                  \
+        S##b1 = gB[o_ + rstep];                                                                                          \
+    } while (0)
+#define F16_STORE(S, BUF)                                                         \
+    do {                                                                          \
+        *reinterpret_cast<uint4*>(&sA[BUF][srow][spart * 8]) = S##a0;             \
+        *reinterpret_cast<uint4*>(&sA[BUF][srow + RS][spart * 8]) = S##a1;        \
+        *reinterpret_cast<uint4*>(&sB[BUF][srow][spart * 8]) = S##b0;             \
+        *reinterpret_cast<uint4*>(&sB[BUF][srow + RS][spart * 8]) = S##b1;        \
+    } while (0)
     auto multiply = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ks++) {
-            half8 av[2], bv[2];
+            half8 av[MI], bv[NI];
 #pragma unroll
-            for (int i = 0; i < 2; i++) av[i] = *reinterpret_cast<const half8*>(&sA[buf][wm * 64 + i * 32 + l32][ks * 16 + lhi * 8]);
+            for (int i = 0; i < MI; i++) av[i] = *reinterpret_cast<const half8*>(&sA[buf][wm * 32 * MI + i * 32 + l32][ks * 16 + lhi * 8]);
 #pragma unroll
-            for (int j = 0; j < 2; j++) bv[j] = *reinterpret_cast<const half8*>(&sB[buf][wn * 64 + j * 32 + l32][ks * 16 + lhi * 8]);
+            for (int j = 0; j < NI; j++) bv[j] = *reinterpret_cast<const half8*>(&sB[buf][wn * 32 * NI + j * 32 + l32][ks * 16 + lhi * 8]);
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < MI; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < NI; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[j], acc[i][j], 0, 0, 0);
         }
     };
 
-    const uint32_t nk = a.ld / BK;
-    load(0);
-    store(0);
+    uint32_t bound_key = 0;
+    if constexpr (CAND) bound_key = candidate_bound_prefetch<MI, WM>(a.cand, row0, a.batch, tid);
+    uint4 s0a0, s0a1, s0b0, s0b1, s1a0, s1a1, s1b0, s1b1;
+    F16_LOAD(s0, 0);
+    F16_LOAD(s1, 1);
+    if constexpr (CAND) asm volatile("" ::"v"(bound_key));   // the bound's load is issued up here, not moved down to its use
+    F16_STORE(s0, 0);
     __syncthreads();
-    for (uint32_t kt = 0; kt < nk; kt++) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) load(kt + 1);
-        multiply(buf);
-        if (kt + 1 < nk) store(buf ^ 1);
+    for (uint32_t kt = 0; kt < nk; kt += 2) {
+        // step kt + j multiplies LDS buffer j; its stage's registers are free again and take step kt + j + 2
+        F16_LOAD(s0, kt + 2);
+        multiply(0);
+        F16_STORE(s1, 1);
+        __syncthreads();
+        F16_LOAD(s1, kt + 3);
+        multiply(1);
+        F16_STORE(s0, 0);
         __syncthreads();
     }
+#undef F16_LOAD
+#undef F16_STORE
 
     if constexpr (CAND) {
-        static_assert(sizeof(sA) >= BM * sizeof(float), "the bounds reuse the query tile's LDS");
-        candidate_epilogue<2, 2>(acc, reinterpret_cast<float*>(&sA[0][0][0]), a.cand, row0, col0, a.batch, a.n, tid, wm, wn, l32, lhi);
+        static_assert(sizeof(sA) >= kCandLdsBytes<MI, WM, WN>, "the epilogue reuses the query tile's LDS");
+        candidate_epilogue<MI, NI, WM, WN>(acc, reinterpret_cast<float*>(&sA[0][0][0]), a.cand, bound_key, row0, col0, a.batch, a.n, tid, wm, wn,
+                                           l32, lhi);
     } else {
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const uint32_t c = col0 + wn * 64 + j * 32 + l32;
+        for (int j = 0; j < NI; j++) {
+            const uint32_t c = col0 + wn * 32 * NI + j * 32 + l32;
             if (c >= a.n) continue;
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < MI; i++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
-                    const uint32_t r = row0 + wm * 64 + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
+                    const uint32_t r = row0 + wm * 32 * MI + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
                     if (r < a.batch) a.Z[(uint64_t)r * a.ldz + c] = acc[i][j][v];
                 }
         }
@@ -154,8 +177,8 @@ __global__ __launch_bounds__(256) void knn_to_f16_kernel(const float* src, uint6
     *reinterpret_cast<half8*>(dst + (uint64_t)row * ld + part * 8) = h;
 }
 
-uint32_t knn_f16_ld(uint32_t dim) { return (dim + 31) / 32 * 32; }
-uint64_t knn_f16_rows(uint64_t rows) { return (rows + 127) / 128 * 128; }
+uint32_t knn_f16_ld(uint32_t dim) { return (dim + 63) / 64 * 64; }   // two pipeline steps of 32 components
+uint64_t knn_f16_rows(uint64_t rows) { return (rows + 255) / 256 * 256; }   // the tallest tile
 
 int knn_to_f16(const float* src, bool colmajor, uint64_t src_ld, uint32_t rows_valid, uint32_t dim, void* dst, uint32_t rows_out)
 {
@@ -168,6 +191,21 @@ int knn_to_f16(const float* src, bool colmajor, uint64_t src_ld, uint32_t rows_v
         hipLaunchKernelGGL((knn_to_f16_kernel<false>), dim3(grid), dim3(256), 0, ctx().stream, src, src_ld, rows_valid, dim, (_Float16*)dst, rows_out, ld);
     DSX_LAUNCH_CHECK("knn_to_f16_kernel");
     return DSX_OK;
+}
+
+template <int MI, int NI, int WM, int WN, int WPE> static void launch_f16(KnnF16Args& a, const CandArgs* cand)
+{
+    constexpr int BM = 32 * MI * WM, BN = 32 * NI * WN;
+    a.tiles_m = (a.batch + BM - 1) / BM;
+    a.tiles_n = (a.n + BN - 1) / BN;
+    const uint32_t total = a.tiles_m * a.tiles_n;
+    const uint32_t grid = ((total + kF16Xcds - 1) / kF16Xcds) * kF16Xcds;
+    if (cand) {
+        a.cand = *cand;
+        hipLaunchKernelGGL((knn_f16_kernel<MI, NI, WM, WN, WPE, true>), dim3(grid), dim3(64 * WM * WN), 0, ctx().stream, a);
+    } else {
+        hipLaunchKernelGGL((knn_f16_kernel<MI, NI, WM, WN, WPE, false>), dim3(grid), dim3(64 * WM * WN), 0, ctx().stream, a);
+    }
 }
 
 // Scores of `batch` queries against `n` items starting at items16 (both in the padded fp16 layout): stored into Z[batch][ldz]
@@ -183,16 +221,9 @@ int knn_f16_scores_run(const void* queries16, const void* items16, uint32_t ld, 
     a.n = n;
     a.Z = Z;
     a.ldz = ldz;
-    a.tiles_m = (batch + 127) / 128;
-    a.tiles_n = (n + 127) / 128;
-    const uint32_t total = a.tiles_m * a.tiles_n;
-    const uint32_t grid = ((total + kF16Xcds - 1) / kF16Xcds) * kF16Xcds;
-    if (cand) {
-        a.cand = *cand;
-        hipLaunchKernelGGL((knn_f16_kernel<true>), dim3(grid), dim3(kF16Threads), 0, ctx().stream, a);
-    } else {
-        hipLaunchKernelGGL((knn_f16_kernel<false>), dim3(grid), dim3(kF16Threads), 0, ctx().stream, a);
-    }
+    // 128 x 128 tiles, four workgroups per CU (their 40 KiB of LDS each fill the CU's 160 KiB).  Measured against it on config 5:
+    // 256 x 256 tiles with eight wavefronts (6.6 ms vs 6.0), three workgroups per CU (6.3 ms).
+    launch_f16<2, 2, 2, 2, 4>(a, cand);
     DSX_LAUNCH_CHECK("knn_f16_kernel");
     return DSX_OK;
 }

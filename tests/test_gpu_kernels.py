@@ -683,7 +683,7 @@ def test_knn_search_f16(pkg, dsx, orc, synth, items, queries, dim, k, blocks):
 
 
 def test_knn_f16_table_layout_and_rounding(pkg, dsx, rng):
-    """The converted table: item-major rows of ld = dim rounded up to 32 halves, rows rounded up to 128, values rounded to
+    """The converted table: item-major rows of ld = dim rounded up to 64 halves, rows rounded up to 256, values rounded to
     nearest even, padding rows and components zero."""
     items, dim = 1003, 24
     rows = (items + 7) // 8 * 8
@@ -693,7 +693,7 @@ def test_knn_f16_table_layout_and_rounding(pkg, dsx, rng):
     cm[:, :items] = it.T
     table = pkg.DeviceArray((dsx.dsx_knn_f16_table_bytes(rows, dim),), np.uint8)
     pkg.check(dsx.dsx_knn_f16_convert_items(dev(pkg, cm).ptr, rows, rows - items, dim, table.ptr))
-    t = table.numpy().view(np.float16).reshape(-1, 32)
+    t = table.numpy().view(np.float16).reshape(-1, 64)
     assert t.shape[0] == 1024
     assert np.array_equal(t[:items, :dim].view(np.uint16), it.astype(np.float16).view(np.uint16))
     assert (t[items:] == 0).all() and (t[:, dim:] == 0).all()
