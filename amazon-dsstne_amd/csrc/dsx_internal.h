@@ -20,6 +20,7 @@ struct Context {
 };
 
 Context& ctx();
+int current_lane();   // 0 or 1: which of the two in-order streams ctx().stream is (scratch buffers are kept per lane)
 int set_error(int code, const char* fmt, ...);
 
 // engine/NNTypes.h:49

@@ -18,8 +18,8 @@
 
 namespace dsx {
 
-static void* g_knn_ws = nullptr;
-static size_t g_knn_ws_bytes = 0;
+static void* g_knn_ws_of[2] = {nullptr, nullptr};   // per lane
+static size_t g_knn_ws_bytes_of[2] = {0, 0};
 
 static uint32_t g_knn_block_columns = 0;   // 0: sized by the rule below
 static int g_knn_last_path = 0;            // how the last search ran: DSX_KNN_PATH_*
@@ -232,6 +232,8 @@ static int knn_search_common(KnnOperands& op, uint32_t padding, uint32_t num_que
         DSX_CHECK_ARG(workspace_bytes >= need, "dsx_knn_search: workspace of %zu bytes, %zu needed", workspace_bytes, need);
         DSX_CHECK_ARG(((uintptr_t)workspace % 256) == 0, "dsx_knn_search: workspace is not 256-byte aligned");
     } else {
+        void*& g_knn_ws = g_knn_ws_of[current_lane()];
+        size_t& g_knn_ws_bytes = g_knn_ws_bytes_of[current_lane()];
         if (g_knn_ws_bytes < need) {
             if (g_knn_ws) {
                 DSX_HIP(hipStreamSynchronize(ctx().stream));

@@ -56,6 +56,63 @@ static void upload_ring_release()
 }
 
 
+// Two lanes: independent in-order streams, so that the kernels of two batches can be in flight together (one batch's top-K
+// and input layers fill the gaps of the other's GEMM).  ctx().stream is always the selected lane's stream; everything the
+// library launches goes there.  Operations whose effect both lanes must see in order — uploads, clears, device copies,
+// allocation fills, timers — join the lanes around themselves; downloads and dsx_sync wait for both.
+static hipStream_t g_lane_stream[2] = {nullptr, nullptr};
+static hipEvent_t g_lane_event[2] = {nullptr, nullptr};   // [l]: last join point recorded on lane l
+static int g_lane = 0;
+
+namespace dsx {
+int current_lane() { return g_lane; }
+}  // namespace dsx
+
+static hipStream_t other_lane_stream() { return g_lane_stream[g_lane ^ 1]; }
+
+// Work can only be queued on a lane while it is selected, so "the other lane has been selected since this lane last waited
+// for it" is all that has to be tracked: a burst of uploads between two batches then costs one cross-stream wait, not one
+// per call (each is an event record, a wait and a barrier packet between two hardware queues).
+static uint32_t g_lane_selected[2] = {1, 0};   // how often each lane has been selected
+static uint32_t g_lane_seen[2] = {0, 0};       // [l]: g_lane_selected[other] when lane l last waited for the other lane
+static bool g_lane_publish[2] = {false, false};   // [l]: lane l holds ordered work the other lane has not been told to wait for
+
+// The selected lane waits for everything queued so far on the other one.
+static int lanes_join_before()
+{
+    hipStream_t other = other_lane_stream();
+    if (!other) return DSX_OK;
+    const int o = g_lane ^ 1;
+    if (g_lane_seen[g_lane] != g_lane_selected[o]) {
+        DSX_HIP(hipEventRecord(g_lane_event[o], other));
+        DSX_HIP(hipStreamWaitEvent(ctx().stream, g_lane_event[o], 0));
+        g_lane_seen[g_lane] = g_lane_selected[o];
+    }
+    return DSX_OK;
+}
+
+// The other lane must wait for what was just queued on the selected one: arranged when the other lane is selected next.
+static int lanes_join_after()
+{
+    if (other_lane_stream()) g_lane_publish[g_lane] = true;
+    return DSX_OK;
+}
+
+static void lanes_release()
+{
+    // lane 0's stream is ctx().stream's original and is destroyed with the context
+    if (g_lane_stream[1]) hipStreamDestroy(g_lane_stream[1]);
+    for (auto& e : g_lane_event)
+        if (e) hipEventDestroy(e);
+    g_lane_stream[0] = g_lane_stream[1] = nullptr;
+    g_lane_event[0] = g_lane_event[1] = nullptr;
+    g_lane = 0;
+    g_lane_selected[0] = 1;
+    g_lane_selected[1] = 0;
+    g_lane_seen[0] = g_lane_seen[1] = 0;
+    g_lane_publish[0] = g_lane_publish[1] = false;
+}
+
 extern "C" {
 
 const char* dsx_last_error(void) { return g_error; }
@@ -96,7 +153,10 @@ int dsx_shutdown(void)
     Context& c = ctx();
     if (!c.initialized) return DSX_OK;
     if (--c.users > 0) return DSX_OK;
+    if (g_lane_stream[1]) hipStreamSynchronize(g_lane_stream[1]);
+    if (g_lane_stream[0]) c.stream = g_lane_stream[0];
     hipStreamSynchronize(c.stream);
+    lanes_release();
     upload_ring_release();
     {
         std::lock_guard<std::mutex> lock(g_alloc_mutex);
@@ -143,6 +203,36 @@ int dsx_get_memory_usage(int* gpu_kib, int* cpu_kib)
 
 void* dsx_stream(void) { return (void*)ctx().stream; }
 
+int dsx_set_lane(int lane)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(lane == 0 || lane == 1, "dsx_set_lane: lane %d (0 or 1)", lane);
+    if (!g_lane_stream[0]) {
+        if (lane == 0) return DSX_OK;   // nothing to set up until the second lane is asked for
+        g_lane_stream[0] = ctx().stream;
+        DSX_HIP(hipStreamCreateWithFlags(&g_lane_stream[1], hipStreamNonBlocking));
+        for (auto& e : g_lane_event) DSX_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+        // the new lane starts after everything queued so far
+        DSX_HIP(hipEventRecord(g_lane_event[0], g_lane_stream[0]));
+        DSX_HIP(hipStreamWaitEvent(g_lane_stream[1], g_lane_event[0], 0));
+    }
+    if (lane != g_lane) {
+        const int old = g_lane;
+        if (g_lane_publish[old]) {   // ordered work (uploads, clears, copies) of the lane being left: the new lane runs after it
+            DSX_HIP(hipEventRecord(g_lane_event[old], g_lane_stream[old]));
+            DSX_HIP(hipStreamWaitEvent(g_lane_stream[lane], g_lane_event[old], 0));
+            g_lane_publish[old] = false;
+            g_lane_seen[lane] = g_lane_selected[old];
+        }
+        g_lane = lane;
+        g_lane_selected[lane]++;
+        ctx().stream = g_lane_stream[lane];
+    }
+    return DSX_OK;
+}
+
+int dsx_get_lane(void) { return g_lane; }
+
 int dsx_malloc(void** p, size_t bytes)
 {
     DSX_REQUIRE_INIT();
@@ -152,6 +242,7 @@ int dsx_malloc(void** p, size_t bytes)
     hipError_t e = hipMalloc(p, bytes);
     if (e != hipSuccess) return set_error(DSX_ENOMEM, "dsx_malloc: hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
     DSX_HIP(hipMemsetAsync(*p, 0, bytes, ctx().stream));
+    if (int rc = lanes_join_after()) return rc;
     std::lock_guard<std::mutex> lock(g_alloc_mutex);
     g_device_allocs[*p] = bytes;
     ctx().gpu_bytes += bytes;
@@ -219,8 +310,9 @@ int dsx_memset(void* p, int value, size_t bytes)
     DSX_REQUIRE_INIT();
     if (bytes == 0) return DSX_OK;
     DSX_CHECK_ARG(p, "dsx_memset: null pointer");
+    if (int rc = lanes_join_before()) return rc;
     DSX_HIP(hipMemsetAsync(p, value, bytes, ctx().stream));
-    return DSX_OK;
+    return lanes_join_after();
 }
 
 int dsx_memcpy_h2d(void* dst, const void* src, size_t bytes)
@@ -228,10 +320,12 @@ int dsx_memcpy_h2d(void* dst, const void* src, size_t bytes)
     DSX_REQUIRE_INIT();
     if (bytes == 0) return DSX_OK;
     DSX_CHECK_ARG(dst && src, "dsx_memcpy_h2d: null pointer");
+    // the destination may still be read by kernels of the other lane, and is read by whatever either lane runs next
+    if (int rc = lanes_join_before()) return rc;
     if (bytes > kUploadSlotBytes) {
         DSX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx().stream));
         DSX_HIP(hipStreamSynchronize(ctx().stream));   // src may be pageable: wait until it has been read
-        return DSX_OK;
+        return lanes_join_after();
     }
     std::lock_guard<std::mutex> lock(g_alloc_mutex);
     const int slot = g_upload_next;
@@ -245,7 +339,7 @@ int dsx_memcpy_h2d(void* dst, const void* src, size_t bytes)
     DSX_HIP(hipMemcpyAsync(dst, g_upload_host[slot], bytes, hipMemcpyHostToDevice, ctx().stream));
     DSX_HIP(hipEventRecord(g_upload_done[slot], ctx().stream));
     g_upload_busy[slot] = true;
-    return DSX_OK;
+    return lanes_join_after();
 }
 
 int dsx_memcpy_d2h(void* dst, const void* src, size_t bytes)
@@ -253,6 +347,7 @@ int dsx_memcpy_d2h(void* dst, const void* src, size_t bytes)
     DSX_REQUIRE_INIT();
     if (bytes == 0) return DSX_OK;
     DSX_CHECK_ARG(dst && src, "dsx_memcpy_d2h: null pointer");
+    if (other_lane_stream()) DSX_HIP(hipStreamSynchronize(other_lane_stream()));   // the data may come from either lane
     DSX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx().stream));
     DSX_HIP(hipStreamSynchronize(ctx().stream));
     return DSX_OK;
@@ -263,27 +358,45 @@ int dsx_memcpy_d2d(void* dst, const void* src, size_t bytes)
     DSX_REQUIRE_INIT();
     if (bytes == 0) return DSX_OK;
     DSX_CHECK_ARG(dst && src, "dsx_memcpy_d2d: null pointer");
+    if (int rc = lanes_join_before()) return rc;
     DSX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx().stream));
-    return DSX_OK;
+    return lanes_join_after();
 }
 
 int dsx_sync(void)
 {
     DSX_REQUIRE_INIT();
+    if (other_lane_stream()) DSX_HIP(hipStreamSynchronize(other_lane_stream()));
     DSX_HIP(hipStreamSynchronize(ctx().stream));
+    return DSX_OK;
+}
+
+// Downloads that wait for one lane only: a caller that keeps two batches in flight reads one batch's results while the
+// other batch runs.
+int dsx_memcpy_d2h_lane(int lane, void* dst, const void* src, size_t bytes)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(lane == 0 || lane == 1, "dsx_memcpy_d2h_lane: lane %d (0 or 1)", lane);
+    if (bytes == 0) return DSX_OK;
+    DSX_CHECK_ARG(dst && src, "dsx_memcpy_d2h_lane: null pointer");
+    hipStream_t s = g_lane_stream[lane] ? g_lane_stream[lane] : ctx().stream;
+    DSX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s));
+    DSX_HIP(hipStreamSynchronize(s));
     return DSX_OK;
 }
 
 int dsx_timer_start(void)
 {
     DSX_REQUIRE_INIT();
+    if (int rc = lanes_join_before()) return rc;
     DSX_HIP(hipEventRecord(ctx().ev_start, ctx().stream));
-    return DSX_OK;
+    return lanes_join_after();
 }
 
 int dsx_timer_stop(float* elapsed_ms)
 {
     DSX_REQUIRE_INIT();
+    if (int rc = lanes_join_before()) return rc;
     DSX_HIP(hipEventRecord(ctx().ev_stop, ctx().stream));
     DSX_HIP(hipEventSynchronize(ctx().ev_stop));
     float ms = 0.0f;

@@ -902,21 +902,25 @@ __global__ __launch_bounds__(256) void topk_gather_kernel(const V* in_values, V*
     values[pos] = (j < width) ? in_values[(uint64_t)b * width + col] : (V)0;
 }
 
-static uint64_t* g_partial = nullptr;
-static size_t g_partial_bytes = 0;
+static uint64_t* g_partial_of[2] = {nullptr, nullptr};   // per lane: two lanes may run a split top-K at the same time
+static size_t g_partial_bytes_of[2] = {0, 0};
 
-static int ensure_partial(size_t bytes)
+static int ensure_partial(size_t bytes, uint64_t** out)
 {
-    if (bytes <= g_partial_bytes) return DSX_OK;
-    if (g_partial) {
-        DSX_HIP(hipStreamSynchronize(ctx().stream));
-        DSX_HIP(hipFree(g_partial));
-        g_partial = nullptr;
-        g_partial_bytes = 0;
+    uint64_t*& buf = g_partial_of[current_lane()];
+    size_t& have = g_partial_bytes_of[current_lane()];
+    if (bytes > have) {
+        if (buf) {
+            DSX_HIP(hipStreamSynchronize(ctx().stream));
+            DSX_HIP(hipFree(buf));
+            buf = nullptr;
+            have = 0;
+        }
+        hipError_t e = hipMalloc((void**)&buf, bytes);
+        if (e != hipSuccess) return set_error(DSX_ENOMEM, "top-K: cannot allocate %zu bytes for partial lists: %s", bytes, hipGetErrorString(e));
+        have = bytes;
     }
-    hipError_t e = hipMalloc((void**)&g_partial, bytes);
-    if (e != hipSuccess) return set_error(DSX_ENOMEM, "top-K: cannot allocate %zu bytes for partial lists: %s", bytes, hipGetErrorString(e));
-    g_partial_bytes = bytes;
+    *out = buf;
     return DSX_OK;
 }
 
@@ -985,9 +989,10 @@ int topk_run(const float* in, uint32_t pitch, uint32_t width, uint32_t batch, ui
         a.partial_slots = partial_slots;
         a.partial_slot0 = partial_slot0;
     } else if (a.segments > 1) {
-        int rc = ensure_partial((size_t)batch * a.segments * k * sizeof(uint64_t));
+        uint64_t* scratch = nullptr;
+        int rc = ensure_partial((size_t)batch * a.segments * k * sizeof(uint64_t), &scratch);
         if (rc) return rc;
-        a.partial = g_partial;
+        a.partial = scratch;
         a.partial_slots = a.segments;
         a.partial_slot0 = 0;
     }

@@ -64,6 +64,19 @@ private:
     // (_segWidth == 0: none): NNNetwork::CalculateTopK then reads only the segments that can hold a result.
     unique_ptr<GpuBuffer<NNFloat>> _pbSegMax;
     uint32_t _segWidth = 0;
+    // With two lanes (NNNetwork::SetLanes) every layer has a second set of the three members above: the batch before the
+    // current one may still be running on the other lane's stream.  SwapLane exchanges the sets, so that the names above
+    // always denote the current batch's buffers.
+    unique_ptr<GpuBuffer<NNFloat>> _pbUnitOther;
+    unique_ptr<GpuBuffer<NNFloat>> _pbSegMaxOther;
+    uint32_t _segWidthOther = 0;
+    uint32_t _lanes = 1;
+    void SwapLane()
+    {
+        _pbUnit.swap(_pbUnitOther);
+        _pbSegMax.swap(_pbSegMaxOther);
+        std::swap(_segWidth, _segWidthOther);
+    }
     int32_t _priority;
 
     NNLayer(NNLayerDescriptor& l, uint32_t batch);

@@ -45,6 +45,8 @@ private:
     map<string, NNLayer*> _mLayer;
     bool _bDirty;
     bool _verbose;
+    uint32_t _lanes;                            // 1: one set of unit buffers, one stream; 2: consecutive batches alternate
+    uint32_t _lane;                             // the lane of the current batch
 
     NNNetwork(NNNetworkDescriptor& nd, uint32_t batch = DefaultBatch);
     void CalculatePropagationOrder();
@@ -69,6 +71,13 @@ public:
     void CalculateFilteredTopK(const string& layer, uint32_t k, NNDataSetBase* pFilter, GpuBuffer<NNFloat>* pbKey,
                                GpuBuffer<uint32_t>* pbValue, bool bUseValues = false);
     void SetBatch(uint32_t batch);
+    // No counterpart in the reference.  With two lanes (the default) consecutive PredictBatch calls alternate between two sets
+    // of unit buffers and two device streams: a batch's kernels (and the top-K calls that follow its PredictBatch) overlap
+    // with those of the batch before it.  Everything read back through this API waits as needed; a device pointer obtained
+    // from GetUnitBuffer belongs to the batch predicted last.  One lane restores single buffers.
+    bool SetLanes(uint32_t lanes);
+    uint32_t GetLanes() const { return _lanes; }
+    uint32_t GetLane() const { return _lane; }
     void Randomize();                           // every connection back to its starting values (engine/NNNetwork.cpp:675-679)
     void SetPosition(uint32_t position);
     void SetShuffleIndices(bool bShuffleIndices);

@@ -29,23 +29,34 @@ DsstneContext::DsstneContext(const string& networkFilename, uint32_t batchSize, 
             size_t outputBufferLength = (size_t)maxK * batchSize;
             printf("DsstneContext::DsstneContext: Allocating output score and index buffers, each of size %zu for output layer %s\n",
                    outputBufferLength, layerName.c_str());
-            dOutputScores[layerName] = new GpuBuffer<NNFloat>(outputBufferLength, false, false);
-            dOutputIndexes[layerName] = new GpuBuffer<uint32_t>(outputBufferLength, false, false);
+            for (int lane = 0; lane < 2; lane++) {
+                dOutputScores[lane][layerName] = new GpuBuffer<NNFloat>(outputBufferLength, false, false);
+                dOutputIndexes[lane][layerName] = new GpuBuffer<uint32_t>(outputBufferLength, false, false);
+            }
         }
     }
 }
 
-GpuBuffer<NNFloat>* DsstneContext::getOutputScoresBuffer(const std::string& layerName) { return dOutputScores.at(layerName); }
+// The buffers of the batch predicted last (the network's current lane).
+GpuBuffer<NNFloat>* DsstneContext::getOutputScoresBuffer(const std::string& layerName)
+{
+    return dOutputScores[getNetwork() ? getNetwork()->GetLane() : 0].at(layerName);
+}
 
-GpuBuffer<uint32_t>* DsstneContext::getOutputIndexesBuffer(const std::string& layerName) { return dOutputIndexes.at(layerName); }
+GpuBuffer<uint32_t>* DsstneContext::getOutputIndexesBuffer(const std::string& layerName)
+{
+    return dOutputIndexes[getNetwork() ? getNetwork()->GetLane() : 0].at(layerName);
+}
 
 DsstneContext::~DsstneContext()
 {
     const string networkName = getNetwork() ? getNetwork()->GetName() : string("<none>");
-    for (const auto& kv : dOutputScores) delete kv.second;
-    for (const auto& kv : dOutputIndexes) delete kv.second;
-    dOutputScores.clear();
-    dOutputIndexes.clear();
+    for (int lane = 0; lane < 2; lane++) {
+        for (const auto& kv : dOutputScores[lane]) delete kv.second;
+        for (const auto& kv : dOutputIndexes[lane]) delete kv.second;
+        dOutputScores[lane].clear();
+        dOutputIndexes[lane].clear();
+    }
     delete getNetwork();
     for (auto d : ownedDataSets) delete d;
     ownedDataSets.clear();

@@ -62,6 +62,9 @@ void NNLayer::Deallocate()
     _pbUnit.reset();
     _pbSegMax.reset();
     _segWidth = 0;
+    _pbUnitOther.reset();
+    _pbSegMaxOther.reset();
+    _segWidthOther = 0;
 }
 
 void NNLayer::SetBatch(uint32_t batch)
@@ -80,8 +83,9 @@ void NNLayer::Allocate(bool validate)
     // hidden and output layers, dense inputs and sparse inputs that cannot use the sparse-Z path own an activation buffer
     if (!_bSparse || !_bFastSparse || (_kind != Input) || (_bSparse && (_kind == Input) && validate)) {
         _pbUnit.reset(new GpuBuffer<NNFloat>(size));
-        printf("NNLayer::Allocate: Allocating %" PRIu64 " bytes (%u, %u) of unit data for layer %s\n", size * sizeof(NNFloat), _maxLocalStride,
-               _localBatch, _name.c_str());
+        if (_lanes > 1) _pbUnitOther.reset(new GpuBuffer<NNFloat>(size));
+        printf("NNLayer::Allocate: Allocating %" PRIu64 " bytes (%u, %u) of unit data for layer %s%s\n", size * sizeof(NNFloat), _maxLocalStride,
+               _localBatch, _name.c_str(), _lanes > 1 ? ", twice (two lanes)" : "");
     }
     _bDirty = false;
 }

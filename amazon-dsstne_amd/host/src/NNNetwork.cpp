@@ -38,7 +38,7 @@ static void fatal(const char* fmt, const char* a = "", const char* b = "")
 NNNetwork::NNNetwork(NNNetworkDescriptor& d, uint32_t batch)
     : _name(d._name), _batch(batch), _position(0), _bExamplesFound(false), _bAllDataLoaded(true), _examples(0), _kind(d._kind),
       _errorFunction(d._errorFunction), _mode(Prediction), _bShuffleIndices(d._bShuffleIndices), _pDescriptor(NULL), _bDirty(true),
-      _verbose(false)
+      _verbose(false), _lanes(2), _lane(0)
 {
     // keep the scalar settings (not the weight payloads) for SaveNetCDF round trips
     _pDescriptor = new NNNetworkDescriptor(d);
@@ -51,6 +51,7 @@ NNNetwork::NNNetwork(NNNetworkDescriptor& d, uint32_t batch)
             fatal("NNNetwork::NNNetwork: layer %s is not fully connected; convolutional and pooling layers are not supported by this build.",
                   l._name.c_str());
         NNLayer* pLayer = new NNLayer(l, batch);
+        pLayer->_lanes = _lanes;
         // layers without their own slope / alpha / lambda take the network defaults
         if (std::isnan(pLayer->_RELUSlope)) pLayer->_RELUSlope = d._RELUSlope;
         if (std::isnan(pLayer->_ELUAlpha)) pLayer->_ELUAlpha = d._ELUAlpha;
@@ -144,6 +145,7 @@ NNNetwork::~NNNetwork()
     for (auto l : _vLayer) delete l;
     delete _pDescriptor;
     if (getGpu()._pNetwork == this) getGpu()._pNetwork = NULL;
+    if (dsx_is_initialized()) dsx_set_lane(0);   // whatever runs next starts on the first lane (deleting the buffers above waited for both)
 }
 
 // Forward order: every layer's priority is its longest distance from an input; a stable ordering by priority follows.
@@ -269,11 +271,36 @@ void NNNetwork::PredictBatch(uint32_t layers)
             exit(-1);
         }
     }
+    if (_lanes > 1) {
+        // this batch takes the lane the batch before the last one used
+        _lane ^= 1;
+        for (auto l : _vLayer) l->SwapLane();
+        dsxFatal(dsx_set_lane((int)_lane), "NNNetwork::PredictBatch: lane");
+    }
     uint32_t batch = _batch;
     if (_position + batch > _examples) batch = _examples - _position;
     ClearUpdates();
     LoadBatch();
     for (auto l : _vFPOrder) l->ForwardPropagate(_position, batch, false);
+}
+
+bool NNNetwork::SetLanes(uint32_t lanes)
+{
+    if (lanes < 1 || lanes > 2) {
+        printf("NNNetwork::SetLanes: %u lanes requested (1 or 2).\n", lanes);
+        return false;
+    }
+    if (lanes == _lanes) return true;
+    dsxFatal(dsx_sync(), "NNNetwork::SetLanes");
+    _lanes = lanes;
+    _lane = 0;
+    dsxFatal(dsx_set_lane(0), "NNNetwork::SetLanes");
+    for (auto l : _vLayer) {
+        l->_lanes = lanes;
+        l->_bDirty = true;   // unit buffers are allocated anew
+    }
+    _bDirty = true;
+    return true;
 }
 
 void NNNetwork::CalculateTopK(const string& layer, uint32_t k, GpuBuffer<NNFloat>* pbKey, GpuBuffer<uint32_t>* pbValue)

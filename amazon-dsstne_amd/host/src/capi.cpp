@@ -27,12 +27,12 @@ struct dsstne_context {
     int maxK = 0;
     map<string, NNDataSetBase*> datasets;
     vector<NNDataSetBase*> pending;
-    map<string, GpuBuffer<NNFloat>*> scores;
-    map<string, GpuBuffer<uint32_t>*> indexes;
+    map<string, GpuBuffer<NNFloat>*> scores[2];      // per lane of the network
+    map<string, GpuBuffer<uint32_t>*> indexes[2];
 
     NNNetwork* net() const { return dc ? dc->getNetwork() : network; }
-    GpuBuffer<NNFloat>* scoreBuf(const string& layer) { return dc ? dc->getOutputScoresBuffer(layer) : scores.at(layer); }
-    GpuBuffer<uint32_t>* indexBuf(const string& layer) { return dc ? dc->getOutputIndexesBuffer(layer) : indexes.at(layer); }
+    GpuBuffer<NNFloat>* scoreBuf(const string& layer) { return dc ? dc->getOutputScoresBuffer(layer) : scores[network->GetLane()].at(layer); }
+    GpuBuffer<uint32_t>* indexBuf(const string& layer) { return dc ? dc->getOutputIndexesBuffer(layer) : indexes[network->GetLane()].at(layer); }
 };
 
 #define CAPI_TRY try {
@@ -56,8 +56,10 @@ static void makeResultBuffers(dsstne_context* c)
     if (c->maxK <= 0) return;
     vector<const NNLayer*> outs;
     for (auto it = c->network->GetLayers(NNLayer::Kind::Output, outs); it != outs.end(); ++it) {
-        c->scores[(*it)->GetName()] = new GpuBuffer<NNFloat>((size_t)c->maxK * c->batch);
-        c->indexes[(*it)->GetName()] = new GpuBuffer<uint32_t>((size_t)c->maxK * c->batch);
+        for (int lane = 0; lane < 2; lane++) {
+            c->scores[lane][(*it)->GetName()] = new GpuBuffer<NNFloat>((size_t)c->maxK * c->batch);
+            c->indexes[lane][(*it)->GetName()] = new GpuBuffer<uint32_t>((size_t)c->maxK * c->batch);
+        }
     }
 }
 
@@ -196,8 +198,10 @@ int dsstne_set_weights(dsstne_context* c, const char* input_layer, const char* o
 void dsstne_shutdown(dsstne_context* c)
 {
     if (!c) return;
-    for (auto& kv : c->scores) delete kv.second;
-    for (auto& kv : c->indexes) delete kv.second;
+    for (int lane = 0; lane < 2; lane++) {
+        for (auto& kv : c->scores[lane]) delete kv.second;
+        for (auto& kv : c->indexes[lane]) delete kv.second;
+    }
     if (c->dc) {
         delete c->dc;   // deletes its network and datasets, shuts the device down
     } else {
@@ -352,6 +356,27 @@ int dsstne_get_topk(dsstne_context* c, const char* layer, uint32_t rows, uint32_
     dsxFatal(dsx_memcpy_d2h(scores, c->scoreBuf(layer)->_pDevData, (size_t)rows * k * sizeof(float)), "dsstne_get_topk");
     dsxFatal(dsx_memcpy_d2h(indexes, c->indexBuf(layer)->_pDevData, (size_t)rows * k * sizeof(uint32_t)), "dsstne_get_topk");
     return 0;
+    CAPI_CATCH(-1)
+}
+
+int dsstne_get_topk_previous(dsstne_context* c, const char* layer, uint32_t rows, uint32_t k, float* scores, uint32_t* indexes)
+{
+    CAPI_TRY
+    NNNetwork* n = c->net();
+    if (n->GetLanes() < 2) return fail("dsstne_get_topk_previous: the network runs on one lane");
+    const int lane = (int)(n->GetLane() ^ 1u);
+    GpuBuffer<NNFloat>* s = c->dc ? c->dc->getOutputScoresBuffer(layer, lane) : c->scores[lane].at(layer);
+    GpuBuffer<uint32_t>* i = c->dc ? c->dc->getOutputIndexesBuffer(layer, lane) : c->indexes[lane].at(layer);
+    dsxFatal(dsx_memcpy_d2h_lane(lane, scores, s->_pDevData, (size_t)rows * k * sizeof(float)), "dsstne_get_topk_previous");
+    dsxFatal(dsx_memcpy_d2h_lane(lane, indexes, i->_pDevData, (size_t)rows * k * sizeof(uint32_t)), "dsstne_get_topk_previous");
+    return 0;
+    CAPI_CATCH(-1)
+}
+
+int dsstne_set_lanes(dsstne_context* c, uint32_t lanes)
+{
+    CAPI_TRY
+    return c->net()->SetLanes(lanes) ? 0 : fail("dsstne_set_lanes: %u lanes (1 or 2)", lanes);
     CAPI_CATCH(-1)
 }
 

@@ -40,6 +40,8 @@ SIGNATURES = {
     "dsstne_load_definition": ([_cp, _cp, _u32, _int, C.c_uint64], _vp),
     "dsstne_get_weights": ([_vp, _cp, _cp, _vp, C.c_size_t, _vp, C.c_size_t], _int),
     "dsstne_set_weights": ([_vp, _cp, _cp, _vp, C.c_size_t, _vp, C.c_size_t], _int),
+    "dsstne_get_topk_previous": ([_vp, _cp, _u32, _u32, _vp, _vp], _int),
+    "dsstne_set_lanes": ([_vp, _u32], _int),
     "dsstne_knn_create_typed": ([_u32, _u32, _cp], _vp),
     "dsstne_knn_search": ([_vp, _u32, _vp, _u32, _vp, _vp], _int),
     "dsstne_knn_elapsed": ([_vp, C.POINTER(_f32), C.POINTER(_f32)], _int),
@@ -139,6 +141,17 @@ class Network:
         idx = np.empty((rows, k), dtype=np.uint32)
         _check(self.lib.dsstne_get_topk(self.ctx, layer.encode(), rows, k, scores.ctypes.data, idx.ctypes.data))
         return scores, idx
+
+    def get_topk_previous(self, rows, k=None, layer="Output"):
+        """Results of the batch before the current one (two lanes): waits for that batch only."""
+        k = k or self.p.k
+        scores = np.empty((rows, k), dtype=np.float32)
+        idx = np.empty((rows, k), dtype=np.uint32)
+        _check(self.lib.dsstne_get_topk_previous(self.ctx, layer.encode(), rows, k, scores.ctypes.data, idx.ctypes.data))
+        return scores, idx
+
+    def set_lanes(self, lanes):
+        _check(self.lib.dsstne_set_lanes(self.ctx, lanes))
 
     def units(self, layer="Output", rows=None, width=None):
         width = width or self.p.widths[-1]

@@ -98,9 +98,29 @@ def network_bench(args, pkg, lib):
     t1 = time.perf_counter()
     ms_step = (t1 - t0) * 1e3 / args.steps
 
+    # The step above runs as NNNetwork does by default: consecutive batches alternate between two lanes (two sets of unit
+    # buffers on two streams), so one batch's input layers and top-K overlap with the next one's GEMM.  The same on one
+    # lane — the reference's single set of buffers, one batch's kernels strictly after the other's — for comparison.
+    net.set_lanes(1)
+    for _ in range(max(2, args.warmup // 4)):
+        step()
+    net.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    net.sync()
+    ms_one_lane = (time.perf_counter() - t0) * 1e3 / args.steps
+    net.set_lanes(2)
+    step()
+    net.sync()
+
     # The same step when the batch's CSR arrays are handed over as host buffers every time (NNDataSet::LoadSparseData, as the
     # reference's JNI predict does): never `value`, reported beside it.
     up_steps = max(5, min(50, args.steps))
+    for _ in range(4):   # untimed: the first uploads allocate the pinned staging buffers
+        net.load_sparse(p.start, p.end, p.sparse_data, p.sparse_index)
+        step()
+    net.sync()
     t0 = time.perf_counter()
     for _ in range(up_steps):
         net.load_sparse(p.start, p.end, p.sparse_data, p.sparse_index)
@@ -218,6 +238,8 @@ def network_bench(args, pkg, lib):
         "roofline": roofline,
         "kernels": {n: {k: (round(v, 5) if isinstance(v, float) else v) for k, v in kv.items()} for n, kv in kernels.items()},
         "cpu_baseline": cpu,
+        "one_lane": {"ms_per_step": round(ms_one_lane, 5), "value": round(B / (ms_one_lane / 1e3), 1), "unit": "samples/s",
+                     "note": "NNNetwork::SetLanes(1): one set of buffers, one stream, batches strictly one after the other"},
         "with_input_upload": {"ms_per_step": round(ms_upload, 5), "value": round(B / (ms_upload / 1e3), 1), "unit": "samples/s",
                               "note": "host CSR arrays of the whole dataset copied and uploaded before every step (PCIe-inclusive)"},
     }

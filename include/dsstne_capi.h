@@ -80,6 +80,13 @@ int dsstne_predict_batch(dsstne_context* ctx, uint32_t position);
 int dsstne_topk(dsstne_context* ctx, const char* layer, uint32_t k, const char* filter_dataset);
 /* Copies the last top-K results to the host: scores/indexes are [rows][k]. */
 int dsstne_get_topk(dsstne_context* ctx, const char* layer, uint32_t rows, uint32_t k, float* scores, uint32_t* indexes);
+/* No counterpart in the reference.  A network runs on two lanes by default: consecutive dsstne_predict_batch calls alternate
+ * between two sets of unit and result buffers on two device streams, so a batch's kernels overlap with those of the batch
+ * before it (NNNetwork::SetLanes).  dsstne_get_topk reads the batch predicted last; dsstne_get_topk_previous the one before
+ * it, waiting for that batch only — a loop that issues batch i+1 and then collects batch i keeps the device busy.
+ * dsstne_set_lanes(ctx, 1) goes back to one set of buffers and one stream. */
+int dsstne_get_topk_previous(dsstne_context* ctx, const char* layer, uint32_t rows, uint32_t k, float* scores, uint32_t* indexes);
+int dsstne_set_lanes(dsstne_context* ctx, uint32_t lanes);
 /* Dsstne.predict in one call: position 0, predict, unfiltered (filter_dataset NULL) or filtered top-k, copy back. */
 int dsstne_predict(dsstne_context* ctx, const char* layer, uint32_t k, const char* filter_dataset, float* scores, uint32_t* indexes);
 /* NNLayer::GetUnits: the layer's [batch][width] activations. */

@@ -114,7 +114,14 @@ int dsx_memset(void* device_ptr, int value, size_t bytes);
 int dsx_memcpy_h2d(void* device_dst, const void* host_src, size_t bytes);
 int dsx_memcpy_d2h(void* host_dst, const void* device_src, size_t bytes);   /* GpuBuffer::Download */
 int dsx_memcpy_d2d(void* device_dst, const void* device_src, size_t bytes); /* GpuBuffer::Copy     */
-int dsx_sync(void);
+int dsx_sync(void);                                                          /* waits for both lanes */
+/* No counterpart in the reference (which runs everything on the default stream with blocking copies): the library has two
+ * lanes, each an in-order stream; whatever is launched goes to the selected one (lane 0 until told otherwise).  Two batches
+ * issued on different lanes run concurrently; uploads, clears, device-to-device copies and timers order both lanes around
+ * themselves, dsx_memcpy_d2h and dsx_sync wait for both, dsx_memcpy_d2h_lane for one lane only. */
+int dsx_set_lane(int lane);
+int dsx_get_lane(void);
+int dsx_memcpy_d2h_lane(int lane, void* host_dst, const void* device_src, size_t bytes);
 
 /* Event timing on the library stream (the reference keeps cudaEvent timings for KNN, knn/KnnExactGpu.cu:130-148). */
 int dsx_timer_start(void);

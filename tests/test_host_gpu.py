@@ -310,3 +310,77 @@ def test_knn_api_fp16_storage(pkg, dsx, orc, synth):
         assert np.abs(scores - np.take_along_axis(exact, idx.astype(np.int64), axis=1)).max() > 1e-5
     finally:
         lib.dsstne_knn_destroy(knn)
+
+
+def reference_batches(orc, p, positions):
+    out = []
+    for pos in positions:
+        rows = min(p.batch, p.examples - pos)
+        _, unit, _, _ = orc.forward(p, pos, rows, filtered=False, want_unit=True, want_topk=False)
+        _, _, keys, idx = orc.forward(p, pos, rows, filtered=True)
+        scores = unit.copy()
+        orc.lib().orc_apply_filter(scores.ctypes.data, rows, scores.shape[1], 0, pos, None, p.start.ctypes.data, p.end.ctypes.data,
+                                   p.sparse_index.ctypes.data, None)
+        out.append((rows, keys, idx, scores))
+    return out
+
+
+@pytest.mark.parametrize("config,batches", [(1, 7), (2, 3)])
+def test_two_lanes_keep_batches_apart(pkg, dsx, orc, synth, config, batches):
+    """Consecutive PredictBatch calls alternate between two sets of buffers on two streams (NNNetwork::SetLanes).  A loop that
+    issues batch i+1 before it collects batch i must get every batch's own results; the last batch is short."""
+    from amazon_dsstne_amd import host_api
+    p = synth.config(config, batches=batches)
+    short = p.batch // 3
+    p.examples -= short
+    p.unique_examples -= short
+    p.start, p.end = p.start[:p.examples], p.end[:p.examples]
+    positions = list(range(0, p.examples, p.batch))
+    want = reference_batches(orc, p, positions)
+    net = host_api.Network(p, max_k=p.k)
+    try:
+        net.bind_input()
+        got = []
+        for n, pos in enumerate(positions):
+            net.predict_batch(pos)
+            net.topk(p.k, filter_dataset="input")
+            if n > 0:
+                got.append(net.get_topk_previous(want[n - 1][0]))       # the batch before, while this one runs
+        got.append(net.get_topk(want[-1][0]))
+        for n, ((rows, keys, idx, scores), (gk, gi)) in enumerate(zip(want, got)):
+            assert_topk_parity(gk, gi, keys, idx, scores, "%s batch %d on two lanes" % (p.name, n))
+        # many batches in flight without reading anything back, then the last two
+        for rep in range(3):
+            for pos in positions:
+                net.predict_batch(pos)
+                net.topk(p.k, filter_dataset="input")
+        gk, gi = net.get_topk(want[-1][0])
+        assert_topk_parity(gk, gi, want[-1][1], want[-1][2], want[-1][3], p.name + " last batch after a run")
+        gk, gi = net.get_topk_previous(want[-2][0])
+        assert_topk_parity(gk, gi, want[-2][1], want[-2][2], want[-2][3], p.name + " batch before the last after a run")
+        # units of the current batch, and a new input upload between batches (orders both lanes)
+        net.predict_batch(positions[1])
+        unit = net.units(rows=p.batch)
+        _, ref_unit, _, _ = orc.forward(p, positions[1], p.batch, filtered=False, want_unit=True, want_topk=False)
+        assert_close(unit, ref_unit, p.name + " units on two lanes", rel=1e-4, abs_floor=1e-3)
+        net.load_sparse(p.start, p.end, p.sparse_data, p.sparse_index)
+        net.predict_batch(positions[0])
+        net.topk(p.k, filter_dataset="input")
+        gk, gi = net.get_topk(want[0][0])
+        assert_topk_parity(gk, gi, want[0][1], want[0][2], want[0][3], p.name + " after a reload")
+        # one lane: the reference's single set of buffers
+        net.set_lanes(1)
+        with pytest.raises(host_api.DsxError):
+            net.get_topk_previous(1)
+        for n, pos in enumerate(positions[:2]):
+            net.predict_batch(pos)
+            net.topk(p.k, filter_dataset="input")
+            gk, gi = net.get_topk(want[n][0])
+            assert_topk_parity(gk, gi, want[n][1], want[n][2], want[n][3], "%s batch %d on one lane" % (p.name, n))
+        net.set_lanes(2)
+        net.predict_batch(positions[0])
+        net.topk(p.k, filter_dataset="input")
+        gk, gi = net.get_topk(want[0][0])
+        assert_topk_parity(gk, gi, want[0][1], want[0][2], want[0][3], p.name + " back on two lanes")
+    finally:
+        net.close()
