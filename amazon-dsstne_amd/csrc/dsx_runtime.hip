@@ -43,8 +43,22 @@ static hipEvent_t g_upload_done[kUploadSlots] = {};
 static bool g_upload_busy[kUploadSlots] = {};
 static int g_upload_next = 0;
 
+// Downloads of up to kUploadSlotBytes land in a pinned buffer first and are copied to the caller's memory by the host: a copy
+// straight into pageable memory costs the runtime a staging round trip of its own that is several times slower.
+static char* g_download_host = nullptr;
+
+static int download_small(void* dst, const void* src, size_t bytes, hipStream_t s, size_t slot_offset)
+{
+    if (!g_download_host) DSX_HIP(hipHostMalloc((void**)&g_download_host, kUploadSlotBytes, hipHostMallocDefault));
+    DSX_HIP(hipMemcpyAsync(g_download_host + slot_offset, src, bytes, hipMemcpyDeviceToHost, s));
+    (void)dst;
+    return DSX_OK;
+}
+
 static void upload_ring_release()
 {
+    if (g_download_host) hipHostFree(g_download_host);
+    g_download_host = nullptr;
     for (int i = 0; i < kUploadSlots; i++) {
         if (g_upload_host[i]) hipHostFree(g_upload_host[i]);
         if (g_upload_done[i]) hipEventDestroy(g_upload_done[i]);
@@ -348,7 +362,36 @@ int dsx_memcpy_d2h(void* dst, const void* src, size_t bytes)
     if (bytes == 0) return DSX_OK;
     DSX_CHECK_ARG(dst && src, "dsx_memcpy_d2h: null pointer");
     if (other_lane_stream()) DSX_HIP(hipStreamSynchronize(other_lane_stream()));   // the data may come from either lane
+    if (bytes <= kUploadSlotBytes) {
+        std::lock_guard<std::mutex> lock(g_alloc_mutex);
+        if (int rc = download_small(dst, src, bytes, ctx().stream, 0)) return rc;
+        DSX_HIP(hipStreamSynchronize(ctx().stream));
+        memcpy(dst, g_download_host, bytes);
+        return DSX_OK;
+    }
     DSX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx().stream));
+    DSX_HIP(hipStreamSynchronize(ctx().stream));
+    return DSX_OK;
+}
+
+// Two downloads with one wait (a top-K's scores and indexes): the second copy does not pay a round trip of its own.
+int dsx_memcpy_d2h_pair(void* dst0, const void* src0, size_t bytes0, void* dst1, const void* src1, size_t bytes1)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG((bytes0 == 0 || (dst0 && src0)) && (bytes1 == 0 || (dst1 && src1)), "dsx_memcpy_d2h_pair: null pointer");
+    if (other_lane_stream()) DSX_HIP(hipStreamSynchronize(other_lane_stream()));   // the data may come from either lane
+    const size_t off1 = (bytes0 + 255) / 256 * 256;
+    if (off1 + bytes1 <= kUploadSlotBytes) {
+        std::lock_guard<std::mutex> lock(g_alloc_mutex);
+        if (bytes0) if (int rc = download_small(dst0, src0, bytes0, ctx().stream, 0)) return rc;
+        if (bytes1) if (int rc = download_small(dst1, src1, bytes1, ctx().stream, off1)) return rc;
+        DSX_HIP(hipStreamSynchronize(ctx().stream));
+        if (bytes0) memcpy(dst0, g_download_host, bytes0);
+        if (bytes1) memcpy(dst1, g_download_host + off1, bytes1);
+        return DSX_OK;
+    }
+    if (bytes0) DSX_HIP(hipMemcpyAsync(dst0, src0, bytes0, hipMemcpyDeviceToHost, ctx().stream));
+    if (bytes1) DSX_HIP(hipMemcpyAsync(dst1, src1, bytes1, hipMemcpyDeviceToHost, ctx().stream));
     DSX_HIP(hipStreamSynchronize(ctx().stream));
     return DSX_OK;
 }
@@ -380,6 +423,13 @@ int dsx_memcpy_d2h_lane(int lane, void* dst, const void* src, size_t bytes)
     if (bytes == 0) return DSX_OK;
     DSX_CHECK_ARG(dst && src, "dsx_memcpy_d2h_lane: null pointer");
     hipStream_t s = g_lane_stream[lane] ? g_lane_stream[lane] : ctx().stream;
+    if (bytes <= kUploadSlotBytes) {
+        std::lock_guard<std::mutex> lock(g_alloc_mutex);
+        if (int rc = download_small(dst, src, bytes, s, 0)) return rc;
+        DSX_HIP(hipStreamSynchronize(s));
+        memcpy(dst, g_download_host, bytes);
+        return DSX_OK;
+    }
     DSX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s));
     DSX_HIP(hipStreamSynchronize(s));
     return DSX_OK;

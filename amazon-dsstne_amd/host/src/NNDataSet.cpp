@@ -204,8 +204,22 @@ template <typename T>
 void NNDataSet<T>::LoadSparseData(const uint64_t* srcSparseStart, const uint64_t* srcSparseEnd, const void* srcSparseData,
                                   const uint32_t* srcSparseIndex)
 {
+    if (!(_attributes & NNDataSetEnums::Attributes::Sparse)) throw std::runtime_error("Cannot set sparse data on a non sparse NNDataSet");
+    checkSparseLoad(srcSparseStart[0], srcSparseEnd[_uniqueExamples - 1]);
+    // The device copies are queued first, straight from the caller's arrays and only as long as this batch's data (the
+    // buffers may be larger): the device starts on them while the host shadows below are still being filled.
+    const uint64_t dataLength = srcSparseEnd[_uniqueExamples - 1];
+    const bool direct = _pbSparseStart && _pbSparseEnd && _pbSparseIndex && _pbSparseStart->_length >= _uniqueExamples &&
+                        _pbSparseIndex->_length >= dataLength && (!_pbSparseData || _pbSparseData->_length >= dataLength);
+    if (direct) {
+        dsxFatal(dsx_memcpy_h2d(_pbSparseStart->_pDevData, srcSparseStart, _uniqueExamples * sizeof(uint64_t)), "NNDataSet::LoadSparseData");
+        dsxFatal(dsx_memcpy_h2d(_pbSparseEnd->_pDevData, srcSparseEnd, _uniqueExamples * sizeof(uint64_t)), "NNDataSet::LoadSparseData");
+        dsxFatal(dsx_memcpy_h2d(_pbSparseIndex->_pDevData, srcSparseIndex, dataLength * sizeof(uint32_t)), "NNDataSet::LoadSparseData");
+        if (_pbSparseData && srcSparseData)
+            dsxFatal(dsx_memcpy_h2d(_pbSparseData->_pDevData, srcSparseData, dataLength * sizeof(T)), "NNDataSet::LoadSparseData");
+    }
     CopySparseData(srcSparseStart, srcSparseEnd, srcSparseData, srcSparseIndex);
-    uploadSparse();
+    if (!direct) uploadSparse();
 }
 
 template <typename T>

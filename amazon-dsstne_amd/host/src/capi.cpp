@@ -353,8 +353,9 @@ int dsstne_topk(dsstne_context* c, const char* layer, uint32_t k, const char* fi
 int dsstne_get_topk(dsstne_context* c, const char* layer, uint32_t rows, uint32_t k, float* scores, uint32_t* indexes)
 {
     CAPI_TRY
-    dsxFatal(dsx_memcpy_d2h(scores, c->scoreBuf(layer)->_pDevData, (size_t)rows * k * sizeof(float)), "dsstne_get_topk");
-    dsxFatal(dsx_memcpy_d2h(indexes, c->indexBuf(layer)->_pDevData, (size_t)rows * k * sizeof(uint32_t)), "dsstne_get_topk");
+    dsxFatal(dsx_memcpy_d2h_pair(scores, c->scoreBuf(layer)->_pDevData, (size_t)rows * k * sizeof(float), indexes,
+                                 c->indexBuf(layer)->_pDevData, (size_t)rows * k * sizeof(uint32_t)),
+             "dsstne_get_topk");
     return 0;
     CAPI_CATCH(-1)
 }

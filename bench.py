@@ -128,6 +128,18 @@ def network_bench(args, pkg, lib):
     net.sync()
     ms_upload = (time.perf_counter() - t0) * 1e3 / up_steps
 
+    # One request at a time, as the reference's JNI predict serves them: upload the batch, predict, top-K, read the results
+    # back, and only then the next one.
+    rt = []
+    for n in range(up_steps + 5):
+        t0 = time.perf_counter()
+        net.load_sparse(p.start, p.end, p.sparse_data, p.sparse_index)
+        step()
+        net.get_topk(B)
+        if n >= 5:
+            rt.append(time.perf_counter() - t0)
+    ms_request = float(np.median(rt)) * 1e3
+
     # The same kernels one at a time on the same shapes (raw C ABI of the kernel library, same stream).
     pipe = DevicePipeline(p, lib)
     pipe.step()
@@ -242,6 +254,8 @@ def network_bench(args, pkg, lib):
                      "note": "NNNetwork::SetLanes(1): one set of buffers, one stream, batches strictly one after the other"},
         "with_input_upload": {"ms_per_step": round(ms_upload, 5), "value": round(B / (ms_upload / 1e3), 1), "unit": "samples/s",
                               "note": "host CSR arrays of the whole dataset copied and uploaded before every step (PCIe-inclusive)"},
+        "request_round_trip": {"ms": round(ms_request, 5), "value": round(B / (ms_request / 1e3), 1), "unit": "samples/s",
+                               "note": "median over requests served one at a time: upload, predict, filtered top-K, results read back"},
     }
     return out
 

@@ -122,6 +122,8 @@ int dsx_sync(void);                                                          /* 
 int dsx_set_lane(int lane);
 int dsx_get_lane(void);
 int dsx_memcpy_d2h_lane(int lane, void* host_dst, const void* device_src, size_t bytes);
+/* Two downloads, one wait (no counterpart in the reference, which copies scores and indexes one after the other). */
+int dsx_memcpy_d2h_pair(void* host_dst0, const void* device_src0, size_t bytes0, void* host_dst1, const void* device_src1, size_t bytes1);
 
 /* Event timing on the library stream (the reference keeps cudaEvent timings for KNN, knn/KnnExactGpu.cu:130-148). */
 int dsx_timer_start(void);
