@@ -117,7 +117,8 @@ def network_bench(args, pkg, lib):
     # The same step when the batch's CSR arrays are handed over as host buffers every time (NNDataSet::LoadSparseData, as the
     # reference's JNI predict does): never `value`, reported beside it.
     up_steps = max(5, min(50, args.steps))
-    for _ in range(4):   # untimed: the first uploads allocate the pinned staging buffers
+    for _ in range(20):   # untimed: the first uploads allocate the pinned staging buffers, and the first time this many
+        # copies and kernels are queued without a wait the HIP runtime grows its pools once (about 10 ms)
         net.load_sparse(p.start, p.end, p.sparse_data, p.sparse_index)
         step()
     net.sync()
