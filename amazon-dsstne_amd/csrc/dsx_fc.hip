@@ -6,6 +6,7 @@
 // registers.  X and W tiles of 16 k-steps are staged k-major in LDS (double buffered, one barrier per step) so that the
 // 64 lanes of an MFMA operand read 2 x 32 consecutive floats.  Workgroup ids are remapped so that the workgroups that land
 // on one XCD (id mod 8) sweep all row tiles of a few column tiles: a W tile is then fetched by one L2 only.
+#include <type_traits>
 #include "dsx_device.h"
 #include "dsx_internal.h"
 
@@ -31,6 +32,119 @@ struct FcArgs {
     CandArgs cand;       // candidate mode (template flag CAND): Z is not written, see candidate_epilogue
 };
 
+// Epilogue shared by the GEMM kernels: bias, accumulate, activation, store, and on request the maxima of 64-column segments.
+// (row_w, col_w): origin of this wavefront's (32 MI) x (32 NI) part of Z.  sT: 512 floats of LDS that belong to this
+// wavefront alone (only touched when a.seg_max is set).
+template <int MI, int NI, int ACT>
+__device__ __forceinline__ void fc_epilogue(floatx16 (&acc)[MI][NI], const FcArgs& a, uint32_t row_w, uint32_t col_w, int lane, float* sT)
+{
+    const int l32 = lane & 31, lhi = lane >> 5;
+    // Epilogue: accumulator register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 block.
+    // With seg_max set (128 x 128 tiles only), every wavefront also reduces the 64 columns it owns to one maximum per row:
+    // a later top-K can then skip the column segments that cannot hold a result.
+    constexpr bool kCanSegMax = (MI == 2 && NI == 2);
+    const bool want_max = kCanSegMax && a.seg_max != nullptr;
+    float smax[kCanSegMax ? 32 : 1];
+    if constexpr (kCanSegMax) {
+#pragma unroll
+        for (int q = 0; q < 32; q++) smax[q] = -__builtin_inff();
+    }
+    // Interior tiles: every store is "wave-uniform row base + this lane's constant 32-bit byte offset" (scalar address
+    // arithmetic only), the accumulate case is a branch around the whole loop and not one per element (so the 64 outputs of
+    // a wavefront are independent instructions the scheduler can interleave), and the sigmoid folds the bias and the
+    // exponent's scale into one multiply-add.  Vector instructions here are matrix-core time lost, see above.
+    const uint32_t row_u = __builtin_amdgcn_readfirstlane(row_w), col_u = __builtin_amdgcn_readfirstlane(col_w);
+    const bool full_tile = (row_u + 32 * MI <= a.batch) && (col_u + 32 * NI <= a.n) && a.ldz < (1u << 27);
+    if (full_tile) {
+        const uint32_t lane_off = (4u * lhi * a.ldz + l32) * 4u;
+        auto interior = [&](auto accumulate_tag) __attribute__((always_inline)) {
+            constexpr bool ACCUM = decltype(accumulate_tag)::value;
+            constexpr float kNegLog2e = -1.4426950408889634f;
+            // (row index outermost, the column blocks innermost: an accumulator register is dead as soon as its output is
+            // stored and folded into the row's maximum, so the maxima need no registers of their own on top of the tile)
+            float bias[NI];
+#pragma unroll
+            for (int j = 0; j < NI; j++) {
+                bias[j] = a.bias ? a.bias[col_u + j * 32 + l32] : 0.0f;
+                if constexpr (ACT == DSX_ACT_SIGMOID && !ACCUM) bias[j] *= kNegLog2e;
+            }
+#pragma unroll
+            for (int i = 0; i < MI; i++) {
+                char* base = reinterpret_cast<char*>(a.Z) + ((uint64_t)(row_u + i * 32) * a.ldz + col_u) * 4;
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+#pragma unroll
+                    for (int j = 0; j < NI; j++) {
+                        float* dst = reinterpret_cast<float*>(base + (uint64_t)(8 * (v / 4) + (v % 4)) * a.ldz * 4 + j * 128 + lane_off);
+                        float y;
+                        if constexpr (ACT == DSX_ACT_SIGMOID && !ACCUM) {
+                            y = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(fmaf(acc[i][j][v], kNegLog2e, bias[j])));
+                        } else {
+                            float x = acc[i][j][v] + bias[j];
+                            if constexpr (ACCUM) x += *dst;
+                            y = activate<ACT>(x, a.slope, a.alpha, a.lambda);
+                        }
+                        *dst = y;
+                        if constexpr (kCanSegMax) smax[i * 16 + v] = (j == 0) ? y : fmaxf(smax[i * 16 + v], y);
+                    }
+                }
+            }
+        };
+        if (a.accumulate) interior(std::true_type{});
+        else interior(std::false_type{});
+    } else {
+#pragma unroll
+        for (int j = 0; j < NI; j++) {
+            const uint32_t c = col_u + j * 32 + l32;
+            if (c >= a.n) continue;
+            const float bias = a.bias ? a.bias[c] : 0.0f;
+#pragma unroll
+            for (int i = 0; i < MI; i++) {
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const uint32_t r = row_u + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
+                    if (r < a.batch) {
+                        float* dst = a.Z + (uint64_t)r * a.ldz + c;
+                        float x = acc[i][j][v] + bias;
+                        if (a.accumulate) x += *dst;
+                        const float y = activate<ACT>(x, a.slope, a.alpha, a.lambda);
+                        *dst = y;
+                        if constexpr (kCanSegMax) smax[i * 16 + v] = fmaxf(smax[i * 16 + v], y);
+                    }
+                }
+            }
+        }
+    }
+    if constexpr (kCanSegMax) {
+        if (want_max) {
+            // Each lane holds 32 row maxima over its own column; what is wanted is, per row, the maximum over the 32 lanes of a
+            // half wave.  Transposed through LDS, eight row indices at a time (2 KiB per wavefront): LDS instructions do not
+            // compete with the matrix cores the way a cross-lane reduction in vector registers would.  Lane L reads an eighth
+            // of the 32 values of result e = L / 4 (row index 8c + e % 8, lane half e / 8), rotated by e so that the lanes of
+            // a quad and the 16 results spread over all banks; the four partial maxima meet through two lane exchanges.
+            const int e = lane >> 2, part = lane & 3;
+            const uint32_t seg = col_u / 64;
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+#pragma unroll
+                for (int q = 0; q < 8; q++) sT[q * 64 + lane] = smax[8 * c + q];
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                float m = -__builtin_inff();
+#pragma unroll
+                for (int u = 0; u < 8; u++) m = fmaxf(m, sT[(e & 7) * 64 + (e >> 3) * 32 + part * 8 + ((u + e) & 7)]);
+                m = fmaxf(m, __shfl_xor(m, 1));
+                m = fmaxf(m, __shfl_xor(m, 2));
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();   // the next round overwrites what was just read
+                const int q = 8 * c + (e & 7), i = q >> 4, v = q & 15;
+                const uint32_t r = row_u + i * 32 + 8 * (v >> 2) + 4 * (e >> 3) + (v & 3);
+                if (part == 0 && r < a.batch && seg < a.nseg) a.seg_max[(uint64_t)r * a.nseg + seg] = m;
+            }
+        }
+    }
+}
+
 // MI, NI: 32x32 MFMA blocks per wavefront in M and N.  XV / WV: vector width (floats) of the global loads of X / W.
 // TRANS: W is stored [n][k].
 template <int MI, int NI, int BK, int XV, int WV, bool TRANS, int ACT, bool CAND = false>
@@ -52,7 +166,9 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
         wg = xcd * per_xcd + local;
         if (local >= per_xcd || wg >= total) return;
     }
-    const uint32_t tm = wg % a.tiles_m, tn = wg / a.tiles_m;
+    // Column tiles are taken from the last to the first: a partial last tile (bounds-checked loads and stores, several times
+    // slower than an interior tile) then starts with the first round of workgroups instead of ending the launch alone.
+    const uint32_t tm = wg % a.tiles_m, tn = a.tiles_n - 1 - wg / a.tiles_m;
     const uint32_t row0 = tm * BM, col0 = tn * BN;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -308,81 +424,12 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
         return;
     }
 
-    // Epilogue: accumulator register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 block.
-    // With seg_max set (128 x 128 tiles only), every wavefront also reduces the 64 columns it owns to one maximum per row:
-    // a later top-K can then skip the column segments that cannot hold a result.
-    constexpr bool kCanSegMax = (MI == 2 && NI == 2);
-    const bool want_max = kCanSegMax && a.seg_max != nullptr;
-    float smax[kCanSegMax ? 32 : 1];
-    if constexpr (kCanSegMax) {
-#pragma unroll
-        for (int q = 0; q < 32; q++) smax[q] = -__builtin_inff();
-    }
-    const bool full_tile = (row0 + BM <= a.batch) && (col0 + BN <= a.n);
-    if (full_tile) {
-#pragma unroll
-        for (int j = 0; j < NI; j++) {
-            const uint32_t c = col0 + wn * 32 * NI + j * 32 + l32;
-            const float bias = a.bias ? a.bias[c] : 0.0f;
-#pragma unroll
-            for (int i = 0; i < MI; i++) {
-                float* base = a.Z + (uint64_t)(row0 + wm * 32 * MI + i * 32 + 4 * lhi) * a.ldz + c;
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    float* dst = base + (uint64_t)(8 * (v / 4) + (v % 4)) * a.ldz;
-                    float x = acc[i][j][v] + bias;
-                    if (a.accumulate) x += *dst;
-                    const float y = activate<ACT>(x, a.slope, a.alpha, a.lambda);
-                    *dst = y;
-                    if constexpr (kCanSegMax) smax[i * 16 + v] = fmaxf(smax[i * 16 + v], y);
-                }
-            }
-        }
-    } else {
-#pragma unroll
-        for (int j = 0; j < NI; j++) {
-            const uint32_t c = col0 + wn * 32 * NI + j * 32 + l32;
-            if (c >= a.n) continue;
-            const float bias = a.bias ? a.bias[c] : 0.0f;
-#pragma unroll
-            for (int i = 0; i < MI; i++) {
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const uint32_t r = row0 + wm * 32 * MI + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
-                    if (r < a.batch) {
-                        float* dst = a.Z + (uint64_t)r * a.ldz + c;
-                        float x = acc[i][j][v] + bias;
-                        if (a.accumulate) x += *dst;
-                        const float y = activate<ACT>(x, a.slope, a.alpha, a.lambda);
-                        *dst = y;
-                        if constexpr (kCanSegMax) smax[i * 16 + v] = fmaxf(smax[i * 16 + v], y);
-                    }
-                }
-            }
-        }
-    }
-    if constexpr (kCanSegMax) {
-        if (want_max) {
-            // Transpose through LDS (the operand tiles are dead by now): lane l wrote its 32 row maxima, and reads back the 32
-            // values that the lanes of its half wave hold for row index q = l % 32.  LDS instructions do not compete with the
-            // matrix cores the way a cross-lane reduction in vector registers would.  Pitch 65 keeps both sides conflict-free.
-            // (the k-loop ended with a barrier: every wavefront is done with sA / sB)
-            float* sT = ((wave < 2) ? &sA[0][0][0] : &sB[0][0][0]) + (wave & 1) * (32 * 65);
-            static_assert(sizeof(sA) >= 2 * 32 * 65 * sizeof(float) && sizeof(sB) >= 2 * 32 * 65 * sizeof(float),
-                          "the transposition reuses the operand tiles' LDS, two wavefronts in each");
-#pragma unroll
-            for (int q = 0; q < 32; q++) sT[q * 65 + lane] = smax[q];
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            float m = -__builtin_inff();
-#pragma unroll
-            for (int t = 0; t < 32; t++) m = fmaxf(m, sT[l32 * 65 + lhi * 32 + t]);
-            smax[0] = m;
-            const int q = l32, i = q >> 4, v = q & 15;
-            const uint32_t r = row0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * lhi + (v & 3);
-            const uint32_t seg = (col0 + wn * 64) / 64;
-            if (r < a.batch && seg < a.nseg) a.seg_max[(uint64_t)r * a.nseg + seg] = smax[0];
-        }
+    {
+        static_assert(sizeof(sA) >= 2 * 512 * sizeof(float) && sizeof(sB) >= 2 * 512 * sizeof(float),
+                      "the segment maxima are transposed through the operand tiles' LDS, two wavefronts in each");
+        // (the k-loop ended with a barrier: every wavefront is done with sA / sB)
+        fc_epilogue<MI, NI, ACT>(acc, a, row0 + wm * 32 * MI, col0 + wn * 32 * NI, lane,
+                                 ((wave < 2) ? &sA[0][0][0] : &sB[0][0][0]) + (wave & 1) * 512);
     }
 }
 
