@@ -171,6 +171,9 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
     const uint32_t tm = wg % a.tiles_m, tn = a.tiles_n - 1 - wg / a.tiles_m;
     const uint32_t row0 = tm * BM, col0 = tn * BN;
 
+    // Wavefronts in the k-loop go first, wavefronts in the epilogue take the issue slots that are left: the matrix cores then
+    // idle less while a workgroup activates and stores its tile (measured 1.5 % on a 1024 x 128 x 27,278 layer).
+    __builtin_amdgcn_s_setprio(3);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, lhi = lane >> 5;
@@ -417,6 +420,7 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
         }
     }
 
+    __builtin_amdgcn_s_setprio(0);
     if constexpr (CAND) {
         static_assert(sizeof(sA) >= kCandLdsBytes<MI>, "the epilogue reuses the X tile's LDS");
         // (the k-loop ended with a barrier: every wavefront is done with sA)
