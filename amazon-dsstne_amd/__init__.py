@@ -65,6 +65,8 @@ SIGNATURES = {
     "dsx_get_lane": [],
     "dsx_memcpy_d2h_lane": [_int, _vp, _vp, _sz],
     "dsx_memcpy_d2h_pair": [_vp, _vp, _sz, _vp, _vp, _sz],
+    "dsx_memcpy_h2d_unordered": [_vp, _vp, _sz],
+    "dsx_lane_wait_other": [],
     "dsx_timer_start": [],
     "dsx_timer_stop": [C.POINTER(_f32)],
     "dsx_clear_unit": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32],

@@ -329,17 +329,14 @@ int dsx_memset(void* p, int value, size_t bytes)
     return lanes_join_after();
 }
 
-int dsx_memcpy_h2d(void* dst, const void* src, size_t bytes)
+// Host memory -> device on the selected lane's stream.  Up to kUploadSlotBytes go through the pinned ring and return as soon
+// as the copy is queued; more than that is copied straight from the caller's (possibly pageable) memory and waited for.
+static int upload_on_selected_lane(void* dst, const void* src, size_t bytes)
 {
-    DSX_REQUIRE_INIT();
-    if (bytes == 0) return DSX_OK;
-    DSX_CHECK_ARG(dst && src, "dsx_memcpy_h2d: null pointer");
-    // the destination may still be read by kernels of the other lane, and is read by whatever either lane runs next
-    if (int rc = lanes_join_before()) return rc;
     if (bytes > kUploadSlotBytes) {
         DSX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx().stream));
         DSX_HIP(hipStreamSynchronize(ctx().stream));   // src may be pageable: wait until it has been read
-        return lanes_join_after();
+        return DSX_OK;
     }
     std::lock_guard<std::mutex> lock(g_alloc_mutex);
     const int slot = g_upload_next;
@@ -353,7 +350,38 @@ int dsx_memcpy_h2d(void* dst, const void* src, size_t bytes)
     DSX_HIP(hipMemcpyAsync(dst, g_upload_host[slot], bytes, hipMemcpyHostToDevice, ctx().stream));
     DSX_HIP(hipEventRecord(g_upload_done[slot], ctx().stream));
     g_upload_busy[slot] = true;
+    return DSX_OK;
+}
+
+int dsx_memcpy_h2d(void* dst, const void* src, size_t bytes)
+{
+    DSX_REQUIRE_INIT();
+    if (bytes == 0) return DSX_OK;
+    DSX_CHECK_ARG(dst && src, "dsx_memcpy_h2d: null pointer");
+    // the destination may still be read by kernels of the other lane, and is read by whatever either lane runs next
+    if (int rc = lanes_join_before()) return rc;
+    if (int rc = upload_on_selected_lane(dst, src, bytes)) return rc;
     return lanes_join_after();
+}
+
+int dsx_memcpy_h2d_unordered(void* dst, const void* src, size_t bytes)
+{
+    DSX_REQUIRE_INIT();
+    if (bytes == 0) return DSX_OK;
+    DSX_CHECK_ARG(dst && src, "dsx_memcpy_h2d_unordered: null pointer");
+    return upload_on_selected_lane(dst, src, bytes);
+}
+
+int dsx_lane_wait_other(void)
+{
+    DSX_REQUIRE_INIT();
+    hipStream_t other = other_lane_stream();
+    if (!other) return DSX_OK;
+    const int o = g_lane ^ 1;
+    DSX_HIP(hipEventRecord(g_lane_event[o], other));
+    DSX_HIP(hipStreamWaitEvent(ctx().stream, g_lane_event[o], 0));
+    g_lane_seen[g_lane] = g_lane_selected[o];
+    return DSX_OK;
 }
 
 int dsx_memcpy_d2h(void* dst, const void* src, size_t bytes)

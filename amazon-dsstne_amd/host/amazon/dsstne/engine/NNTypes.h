@@ -75,6 +75,24 @@ struct NNDataSetBase {
     bool _bIndexed;
     uint32_t _batch;
 
+    // No counterpart in the reference (one set of arrays, blocking uploads).  Sparse data that arrives batch by batch
+    // (LoadSparseData) goes to a second set of device arrays, the one no kernel in flight reads, on the lane the next
+    // PredictBatch will use: the copy overlaps with the batch before it.  _pbSparseStart / End / Index / Data above always
+    // name the set that holds the latest load; kernels launched earlier keep reading the set they were given.
+    unique_ptr<GpuBuffer<uint64_t>> _pbSparseStartOther;
+    unique_ptr<GpuBuffer<uint64_t>> _pbSparseEndOther;
+    unique_ptr<GpuBuffer<uint32_t>> _pbSparseIndexOther;
+    struct SparseSetState {
+        int _uploadLane = -1;        // lane whose stream carries the set's last unordered upload (-1: ordered on both lanes)
+        uint32_t _readLanes = 0;     // lanes that have launched readers of the set since that upload
+        uint32_t _orderedLanes = 3;  // lanes that are known to run after that upload
+    };
+    SparseSetState _sparseSet, _sparseSetOther;
+    // Call before launching a kernel that reads the _pbSparse* arrays on the selected lane.
+    void NoteSparseRead();
+    // The lane the next PredictBatch will run on (kept by NNNetwork); a wrong value costs a wait between the lanes, no more.
+    static int s_nextLane;
+
     NNDataSetBase();
     virtual ~NNDataSetBase() = 0;
     NNDataSetDimensions GetDimensions();
@@ -126,6 +144,7 @@ public:
     unique_ptr<GpuBuffer<T>> _pbData;
     vector<T> _vSparseData;
     unique_ptr<GpuBuffer<T>> _pbSparseData;
+    unique_ptr<GpuBuffer<T>> _pbSparseDataOther;   // see _pbSparseStartOther
 
     // dense
     NNDataSet(uint32_t examples, const NNDataSetDimensions& dim, const string& name = "");

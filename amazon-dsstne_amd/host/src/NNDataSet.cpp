@@ -179,6 +179,7 @@ template <typename T> void NNDataSet<T>::checkSparseLoad(const uint64_t start0, 
 
 template <typename T> void NNDataSet<T>::uploadSparse()
 {
+    _sparseSet = SparseSetState();   // the uploads below are ordered on both lanes
     // The buffers were sized at construction (or by Shard); batches loaded later reuse them without reallocation.
     _pbSparseStart->Upload(_vSparseStart.data());
     _pbSparseEnd->Upload(_vSparseEnd.data());
@@ -207,16 +208,37 @@ void NNDataSet<T>::LoadSparseData(const uint64_t* srcSparseStart, const uint64_t
     if (!(_attributes & NNDataSetEnums::Attributes::Sparse)) throw std::runtime_error("Cannot set sparse data on a non sparse NNDataSet");
     checkSparseLoad(srcSparseStart[0], srcSparseEnd[_uniqueExamples - 1]);
     // The device copies are queued first, straight from the caller's arrays and only as long as this batch's data (the
-    // buffers may be larger): the device starts on them while the host shadows below are still being filled.
+    // buffers may be larger): the device starts on them while the host shadows below are still being filled.  They go to the
+    // set of device arrays that the kernels in flight do not read, on the lane the next PredictBatch will use, and are
+    // ordered against that lane only.
     const uint64_t dataLength = srcSparseEnd[_uniqueExamples - 1];
     const bool direct = _pbSparseStart && _pbSparseEnd && _pbSparseIndex && _pbSparseStart->_length >= _uniqueExamples &&
                         _pbSparseIndex->_length >= dataLength && (!_pbSparseData || _pbSparseData->_length >= dataLength);
     if (direct) {
-        dsxFatal(dsx_memcpy_h2d(_pbSparseStart->_pDevData, srcSparseStart, _uniqueExamples * sizeof(uint64_t)), "NNDataSet::LoadSparseData");
-        dsxFatal(dsx_memcpy_h2d(_pbSparseEnd->_pDevData, srcSparseEnd, _uniqueExamples * sizeof(uint64_t)), "NNDataSet::LoadSparseData");
-        dsxFatal(dsx_memcpy_h2d(_pbSparseIndex->_pDevData, srcSparseIndex, dataLength * sizeof(uint32_t)), "NNDataSet::LoadSparseData");
+        if (!_pbSparseStartOther) {
+            _pbSparseStartOther.reset(new GpuBuffer<uint64_t>(_pbSparseStart->_length, false, _bStreaming));
+            _pbSparseEndOther.reset(new GpuBuffer<uint64_t>(_pbSparseEnd->_length, false, _bStreaming));
+            _pbSparseIndexOther.reset(new GpuBuffer<uint32_t>(_pbSparseIndex->_length, false, _bStreaming));
+            if (_pbSparseData) _pbSparseDataOther.reset(new GpuBuffer<T>(_pbSparseData->_length, false, _bStreaming));
+        }
+        _pbSparseStart.swap(_pbSparseStartOther);
+        _pbSparseEnd.swap(_pbSparseEndOther);
+        _pbSparseIndex.swap(_pbSparseIndexOther);
+        _pbSparseData.swap(_pbSparseDataOther);
+        std::swap(_sparseSet, _sparseSetOther);
+        const int selected = dsx_get_lane();
+        const int target = (s_nextLane == 1) ? 1 : 0;
+        if (target != selected) dsxFatal(dsx_set_lane(target), "NNDataSet::LoadSparseData");
+        if (_sparseSet._readLanes & ~(1u << target)) dsxFatal(dsx_lane_wait_other(), "NNDataSet::LoadSparseData");   // readers on the other lane
+        dsxFatal(dsx_memcpy_h2d_unordered(_pbSparseStart->_pDevData, srcSparseStart, _uniqueExamples * sizeof(uint64_t)), "NNDataSet::LoadSparseData");
+        dsxFatal(dsx_memcpy_h2d_unordered(_pbSparseEnd->_pDevData, srcSparseEnd, _uniqueExamples * sizeof(uint64_t)), "NNDataSet::LoadSparseData");
+        dsxFatal(dsx_memcpy_h2d_unordered(_pbSparseIndex->_pDevData, srcSparseIndex, dataLength * sizeof(uint32_t)), "NNDataSet::LoadSparseData");
         if (_pbSparseData && srcSparseData)
-            dsxFatal(dsx_memcpy_h2d(_pbSparseData->_pDevData, srcSparseData, dataLength * sizeof(T)), "NNDataSet::LoadSparseData");
+            dsxFatal(dsx_memcpy_h2d_unordered(_pbSparseData->_pDevData, srcSparseData, dataLength * sizeof(T)), "NNDataSet::LoadSparseData");
+        _sparseSet._uploadLane = target;
+        _sparseSet._readLanes = 0;
+        _sparseSet._orderedLanes = 1u << target;
+        if (target != selected) dsxFatal(dsx_set_lane(selected), "NNDataSet::LoadSparseData");
     }
     CopySparseData(srcSparseStart, srcSparseEnd, srcSparseData, srcSparseIndex);
     if (!direct) uploadSparse();
@@ -386,6 +408,18 @@ template <typename T> bool NNDataSet<T>::SetDenoising(bool flag)
     return !flag;
 }
 
+int NNDataSetBase::s_nextLane = 0;
+
+void NNDataSetBase::NoteSparseRead()
+{
+    const uint32_t lane = 1u << (dsx_get_lane() & 1);
+    if (_sparseSet._uploadLane >= 0 && !(_sparseSet._orderedLanes & lane)) {   // loaded on the other lane: run after that copy
+        dsxFatal(dsx_lane_wait_other(), "NNDataSetBase::NoteSparseRead");
+        _sparseSet._orderedLanes |= lane;
+    }
+    _sparseSet._readLanes |= lane;
+}
+
 // ------------------------------------------------------------------------------------------------------------- device work
 
 template <typename T> bool NNDataSet<T>::LoadInputUnit(uint32_t position, uint32_t batch, uint32_t stride, NNFloat* pUnit)
@@ -397,6 +431,7 @@ template <typename T> bool NNDataSet<T>::LoadInputUnit(uint32_t position, uint32
 
 template <typename T> bool NNDataSet<T>::LoadSparseInputUnit(uint32_t position, uint32_t batch, uint32_t stride, NNFloat* pUnit)
 {
+    NoteSparseRead();
     dsxFatal(dsx_load_sparse_input_unit(_attributes, (uint32_t)_dataType, position, batch, stride, pUnit, _pbIndex ? _pbIndex->_pDevData : NULL,
                                         _pbSparseStart->_pDevData, _pbSparseEnd->_pDevData, _pbSparseIndex->_pDevData,
                                         _pbDataWeight ? _pbDataWeight->_pDevData : NULL, _pbSparseData ? _pbSparseData->_pDevData : NULL),
@@ -407,6 +442,7 @@ template <typename T> bool NNDataSet<T>::LoadSparseInputUnit(uint32_t position, 
 template <typename T>
 bool NNDataSet<T>::CalculateSparseZ(uint32_t position, uint32_t batch, uint32_t stride, NNFloat* pWeight, NNFloat* pUnit, NNFloat beta)
 {
+    NoteSparseRead();
     dsxFatal(dsx_sparse_z(_attributes, (uint32_t)_dataType, position, batch, stride, pWeight, _pbIndex ? _pbIndex->_pDevData : NULL,
                           _pbSparseStart->_pDevData, _pbSparseEnd->_pDevData, _pbSparseIndex->_pDevData,
                           _pbDataWeight ? _pbDataWeight->_pDevData : NULL, _pbSparseData ? _pbSparseData->_pDevData : NULL, pUnit, beta),
@@ -418,6 +454,7 @@ template <typename T>
 bool NNDataSet<T>::CalculateSparseLayer(uint32_t position, uint32_t batch, uint32_t stride, NNFloat* pWeight, NNFloat* pBias,
                                         Activation activation, NNFloat slope, NNFloat alpha, NNFloat lambda, NNFloat* pUnit)
 {
+    NoteSparseRead();
     dsx_act_params p = {slope, alpha, lambda};
     dsxFatal(dsx_sparse_layer_forward(_attributes, (uint32_t)_dataType, position, batch, stride, pWeight, _pbIndex ? _pbIndex->_pDevData : NULL,
                                       _pbSparseStart->_pDevData, _pbSparseEnd->_pDevData, _pbSparseIndex->_pDevData,

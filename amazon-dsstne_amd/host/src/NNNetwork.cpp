@@ -145,6 +145,7 @@ NNNetwork::~NNNetwork()
     for (auto l : _vLayer) delete l;
     delete _pDescriptor;
     if (getGpu()._pNetwork == this) getGpu()._pNetwork = NULL;
+    NNDataSetBase::s_nextLane = 0;
     if (dsx_is_initialized()) dsx_set_lane(0);   // whatever runs next starts on the first lane (deleting the buffers above waited for both)
 }
 
@@ -277,6 +278,7 @@ void NNNetwork::PredictBatch(uint32_t layers)
         for (auto l : _vLayer) l->SwapLane();
         dsxFatal(dsx_set_lane((int)_lane), "NNNetwork::PredictBatch: lane");
     }
+    NNDataSetBase::s_nextLane = (_lanes > 1) ? (int)(_lane ^ 1) : (int)_lane;   // where a LoadSparseData for the next batch should go
     uint32_t batch = _batch;
     if (_position + batch > _examples) batch = _examples - _position;
     ClearUpdates();
@@ -295,6 +297,7 @@ bool NNNetwork::SetLanes(uint32_t lanes)
     _lanes = lanes;
     _lane = 0;
     dsxFatal(dsx_set_lane(0), "NNNetwork::SetLanes");
+    NNDataSetBase::s_nextLane = (lanes > 1) ? 1 : 0;
     for (auto l : _vLayer) {
         l->_lanes = lanes;
         l->_bDirty = true;   // unit buffers are allocated anew
@@ -362,6 +365,7 @@ void NNNetwork::CalculateFilteredTopK(const string& layer, uint32_t k, NNDataSet
         NNDataSet<float>* pf = dynamic_cast<NNDataSet<float>*>(pFilter);
         if (pf && pf->_pbSparseData) pMul = pf->_pbSparseData->_pDevData;
     }
+    pFilter->NoteSparseRead();
     const uint32_t* pIndex = (pFilter->_attributes & NNDataSetEnums::Indexed) ? pFilter->_pbIndex->_pDevData : NULL;
     // with segment maxima of the current batch (left by the layer's dense kernel) only the segments that can hold a result are read
     const NNFloat* pSegMax = (pLayer->_segWidth != 0 && pLayer->_pbSegMax) ? pLayer->_pbSegMax->_pDevData : NULL;

@@ -254,7 +254,7 @@ def network_bench(args, pkg, lib):
         "one_lane": {"ms_per_step": round(ms_one_lane, 5), "value": round(B / (ms_one_lane / 1e3), 1), "unit": "samples/s",
                      "note": "NNNetwork::SetLanes(1): one set of buffers, one stream, batches strictly one after the other"},
         "with_input_upload": {"ms_per_step": round(ms_upload, 5), "value": round(B / (ms_upload / 1e3), 1), "unit": "samples/s",
-                              "note": "host CSR arrays of the whole dataset copied and uploaded before every step (PCIe-inclusive)"},
+                              "note": "the batch's CSR arrays handed over as host memory before every step (NNDataSet::LoadSparseData; PCIe-inclusive): uploads go to alternating sets of device arrays on the lane of the batch they belong to"},
         "request_round_trip": {"ms": round(ms_request, 5), "value": round(B / (ms_request / 1e3), 1), "unit": "samples/s",
                                "note": "median over requests served one at a time: upload, predict, filtered top-K, results read back"},
     }

@@ -122,6 +122,13 @@ int dsx_sync(void);                                                          /* 
 int dsx_set_lane(int lane);
 int dsx_get_lane(void);
 int dsx_memcpy_d2h_lane(int lane, void* host_dst, const void* device_src, size_t bytes);
+/* For data that arrives batch by batch (no counterpart in the reference, whose uploads block).  dsx_memcpy_h2d_unordered is
+ * dsx_memcpy_h2d on the selected lane only: the other lane is neither waited for nor told to wait, so the copy overlaps with
+ * whatever the other lane runs.  The caller guarantees that nothing queued on the other lane touches device_dst, and calls
+ * dsx_lane_wait_other (the selected lane waits for everything queued so far on the other one) before work on one lane
+ * depends on what the other lane wrote. */
+int dsx_memcpy_h2d_unordered(void* device_dst, const void* host_src, size_t bytes);
+int dsx_lane_wait_other(void);
 /* Two downloads, one wait (no counterpart in the reference, which copies scores and indexes one after the other). */
 int dsx_memcpy_d2h_pair(void* host_dst0, const void* device_src0, size_t bytes0, void* host_dst1, const void* device_src1, size_t bytes1);
 

@@ -325,6 +325,66 @@ def reference_batches(orc, p, positions):
     return out
 
 
+@pytest.mark.parametrize("config,batches,lanes", [(1, 9, 2), (2, 4, 2), (1, 5, 1)])
+def test_streamed_batches_on_two_lanes(pkg, dsx, orc, synth, config, batches, lanes):
+    """Batches handed over as host arrays one after the other (NNDataSet::LoadSparseData, as the reference's JNI predict feeds
+    it): the dataset holds one batch, every load replaces it, and the results of batch i are collected while batch i + 1 is
+    already queued.  The loads go to alternating sets of device arrays on alternating lanes; every batch must still see its
+    own data, as input and as filter."""
+    import copy
+    from amazon_dsstne_amd import host_api
+    big = synth.config(config, batches=batches)
+    positions = list(range(0, big.examples, big.batch))
+    want = reference_batches(orc, big, positions)
+
+    def batch_arrays(pos):
+        s, e = big.start[pos:pos + big.batch], big.end[pos:pos + big.batch]
+        lo, hi = int(s[0]), int(e[-1])
+        data = None if big.sparse_data is None else np.ascontiguousarray(big.sparse_data[lo:hi])
+        return (np.ascontiguousarray(s - lo), np.ascontiguousarray(e - lo), data, np.ascontiguousarray(big.sparse_index[lo:hi]))
+
+    one = copy.copy(big)                      # a dataset of one batch with room for the largest of them
+    one.examples = one.unique_examples = big.batch
+    room = max(int(big.end[pos + big.batch - 1] - big.start[pos]) for pos in positions)
+    one.start, one.end = np.zeros(big.batch, np.uint64), np.zeros(big.batch, np.uint64)
+    one.sparse_index = np.zeros(room, np.uint32)
+    one.sparse_data = None if big.sparse_data is None else np.zeros(room, big.sparse_data.dtype)
+    net = host_api.Network(one, max_k=big.k)
+    try:
+        net.bind_input()
+        if lanes == 1:
+            net.set_lanes(1)
+        got = []
+        for n, pos in enumerate(positions):
+            net.load_sparse(*batch_arrays(pos))
+            net.predict_batch(0)
+            net.topk(big.k, filter_dataset="input")
+            if lanes == 2 and n > 0:
+                got.append(net.get_topk_previous(big.batch))            # the batch before, while this one runs
+            elif lanes == 1:
+                got.append(net.get_topk(big.batch))
+        if lanes == 2:
+            got.append(net.get_topk(big.batch))
+        for n, ((rows, keys, idx, scores), (gk, gi)) in enumerate(zip(want, got)):
+            assert_topk_parity(gk, gi, keys, idx, scores, "%s streamed batch %d on %d lane(s)" % (big.name, n, lanes))
+        # the same data predicted twice after one load (the second batch runs on the lane that did not take the upload),
+        # and two loads in a row (the second finds the lane guess of the first unused)
+        net.load_sparse(*batch_arrays(positions[1]))
+        for rep in range(2):
+            net.predict_batch(0)
+            net.topk(big.k, filter_dataset="input")
+        gk, gi = net.get_topk(big.batch)
+        assert_topk_parity(gk, gi, want[1][1], want[1][2], want[1][3], big.name + " second predict after one load")
+        net.load_sparse(*batch_arrays(positions[2]))
+        net.load_sparse(*batch_arrays(positions[0]))
+        net.predict_batch(0)
+        net.topk(big.k, filter_dataset="input")
+        gk, gi = net.get_topk(big.batch)
+        assert_topk_parity(gk, gi, want[0][1], want[0][2], want[0][3], big.name + " after two loads in a row")
+    finally:
+        net.close()
+
+
 @pytest.mark.parametrize("config,batches", [(1, 7), (2, 3)])
 def test_two_lanes_keep_batches_apart(pkg, dsx, orc, synth, config, batches):
     """Consecutive PredictBatch calls alternate between two sets of buffers on two streams (NNNetwork::SetLanes).  A loop that
