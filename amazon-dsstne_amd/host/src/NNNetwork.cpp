@@ -40,6 +40,7 @@ NNNetwork::NNNetwork(NNNetworkDescriptor& d, uint32_t batch)
       _errorFunction(d._errorFunction), _mode(Prediction), _bShuffleIndices(d._bShuffleIndices), _pDescriptor(NULL), _bDirty(true),
       _verbose(false), _lanes(2), _lane(0)
 {
+    NNDataSetBase::s_nextLane = 1;   // the first PredictBatch of a network with two lanes runs on the second one
     // keep the scalar settings (not the weight payloads) for SaveNetCDF round trips
     _pDescriptor = new NNNetworkDescriptor(d);
     _pDescriptor->_vLayerDescriptor.clear();
