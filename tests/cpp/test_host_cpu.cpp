@@ -400,6 +400,7 @@ static void testNetworkDefinitions(const string& dir, const string& golden)
         CHECK_EQ((int)nd._errorFunction, (int)ErrorFunction::L2);
         CHECK(!nd._bShuffleIndices);
         CHECK_EQ(nd._vLayerDescriptor.size(), (size_t)3);
+        if (nd._vLayerDescriptor.size() != 3) return;   // fixture directory wrong or file unreadable: reported above
         const NNLayerDescriptor& in = nd._vLayerDescriptor[0];
         const NNLayerDescriptor& hid = nd._vLayerDescriptor[1];
         const NNLayerDescriptor& out = nd._vLayerDescriptor[2];
