@@ -52,6 +52,7 @@ __global__ __launch_bounds__(64 * WM * WN) __attribute__((amdgpu_waves_per_eu(WP
     }
     const uint32_t tm = wg % a.tiles_m, tn = wg / a.tiles_m;
     const uint32_t row0 = tm * BM, col0 = tn * BN;
+    __builtin_amdgcn_s_setprio(3);   // k-loop first, epilogue in the issue slots that are left (as in fc_gemm_kernel)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     const int l32 = lane & 31, lhi = lane >> 5;
@@ -125,6 +126,7 @@ __global__ __launch_bounds__(64 * WM * WN) __attribute__((amdgpu_waves_per_eu(WP
 #undef F16_LOAD
 #undef F16_STORE
 
+    __builtin_amdgcn_s_setprio(0);
     if constexpr (CAND) {
         static_assert(sizeof(sA) >= kCandLdsBytes<MI, WM, WN>, "the epilogue reuses the query tile's LDS");
         candidate_epilogue<MI, NI, WM, WN>(acc, reinterpret_cast<float*>(&sA[0][0][0]), a.cand, bound_key, row0, col0, a.batch, a.n, tid, wm, wn,
