@@ -325,7 +325,7 @@ def reference_batches(orc, p, positions):
     return out
 
 
-@pytest.mark.parametrize("config,batches,lanes", [(1, 9, 2), (2, 4, 2), (1, 5, 1)])
+@pytest.mark.parametrize("config,batches,lanes", [(1, 9, 2), (2, 4, 2), (1, 5, 1), (1, 40, 2)])
 def test_streamed_batches_on_two_lanes(pkg, dsx, orc, synth, config, batches, lanes):
     """Batches handed over as host arrays one after the other (NNDataSet::LoadSparseData, as the reference's JNI predict feeds
     it): the dataset holds one batch, every load replaces it, and the results of batch i are collected while batch i + 1 is
