@@ -52,6 +52,34 @@ def test_malloc_zero_fills_and_copies(pkg, dsx, rng):
     assert g.value > 0
 
 
+def test_lanes_unordered_upload_and_explicit_wait(pkg, dsx, rng):
+    """dsx_memcpy_h2d_unordered queues on the selected lane only; dsx_lane_wait_other makes the selected lane run after what
+    the other lane holds.  A kernel over 256 MiB keeps lane 1 busy ahead of the upload, lane 0 reads the buffer after the wait, and
+    dsx_memcpy_d2h_lane waits for lane 0 alone: it can only return the uploaded data if the wait ordered the lanes."""
+    n = 1 << 16
+    big = pkg.DeviceArray((64 << 20,), np.float32)          # 256 MiB
+    buf = pkg.DeviceArray((n,), np.float32)
+    out = pkg.DeviceArray((n,), np.float32)
+    try:
+        for rep in range(4):
+            x = rng.standard_normal(n).astype(np.float32)
+            pkg.check(dsx.dsx_set_lane(1))
+            assert dsx.dsx_get_lane() == 1
+            pkg.check(dsx.dsx_add_buffers(big.ptr, big.ptr, 64 << 20))    # a kernel (kernels order nothing between the lanes)
+            pkg.check(dsx.dsx_memcpy_h2d_unordered(buf.ptr, x.ctypes.data, x.nbytes))
+            pkg.check(dsx.dsx_set_lane(0))
+            pkg.check(dsx.dsx_lane_wait_other())
+            pkg.check(dsx.dsx_add_buffers(out.ptr, buf.ptr, n))           # out += buf on lane 0
+            got = np.empty(n, np.float32)
+            pkg.check(dsx.dsx_memcpy_d2h_lane(0, got.ctypes.data, out.ptr, got.nbytes))
+            want = x if rep == 0 else want + x
+            assert np.array_equal(got, want), "repetition %d" % rep
+        pkg.check(dsx.dsx_lane_wait_other())                              # harmless when nothing is pending
+    finally:
+        pkg.check(dsx.dsx_set_lane(0))
+        pkg.check(dsx.dsx_sync())
+
+
 def test_bad_arguments_are_rejected(pkg, dsx):
     a = pkg.DeviceArray((4, 8), np.float32)
     k = pkg.DeviceArray((4, 8), np.float32)
