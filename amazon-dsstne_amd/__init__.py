@@ -67,6 +67,10 @@ SIGNATURES = {
     "dsx_memcpy_d2h_pair": [_vp, _vp, _sz, _vp, _vp, _sz],
     "dsx_memcpy_h2d_unordered": [_vp, _vp, _sz],
     "dsx_lane_wait_other": [],
+    "dsx_marker_create": [C.POINTER(C.c_void_p)],
+    "dsx_marker_record": [_vp],
+    "dsx_marker_wait": [_vp],
+    "dsx_marker_destroy": [_vp],
     "dsx_timer_start": [],
     "dsx_timer_stop": [C.POINTER(_f32)],
     "dsx_clear_unit": [_vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32],

@@ -32,16 +32,19 @@ static std::map<void*, size_t> g_host_allocs;
 using namespace dsx;
 
 // Uploads of up to kUploadSlotBytes go through a ring of pinned staging buffers: the caller's bytes are copied into a slot,
-// the DMA is queued on the library's stream and the call returns — the source may be reused at once (as after the blocking
-// cudaMemcpy of GpuBuffer::Upload), and everything queued later on the stream sees the data.  A batch's CSR arrays (four
-// uploads, engine/NNTypes.cpp:583-778) then cost four host copies instead of four round trips.  A slot is reused only after
-// its own copy has finished.
+// the DMA is queued on the selected lane's stream and the call returns — the source may be reused at once (as after the
+// blocking cudaMemcpy of GpuBuffer::Upload), and everything queued later on the stream sees the data.  A batch's CSR arrays
+// (four uploads, engine/NNTypes.cpp:583-778) then cost four host copies instead of four round trips.  Consecutive uploads
+// share a slot until it is full (a batch of config 2 is 0.6 MB: the ring holds some fifty batches, so a caller that streams
+// batches is never held up by the ring while the device is several batches behind); a slot is reused only after the copies
+// out of it have finished on both lanes.
 constexpr int kUploadSlots = 8;
 constexpr size_t kUploadSlotBytes = (size_t)4 << 20;
 static char* g_upload_host[kUploadSlots] = {};
-static hipEvent_t g_upload_done[kUploadSlots] = {};
-static bool g_upload_busy[kUploadSlots] = {};
-static int g_upload_next = 0;
+static hipEvent_t g_upload_done[kUploadSlots][2] = {};   // [slot][lane]: after the slot's last copy on that lane
+static bool g_upload_busy[kUploadSlots][2] = {};
+static int g_upload_slot = 0;       // slot being filled
+static size_t g_upload_fill = 0;    // bytes of it handed out
 
 // Downloads of up to kUploadSlotBytes land in a pinned buffer first and are copied to the caller's memory by the host: a copy
 // straight into pageable memory costs the runtime a staging round trip of its own that is several times slower.
@@ -61,12 +64,15 @@ static void upload_ring_release()
     g_download_host = nullptr;
     for (int i = 0; i < kUploadSlots; i++) {
         if (g_upload_host[i]) hipHostFree(g_upload_host[i]);
-        if (g_upload_done[i]) hipEventDestroy(g_upload_done[i]);
         g_upload_host[i] = nullptr;
-        g_upload_done[i] = nullptr;
-        g_upload_busy[i] = false;
+        for (int l = 0; l < 2; l++) {
+            if (g_upload_done[i][l]) hipEventDestroy(g_upload_done[i][l]);
+            g_upload_done[i][l] = nullptr;
+            g_upload_busy[i][l] = false;
+        }
     }
-    g_upload_next = 0;
+    g_upload_slot = 0;
+    g_upload_fill = 0;
 }
 
 
@@ -339,17 +345,26 @@ static int upload_on_selected_lane(void* dst, const void* src, size_t bytes)
         return DSX_OK;
     }
     std::lock_guard<std::mutex> lock(g_alloc_mutex);
-    const int slot = g_upload_next;
-    g_upload_next = (g_upload_next + 1) % kUploadSlots;
+    if (g_upload_fill + bytes > kUploadSlotBytes) {   // on to the next slot, once nothing is being copied out of it any more
+        g_upload_slot = (g_upload_slot + 1) % kUploadSlots;
+        g_upload_fill = 0;
+        for (int l = 0; l < 2; l++)
+            if (g_upload_busy[g_upload_slot][l]) {
+                DSX_HIP(hipEventSynchronize(g_upload_done[g_upload_slot][l]));
+                g_upload_busy[g_upload_slot][l] = false;
+            }
+    }
+    const int slot = g_upload_slot;
     if (!g_upload_host[slot]) {
         DSX_HIP(hipHostMalloc((void**)&g_upload_host[slot], kUploadSlotBytes, hipHostMallocDefault));
-        DSX_HIP(hipEventCreateWithFlags(&g_upload_done[slot], hipEventDisableTiming));
+        for (int l = 0; l < 2; l++) DSX_HIP(hipEventCreateWithFlags(&g_upload_done[slot][l], hipEventDisableTiming));
     }
-    if (g_upload_busy[slot]) DSX_HIP(hipEventSynchronize(g_upload_done[slot]));
-    memcpy(g_upload_host[slot], src, bytes);
-    DSX_HIP(hipMemcpyAsync(dst, g_upload_host[slot], bytes, hipMemcpyHostToDevice, ctx().stream));
-    DSX_HIP(hipEventRecord(g_upload_done[slot], ctx().stream));
-    g_upload_busy[slot] = true;
+    char* staged = g_upload_host[slot] + g_upload_fill;
+    g_upload_fill += (bytes + 255) / 256 * 256;
+    memcpy(staged, src, bytes);
+    DSX_HIP(hipMemcpyAsync(dst, staged, bytes, hipMemcpyHostToDevice, ctx().stream));
+    DSX_HIP(hipEventRecord(g_upload_done[slot][g_lane], ctx().stream));
+    g_upload_busy[slot][g_lane] = true;
     return DSX_OK;
 }
 
@@ -460,6 +475,40 @@ int dsx_memcpy_d2h_lane(int lane, void* dst, const void* src, size_t bytes)
     }
     DSX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s));
     DSX_HIP(hipStreamSynchronize(s));
+    return DSX_OK;
+}
+
+int dsx_marker_create(void** marker)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(marker, "dsx_marker_create: null pointer");
+    hipEvent_t e;
+    DSX_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    *marker = (void*)e;
+    return DSX_OK;
+}
+
+int dsx_marker_record(void* marker)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(marker, "dsx_marker_record: null marker");
+    DSX_HIP(hipEventRecord((hipEvent_t)marker, ctx().stream));
+    return DSX_OK;
+}
+
+int dsx_marker_wait(void* marker)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(marker, "dsx_marker_wait: null marker");
+    DSX_HIP(hipEventSynchronize((hipEvent_t)marker));
+    return DSX_OK;
+}
+
+int dsx_marker_destroy(void* marker)
+{
+    if (!marker) return DSX_OK;
+    DSX_REQUIRE_INIT();
+    DSX_HIP(hipEventDestroy((hipEvent_t)marker));
     return DSX_OK;
 }
 

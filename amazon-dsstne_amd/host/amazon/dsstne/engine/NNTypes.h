@@ -86,6 +86,8 @@ struct NNDataSetBase {
         int _uploadLane = -1;        // lane whose stream carries the set's last unordered upload (-1: ordered on both lanes)
         uint32_t _readLanes = 0;     // lanes that have launched readers of the set since that upload
         uint32_t _orderedLanes = 3;  // lanes that are known to run after that upload
+        void* _uploaded = NULL;      // marker behind that upload: the next load into this set waits for it on the host, which
+                                     // keeps a caller that streams batches two batches ahead of the device and no more
     };
     SparseSetState _sparseSet, _sparseSetOther;
     // Call before launching a kernel that reads the _pbSparse* arrays on the selected lane.

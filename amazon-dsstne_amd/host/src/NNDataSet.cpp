@@ -65,7 +65,13 @@ NNDataSetBase::NNDataSetBase(const string& name, NNDataSetEnums::DataType dataTy
 {
 }
 
-NNDataSetBase::~NNDataSetBase() {}
+NNDataSetBase::~NNDataSetBase()
+{
+    if (dsx_is_initialized()) {
+        dsx_marker_destroy(_sparseSet._uploaded);
+        dsx_marker_destroy(_sparseSetOther._uploaded);
+    }
+}
 
 NNDataSetDimensions NNDataSetBase::GetDimensions() { return NNDataSetDimensions(_width, _height, _length); }
 
@@ -179,7 +185,7 @@ template <typename T> void NNDataSet<T>::checkSparseLoad(const uint64_t start0, 
 
 template <typename T> void NNDataSet<T>::uploadSparse()
 {
-    _sparseSet = SparseSetState();   // the uploads below are ordered on both lanes
+    { void* marker = _sparseSet._uploaded; _sparseSet = SparseSetState(); _sparseSet._uploaded = marker; }   // the uploads below are ordered on both lanes
     // The buffers were sized at construction (or by Shard); batches loaded later reuse them without reallocation.
     _pbSparseStart->Upload(_vSparseStart.data());
     _pbSparseEnd->Upload(_vSparseEnd.data());
@@ -230,6 +236,10 @@ void NNDataSet<T>::LoadSparseData(const uint64_t* srcSparseStart, const uint64_t
         const int target = (s_nextLane == 1) ? 1 : 0;
         if (target != selected) dsxFatal(dsx_set_lane(target), "NNDataSet::LoadSparseData");
         if (_sparseSet._readLanes & ~(1u << target)) dsxFatal(dsx_lane_wait_other(), "NNDataSet::LoadSparseData");   // readers on the other lane
+        // The load before the last went into this set: once its copies are through, the device is at most two batches behind.
+        // (Queues that run many batches deep make the runtime stall in bursts; see the measurement notes.)
+        if (!_sparseSet._uploaded) dsxFatal(dsx_marker_create(&_sparseSet._uploaded), "NNDataSet::LoadSparseData");
+        else dsxFatal(dsx_marker_wait(_sparseSet._uploaded), "NNDataSet::LoadSparseData");
         dsxFatal(dsx_memcpy_h2d_unordered(_pbSparseStart->_pDevData, srcSparseStart, _uniqueExamples * sizeof(uint64_t)), "NNDataSet::LoadSparseData");
         dsxFatal(dsx_memcpy_h2d_unordered(_pbSparseEnd->_pDevData, srcSparseEnd, _uniqueExamples * sizeof(uint64_t)), "NNDataSet::LoadSparseData");
         dsxFatal(dsx_memcpy_h2d_unordered(_pbSparseIndex->_pDevData, srcSparseIndex, dataLength * sizeof(uint32_t)), "NNDataSet::LoadSparseData");
@@ -238,6 +248,7 @@ void NNDataSet<T>::LoadSparseData(const uint64_t* srcSparseStart, const uint64_t
         _sparseSet._uploadLane = target;
         _sparseSet._readLanes = 0;
         _sparseSet._orderedLanes = 1u << target;
+        dsxFatal(dsx_marker_record(_sparseSet._uploaded), "NNDataSet::LoadSparseData");
         if (target != selected) dsxFatal(dsx_set_lane(selected), "NNDataSet::LoadSparseData");
     }
     CopySparseData(srcSparseStart, srcSparseEnd, srcSparseData, srcSparseIndex);

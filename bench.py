@@ -57,10 +57,23 @@ class StdoutToStderr:
         return False
 
 
+SETTLE_SECONDS = 0.06
+
+
+def settle(pkg, lib, fn, seconds=SETTLE_SECONDS):
+    """Untimed: keeps the device busy with fn() for `seconds`.  From idle the clocks of this part ramp up over about 30 ms of
+    sustained load (the same launch takes 85 us at the start of a burst and 73 us from then on), so a timed region that
+    starts cold measures the ramp, not the kernel."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            fn()
+        pkg.check(lib.dsx_sync())
+
+
 def time_launches(pkg, lib, fn, reps):
     """Average milliseconds of one call of fn(), measured with HIP events on the library stream over `reps` launches."""
-    fn()
-    pkg.check(lib.dsx_sync())
+    settle(pkg, lib, fn)
     pkg.check(lib.dsx_timer_start())
     for _ in range(reps):
         fn()
@@ -88,6 +101,7 @@ def network_bench(args, pkg, lib):
     def step():
         net.predict_batch(0)
         net.topk(K, filter_dataset=net.dataset)
+    settle(pkg, lib, step)
     for _ in range(args.warmup):
         step()
     net.sync()
@@ -102,9 +116,7 @@ def network_bench(args, pkg, lib):
     # buffers on two streams), so one batch's input layers and top-K overlap with the next one's GEMM.  The same on one
     # lane — the reference's single set of buffers, one batch's kernels strictly after the other's — for comparison.
     net.set_lanes(1)
-    for _ in range(max(2, args.warmup // 4)):
-        step()
-    net.sync()
+    settle(pkg, lib, step)
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
@@ -116,12 +128,13 @@ def network_bench(args, pkg, lib):
 
     # The same step when the batch's CSR arrays are handed over as host buffers every time (NNDataSet::LoadSparseData, as the
     # reference's JNI predict does): never `value`, reported beside it.
-    up_steps = max(5, min(50, args.steps))
-    for _ in range(20):   # untimed: the first uploads allocate the pinned staging buffers, and the first time this many
-        # copies and kernels are queued without a wait the HIP runtime grows its pools once (about 10 ms)
+    up_steps = max(5, min(200, args.steps))
+    def upload_step():
         net.load_sparse(p.start, p.end, p.sparse_data, p.sparse_index)
         step()
-    net.sync()
+    # untimed: the first uploads allocate the pinned staging buffers, and the first time this many copies and kernels are
+    # queued without a wait the HIP runtime grows its pools once (about 10 ms)
+    settle(pkg, lib, upload_step)
     t0 = time.perf_counter()
     for _ in range(up_steps):
         net.load_sparse(p.start, p.end, p.sparse_data, p.sparse_index)
@@ -251,6 +264,7 @@ def network_bench(args, pkg, lib):
         "roofline": roofline,
         "kernels": {n: {k: (round(v, 5) if isinstance(v, float) else v) for k, v in kv.items()} for n, kv in kernels.items()},
         "cpu_baseline": cpu,
+        "clock_settle_ms": SETTLE_SECONDS * 1e3,
         "one_lane": {"ms_per_step": round(ms_one_lane, 5), "value": round(B / (ms_one_lane / 1e3), 1), "unit": "samples/s",
                      "note": "NNNetwork::SetLanes(1): one set of buffers, one stream, batches strictly one after the other"},
         "with_input_upload": {"ms_per_step": round(ms_upload, 5), "value": round(B / (ms_upload / 1e3), 1), "unit": "samples/s",

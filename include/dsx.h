@@ -129,6 +129,14 @@ int dsx_memcpy_d2h_lane(int lane, void* host_dst, const void* device_src, size_t
  * depends on what the other lane wrote. */
 int dsx_memcpy_h2d_unordered(void* device_dst, const void* host_src, size_t bytes);
 int dsx_lane_wait_other(void);
+/* A marker is a point in the selected lane's queue (no counterpart in the reference): dsx_marker_record places it after
+ * everything queued so far on that lane, dsx_marker_wait blocks the calling host thread until the device has passed it (at
+ * once for a marker never recorded).  A caller that streams batches uses it to stay a bounded number of batches ahead of the
+ * device. */
+int dsx_marker_create(void** marker);
+int dsx_marker_record(void* marker);
+int dsx_marker_wait(void* marker);
+int dsx_marker_destroy(void* marker);
 /* Two downloads, one wait (no counterpart in the reference, which copies scores and indexes one after the other). */
 int dsx_memcpy_d2h_pair(void* host_dst0, const void* device_src0, size_t bytes0, void* host_dst1, const void* device_src1, size_t bytes1);
 
