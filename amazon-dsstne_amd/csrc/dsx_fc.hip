@@ -173,7 +173,7 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
 
     // Wavefronts in the k-loop go first, wavefronts in the epilogue take the issue slots that are left: the matrix cores then
     // idle less while a workgroup activates and stores its tile (measured 1.5 % on a 1024 x 128 x 27,278 layer).
-    __builtin_amdgcn_s_setprio(3);
+    __builtin_amdgcn_s_setprio(1);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, lhi = lane >> 5;
@@ -445,6 +445,7 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
 template <int S, int ACT>
 __global__ __launch_bounds__(kFcThreads) void fc_small_kernel(FcArgs a)
 {
+    __builtin_amdgcn_s_setprio(3);   // short kernels issue ahead of a GEMM's wavefronts that share their SIMD
     constexpr int T = S / 2;   // MFMA steps per wavefront; lane half h supplies k = base + h * T + t at step t
     __shared__ float sPart[4][16][kWave];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;

@@ -95,6 +95,7 @@ struct SparseZArgs {
 template <typename T, bool BOOLEAN, bool UNITVAL, int VEC, bool FUSED>
 __global__ __launch_bounds__(kSparseThreads) void sparse_z_kernel(SparseZArgs a)
 {
+    __builtin_amdgcn_s_setprio(3);   // short kernels issue ahead of a GEMM's wavefronts that share their SIMD
     __shared__ uint32_t sIdx[kSparseChunk];
     __shared__ float sVal[UNITVAL ? 1 : kSparseChunk];
     __shared__ float sRed[kSparseThreads * VEC];

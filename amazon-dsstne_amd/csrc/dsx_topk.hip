@@ -404,6 +404,7 @@ __device__ __forceinline__ void finish_row(WaveTopK<R>& list, uint64_t (*sStage)
 template <int R, bool FILTERED>
 __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kernel(TopKArgs a)
 {
+    __builtin_amdgcn_s_setprio(3);   // short kernels issue ahead of a GEMM's wavefronts that share their SIMD
     using List = WaveTopK<R>;
     __shared__ uint64_t sStage[kTopkWaves][List::kStageWords];
     extern __shared__ uint32_t sBitmap[];
@@ -674,6 +675,7 @@ constexpr uint32_t kGuidedMaxK = 64;
 template <bool FILTERED, int E>
 __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a)
 {
+    __builtin_amdgcn_s_setprio(3);   // short kernels issue ahead of a GEMM's wavefronts that share their SIMD
     using List = WaveTopK<1>;
     static_assert(E * kTopkThreads <= kGuidedMaxSegs, "at most kGuidedMaxSegs segments");
     __shared__ uint64_t sStage[kTopkWaves][List::kStageWords];
@@ -873,6 +875,7 @@ template <int R>
 __global__ __launch_bounds__(kWave) void topk_merge_kernel(const uint64_t* partial, uint32_t slots, uint32_t k, float* keys,
                                                            uint32_t* values)
 {
+    __builtin_amdgcn_s_setprio(3);   // short kernels issue ahead of a GEMM's wavefronts that share their SIMD
     using List = WaveTopK<R>;
     __shared__ uint64_t sStage[List::kStageWords];
     const uint32_t b = blockIdx.x;
