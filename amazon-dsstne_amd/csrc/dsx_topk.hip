@@ -404,7 +404,6 @@ __device__ __forceinline__ void finish_row(WaveTopK<R>& list, uint64_t (*sStage)
 template <int R, bool FILTERED>
 __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kernel(TopKArgs a)
 {
-    __builtin_amdgcn_s_setprio(3);   // short kernels issue ahead of a GEMM's wavefronts that share their SIMD
     using List = WaveTopK<R>;
     __shared__ uint64_t sStage[kTopkWaves][List::kStageWords];
     extern __shared__ uint32_t sBitmap[];
