@@ -88,6 +88,7 @@ SIGNATURES = {
     "dsx_topk_kv_u32": [_vp, _vp, _vp, _vp, _u32, _u32, _u32],
     "dsx_knn_topk": [_vp, _vp, _vp, _u32, _u32, _u32, _u32],
     "dsx_topk_filtered": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp],
+    "dsx_topk_filtered_static": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp],
     "dsx_topk_guided": [_vp, _vp, _vp, _u32, _u32, _u32, _vp, _u32, _u32, _vp, _vp, _vp, _vp, _vp],
     "dsx_knn_search": [_vp, _u32, _u32, _u32, _vp, _u32, _u32, _vp, _vp, _vp, _sz, C.POINTER(_f32)],
     "dsx_knn_set_block_columns": [_u32],

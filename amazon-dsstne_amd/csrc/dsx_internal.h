@@ -54,11 +54,17 @@ constexpr float kMaxValue = 999999999999999.0f;
 namespace dsx {
 // Top-K building blocks shared with the KNN search (dsx_topk.hip).
 // topk_run: per-row top-k of in[batch][pitch] over the first `width` columns.  With partial != NULL the packed lists go to
-// partial[b][partial_slot0 + segment][k] (forced_segments workgroups per row) instead of keys/values.
+// partial[b][partial_slot0 + segment][k] (forced_segments workgroups per row) instead of keys/values.  With fixed_scratch the
+// lists of rows split over segments go there instead of into memory the library allocates; a call whose lists exceed
+// fixed_scratch_words fails.
 int topk_run(const float* in, uint32_t pitch, uint32_t width, uint32_t batch, uint32_t k, float* keys, uint32_t* values,
              uint32_t position, const uint32_t* index, const uint64_t* fstart, const uint64_t* fend, const uint32_t* fidx,
              const float* fmul, uint32_t col_offset, uint64_t* partial, uint32_t partial_slots, uint32_t partial_slot0,
-             uint32_t forced_segments, uint32_t* row_bound = nullptr);
+             uint32_t forced_segments, uint32_t* row_bound = nullptr, uint64_t* fixed_scratch = nullptr,
+             size_t fixed_scratch_words = 0);
+// Looks up this device's address of the fixed scratch array behind dsx_topk_filtered_static (called by dsx_init with the
+// device current).
+int topk_static_setup(int device);
 int topk_merge(const uint64_t* partial, uint32_t slots, uint32_t k, float* keys, uint32_t* values, uint32_t batch);
 // GEMM building block shared with the KNN search (dsx_fc.hip): Z = X.W (+bias, activation), see dsx_fc_forward.
 int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int transposed, const float* bias, float* Z, uint32_t ldz,

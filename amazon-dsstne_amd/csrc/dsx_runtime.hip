@@ -158,6 +158,7 @@ int dsx_init(int device)
     DSX_HIP(hipGetDeviceProperties(&prop, device));
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return set_error(DSX_EUNSUPPORTED, "dsx_init: device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
+    if (int rc = topk_static_setup(device)) return rc;
     DSX_HIP(hipStreamCreateWithFlags(&c.stream, hipStreamNonBlocking));
     DSX_HIP(hipEventCreate(&c.ev_start));
     DSX_HIP(hipEventCreate(&c.ev_stop));

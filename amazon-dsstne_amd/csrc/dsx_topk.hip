@@ -964,7 +964,7 @@ int topk_merge(const uint64_t* partial, uint32_t slots, uint32_t k, float* keys,
 int topk_run(const float* in, uint32_t pitch, uint32_t width, uint32_t batch, uint32_t k, float* keys, uint32_t* values,
              uint32_t position, const uint32_t* index, const uint64_t* fstart, const uint64_t* fend, const uint32_t* fidx,
              const float* fmul, uint32_t col_offset, uint64_t* partial, uint32_t partial_slots, uint32_t partial_slot0,
-             uint32_t forced_segments, uint32_t* row_bound)
+             uint32_t forced_segments, uint32_t* row_bound, uint64_t* fixed_scratch, size_t fixed_scratch_words)
 {
     const bool filtered = fidx != nullptr;
     TopKArgs a{};
@@ -983,6 +983,9 @@ int topk_run(const float* in, uint32_t pitch, uint32_t width, uint32_t batch, ui
     a.values = values;
     a.row_bound = row_bound;
     a.segments = forced_segments ? forced_segments : choose_segments(batch, width, filtered);
+    if (fixed_scratch && !partial && a.segments > 1 && (size_t)batch * a.segments * k > fixed_scratch_words)
+        return set_error(DSX_EINVAL, "top-K: %u rows x %u segments x k = %u need %zu bytes of partial lists, the fixed scratch holds %zu",
+                         batch, a.segments, k, (size_t)batch * a.segments * k * sizeof(uint64_t), fixed_scratch_words * sizeof(uint64_t));
     const uint32_t nvec_max = width / 4 + 1;
     const uint32_t gps = (nvec_max + a.segments - 1) / a.segments;
     const size_t bitmap_bytes = filtered ? ((size_t)(4 * gps + 8 + 31) / 32) * 4 + 16 : 0;
@@ -991,10 +994,12 @@ int topk_run(const float* in, uint32_t pitch, uint32_t width, uint32_t batch, ui
         a.partial_slots = partial_slots;
         a.partial_slot0 = partial_slot0;
     } else if (a.segments > 1) {
-        uint64_t* scratch = nullptr;
-        int rc = ensure_partial((size_t)batch * a.segments * k * sizeof(uint64_t), &scratch);
-        if (rc) return rc;
-        a.partial = scratch;
+        uint64_t* lists = fixed_scratch;
+        if (!lists) {
+            int rc = ensure_partial((size_t)batch * a.segments * k * sizeof(uint64_t), &lists);
+            if (rc) return rc;
+        }
+        a.partial = lists;
         a.partial_slots = a.segments;
         a.partial_slot0 = 0;
     }
@@ -1106,6 +1111,25 @@ int topk_guided_run(const float* in, uint32_t width, uint32_t batch, uint32_t k,
     return DSX_OK;
 }
 
+// Fixed scratch of dsx_topk_filtered_static: the packed partial lists of rows split over several workgroups,
+// [batch][segments][k] words.  Every device the library runs on holds its own copy of the array at its own address; host code
+// must use the address hipGetSymbolAddress reports for the current device, never the array's name.
+constexpr size_t kStaticScratchWords = (size_t)1 << 21;   // 16 MiB
+static __device__ __align__(256) uint64_t scratch[kStaticScratchWords];
+constexpr int kStaticMaxDevices = 64;
+static uint64_t* g_static_scratch[kStaticMaxDevices] = {};
+
+int topk_static_setup(int device)
+{
+    if (device < 0 || device >= kStaticMaxDevices) return set_error(DSX_EINVAL, "dsx_init: device %d is beyond the %d this library keeps scratch for", device, kStaticMaxDevices);
+    if (g_static_scratch[device]) return DSX_OK;
+    void* p = nullptr;
+    DSX_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return set_error(DSX_EHIP, "dsx_init: the fixed top-K scratch has no device address");
+    g_static_scratch[device] = static_cast<uint64_t*>(p);
+    return DSX_OK;
+}
+
 static int check_topk(const char* fn, const float* in, const float* keys, const void* values, uint32_t width, uint32_t k)
 {
     DSX_CHECK_ARG(in && keys && values, "%s: null device pointer", fn);
@@ -1151,6 +1175,23 @@ int dsx_topk_filtered(const float* in, float* keys, uint32_t* values, uint32_t b
     if (batch == 0) return DSX_OK;
     return topk_run(in, width, width, batch, k, keys, values, position, index, filter_start, filter_end, filter_index, filter_mul, 0,
                     nullptr, 0, 0, 0);
+}
+
+int dsx_topk_filtered_static(const float* in, float* keys, uint32_t* values, uint32_t batch, uint32_t width, uint32_t k, uint32_t position,
+                             const uint32_t* index, const uint64_t* filter_start, const uint64_t* filter_end,
+                             const uint32_t* filter_index, const float* filter_mul)
+{
+    DSX_REQUIRE_INIT();
+    int rc = check_topk("dsx_topk_filtered_static", in, keys, values, width, k);
+    if (rc) return rc;
+    DSX_CHECK_ARG(!filter_index || (filter_start && filter_end), "dsx_topk_filtered_static: filter_index without filter_start / filter_end");
+    uint64_t* lists = g_static_scratch[ctx().device];
+    if (!lists) return set_error(DSX_ENOTINIT, "dsx_topk_filtered_static: no scratch address for device %d", ctx().device);
+    if (batch == 0) return DSX_OK;
+    // Every (row, segment) workgroup writes all k words of its list before the merge reads them: nothing in the scratch has
+    // to start at zero, whatever the previous call left there.
+    return topk_run(in, width, width, batch, k, keys, values, position, index, filter_start, filter_end, filter_index, filter_mul, 0,
+                    nullptr, 0, 0, 0, nullptr, lists, kStaticScratchWords);
 }
 
 int dsx_topk_guided(const float* in, float* keys, uint32_t* values, uint32_t batch, uint32_t width, uint32_t k, const float* seg_max,

@@ -235,6 +235,19 @@ int dsx_topk_filtered(const float* in, float* keys, uint32_t* values, uint32_t b
                       const uint32_t* index, const uint64_t* filter_start, const uint64_t* filter_end, const uint32_t* filter_index,
                       const float* filter_mul);
 
+/* dsx_topk_filtered (filter_index == NULL: unfiltered, as dsx_topk) for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  The call allocates and
+ * frees nothing: the packed partial lists of rows that are split over several workgroups (small batches, or filtered rows
+ * wider than 262,080 columns) go to a fixed 16 MiB array in device memory that every GPU the library runs on holds until the
+ * process ends.  Rows are split as in dsx_topk_filtered: s = ceil(4 x compute units / batch) workgroups per row when the batch
+ * alone does not fill the device (at most width / 8192), and at least ceil(width / 262,080) with a filter.  When
+ * batch x s x k exceeds 2,097,152 words (only possible with a filter over more than 262,080 columns) the
+ * call fails with DSX_EINVAL.  Results are those of dsx_topk_filtered / dsx_topk, bit for bit.  All calls on a GPU share the
+ * one array: calls that overlap on one GPU (the two lanes, several threads) race. */
+int dsx_topk_filtered_static(const float* in, float* keys, uint32_t* values, uint32_t batch, uint32_t width, uint32_t k,
+                             uint32_t position, const uint32_t* index, const uint64_t* filter_start, const uint64_t* filter_end,
+                             const uint32_t* filter_index, const float* filter_mul);
+
 /* Top-K (optionally filtered, as dsx_topk_filtered; filter_index == NULL: unfiltered, as dsx_topk) of a score matrix whose
  * producer left segment maxima (dsx_fc_forward_segmax): same results as the scanning calls, but only the segments that can
  * hold a result are read.  seg_max must describe `in` exactly (same batch rows, seg_width 64); with seg_max == NULL,
