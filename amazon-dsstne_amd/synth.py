@@ -7,6 +7,9 @@ with cuRAND streams that cannot be reproduced, so parity is defined on supplied 
 Weights are N(0, 0.01) read as variance 0.01 (standard deviation 0.1): with a smaller spread every sigmoid output of the
 deep configurations collapses to 0.5 +- 1e-5 and the top-K comparison would only see ties.
 """
+import os
+from concurrent.futures import ThreadPoolExecutor
+
 import numpy as np
 
 from . import (ACT_RELU, ACT_SIGMOID, ATTR_BOOLEAN, ATTR_INDEXED, ATTR_SPARSE, T_FLOAT)
@@ -48,10 +51,41 @@ class Problem:
         return int((self.end[rows] - self.start[rows]).sum())
 
 
+BIG = 1 << 26        # arrays of this many elements or more are drawn chunk by chunk on several threads
+CHUNK = 1 << 24
+
+
+def _threads():
+    return min(16, os.cpu_count() or 4)
+
+
+def normal_f32(rng, shape, scale=1.0):
+    """N(0, scale^2) fp32 array.  Small arrays come straight from `rng`; big ones (config 4's matrices, the KNN table) are drawn
+    in chunks of 2^24 values, each from its own PCG64 stream seeded from `rng`, on several threads: the same bytes for the same
+    seed whatever the number of threads."""
+    n = int(np.prod(shape, dtype=np.int64))
+    if n < BIG:
+        a = rng.standard_normal(shape, dtype=np.float32)
+        if scale != 1.0:
+            a *= np.float32(scale)
+        return a
+    flat = np.empty(n, dtype=np.float32)
+    seeds = rng.integers(0, 1 << 62, size=(n + CHUNK - 1) // CHUNK)
+
+    def fill(i):
+        out = flat[i * CHUNK:(i + 1) * CHUNK]
+        np.random.default_rng(int(seeds[i])).standard_normal(out=out, dtype=np.float32)
+        if scale != 1.0:
+            out *= np.float32(scale)
+    with ThreadPoolExecutor(_threads()) as ex:
+        list(ex.map(fill, range(len(seeds))))
+    return flat.reshape(shape)
+
+
 def make_weights(rng, widths, bias_std=0.0):
     ws, bs = [], []
     for i in range(len(widths) - 1):
-        ws.append((rng.standard_normal((widths[i], widths[i + 1]), dtype=np.float32) * np.float32(WEIGHT_STD)))
+        ws.append(normal_f32(rng, (widths[i], widths[i + 1]), WEIGHT_STD))
         if bias_std > 0:
             bs.append(rng.standard_normal(widths[i + 1], dtype=np.float32) * np.float32(bias_std))
         else:
@@ -173,8 +207,14 @@ class KnnProblem:
         """Item table as KnnData::load builds it (knn/KnnData.cpp:186-207): rows padded to a multiple of 8, column-major."""
         m, d = self.items.shape
         rows = (m + pad_to - 1) // pad_to * pad_to
-        t = np.zeros((d, rows), dtype=np.float32)
-        t[:, :m] = self.items.T
+        t = np.empty((d, rows), dtype=np.float32)
+        t[:, m:] = 0
+        step = 1 << 16
+
+        def block(r0):
+            t[:, r0:min(r0 + step, m)] = self.items[r0:r0 + step].T
+        with ThreadPoolExecutor(_threads()) as ex:
+            list(ex.map(block, range(0, m, step)))
         return t, rows, rows - m
 
 
@@ -183,8 +223,14 @@ def knn_config(seed=1005, items=2000000, queries=4096, dim=256, k=100):
     p = KnnProblem()
     p.name = "cfg5-knn-%dx%d" % (items, dim)
     p.k = k
-    it = rng.standard_normal((items, dim), dtype=np.float32)
-    it /= np.linalg.norm(it, axis=1, keepdims=True)
+    it = normal_f32(rng, (items, dim))
+    step = 1 << 16
+
+    def normalise(r0):
+        blk = it[r0:r0 + step]
+        blk /= np.linalg.norm(blk, axis=1, keepdims=True)
+    with ThreadPoolExecutor(_threads()) as ex:
+        list(ex.map(normalise, range(0, items, step)))
     q = rng.standard_normal((queries, dim), dtype=np.float32)
     q /= np.linalg.norm(q, axis=1, keepdims=True)
     p.items, p.queries = it, q

@@ -1,0 +1,187 @@
+"""Configurations 3, 4 and 5 at their full sizes on the GPU (4,096 x 27,278 analog + indexed; 4,096 x 1,000,000 with top-100;
+KNN 4,096 queries x 2,000,000 items x 256 with top-100).
+
+The CPU oracle cannot run these whole in a test's time, so each test compares a fixed sample of rows / queries with it (first,
+last, the row with the most non-zeros, and 16 spread between) under the parity rules, and checks size-independent properties
+on every row of the batch: scores descending, equal scores in ascending index order, indexes inside the catalogue and
+distinct, no item of a sample's own input returned, and score == activation at the reported index on the sampled rows.
+These shapes are where the kernels' large-size paths run: more than 2^31 elements (16.4 GB) in one unit buffer, filtered rows split over
+four segments plus a merge, candidate lists against million-column ranges.
+"""
+import copy
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from parity import assert_close, assert_topk_parity
+
+pytestmark = pytest.mark.gpu
+
+ATTR_INDEXED = 64
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+
+
+def sample_rows(p, batch, extra=16):
+    """First, last, longest row and `extra` rows spread evenly: batch positions, ascending."""
+    rows = np.arange(batch)
+    actual = p.index[rows] if p.index is not None else rows
+    longest = int(np.argmax(p.end[actual] - p.start[actual]))
+    picks = {0, batch - 1, longest} | {int(x) for x in np.linspace(0, batch - 1, extra + 2)[1:-1]}
+    return np.array(sorted(picks), dtype=np.int64)
+
+
+def oracle_rows(orc, p, picks, k):
+    """The oracle's activations, filtered scores and filtered top-k for batch positions `picks` (a view of the problem whose index
+    array names exactly those rows)."""
+    sub = copy.copy(p)
+    actual = p.index[picks] if p.index is not None else picks
+    sub.index = np.ascontiguousarray(actual, dtype=np.uint32)
+    sub.attributes = p.attributes | ATTR_INDEXED
+    sub.batch = len(picks)
+    _, unit, _, _ = orc.forward(sub, 0, len(picks), k, filtered=False, want_unit=True, want_topk=False)
+    _, _, keys, idx = orc.forward(sub, 0, len(picks), k, filtered=True)
+    scores = unit.copy()
+    orc.lib().orc_apply_filter(scores.ctypes.data, len(picks), scores.shape[1], 0, 0, sub.index.ctypes.data, p.start.ctypes.data,
+                               p.end.ctypes.data, p.sparse_index.ctypes.data, None)
+    return unit, scores, keys, idx
+
+
+def download_rows(pkg, dsx, unit_dev, width, picks):
+    out = np.empty((len(picks), width), dtype=np.float32)
+    for i, b in enumerate(picks):
+        pkg.check(dsx.dsx_memcpy_d2h(out[i].ctypes.data, unit_dev.ptr + int(b) * width * 4, width * 4))
+    return out
+
+
+def check_batch_properties(p, keys, idx, filtered_rows=True):
+    batch, k = keys.shape
+    width = p.widths[-1]
+    assert np.all(idx < width), "an index lies outside the catalogue"
+    d = np.diff(keys.astype(np.float64), axis=1)
+    assert np.all(d <= 0), "scores are not descending in %d places" % int((d > 0).sum())
+    same = d == 0
+    if same.any():
+        assert np.all(np.diff(idx.astype(np.int64), axis=1)[same] > 0), "equal scores are not in ascending index order"
+    srt = np.sort(idx, axis=1)
+    assert np.all(srt[:, 1:] != srt[:, :-1]), "an index is reported twice in a row"
+    assert np.all(keys > -1e14), "unfilled slots in a row with more candidates than k"
+    if filtered_rows:
+        rows = np.arange(batch)
+        actual = p.index[rows] if p.index is not None else rows
+        for b in range(batch):
+            own = p.sparse_index[int(p.start[actual[b]]):int(p.end[actual[b]])]
+            assert not np.isin(idx[b], own).any(), "row %d: an item of the sample's own input came back" % b
+
+
+def run_network_config(pkg, dsx, orc, p, guided):
+    from amazon_dsstne_amd.pipeline import DevicePipeline
+    B, N, k = p.batch, p.widths[-1], p.k
+    pipe = DevicePipeline(p, dsx, guided=guided)
+    pipe.step()
+    keys, idx = pipe.results()
+    picks = sample_rows(p, B)
+    say("%s: %d x %d, k = %d, %d sampled rows (longest has %d non-zeros), guided = %s" % (
+        p.name, B, N, k, len(picks), int((p.end - p.start).max()), guided))
+    check_batch_properties(p, keys, idx)
+    ref_unit, ref_scores, ref_keys, ref_idx = oracle_rows(orc, p, picks, k)
+    unit = download_rows(pkg, dsx, pipe.units[-1], N, picks)
+    assert_close(unit, ref_unit, "%s output activations of the sampled rows" % p.name, rel=1e-4, abs_floor=1e-3)
+    assert np.array_equal(unit[np.arange(len(picks))[:, None], idx[picks]], keys[picks]), "score is not the activation at the reported index"
+    n = assert_topk_parity(keys[picks], idx[picks], ref_keys, ref_idx, ref_scores, p.name)
+    say("%s: sampled rows agree with the oracle (%d tie-equivalent index differences)" % (p.name, n))
+    return pipe, keys, idx
+
+
+def test_cfg3_full_size(pkg, dsx, orc, synth):
+    p = synth.config(3)
+    _, k_scan, i_scan = run_network_config(pkg, dsx, orc, p, guided=False)
+    _, k_gd, i_gd = run_network_config(pkg, dsx, orc, p, guided=True)
+    assert np.array_equal(i_gd, i_scan) and np.array_equal(k_gd.view(np.uint32), k_scan.view(np.uint32)), "guided and scanning top-K differ"
+
+
+def test_cfg3_full_size_through_host_layer(pkg, dsx, orc, synth):
+    # the same configuration through NNNetwork::PredictBatch + CalculateFilteredTopK (what bench.py times)
+    from amazon_dsstne_amd.host_api import Network
+    p = synth.config(3)
+    net = Network(p)
+    try:
+        net.bind_input()
+        net.predict_batch(0)
+        net.topk(p.k, filter_dataset=net.dataset)
+        keys, idx = net.get_topk(p.batch, p.k)
+        check_batch_properties(p, keys, idx)
+        picks = sample_rows(p, p.batch)
+        _, ref_scores, ref_keys, ref_idx = oracle_rows(orc, p, picks, p.k)
+        assert_topk_parity(keys[picks], idx[picks], ref_keys, ref_idx, ref_scores, p.name + " (host layer)")
+    finally:
+        net.close()
+
+
+def test_cfg4_full_size(pkg, dsx, orc, synth):
+    p = synth.config(4)
+    assert p.batch * p.widths[-1] > 1 << 31      # element offsets do not fit a signed 32-bit integer, byte offsets no 32-bit one
+    pipe, keys, idx = run_network_config(pkg, dsx, orc, p, guided=False)
+    # the unfiltered top-100 of the same activations on the sampled rows: one segment per row, no merge
+    picks = sample_rows(p, p.batch)
+    pipe.topk(filtered=False)
+    uk, ui = pipe.results()
+    unit = download_rows(pkg, dsx, pipe.units[-1], p.widths[-1], picks)
+    rk, ri = orc.topk(unit, p.k)
+    assert np.array_equal(ui[picks], ri) and np.array_equal(uk[picks].view(np.uint32), rk.view(np.uint32)), "unfiltered top-100 differs"
+    check_batch_properties(p, uk, ui, filtered_rows=False)
+
+
+def test_cfg5_knn_full_size(pkg, dsx, orc, synth):
+    p = synth.knn_config()
+    Q, D = p.queries.shape
+    M = p.items.shape[0]
+    k = p.k
+    table, rows_padded, padding = p.column_major_padded()
+    d_items = pkg.DeviceArray.from_numpy(table)
+    d_q = pkg.DeviceArray.from_numpy(p.queries)
+    scores = pkg.DeviceArray((Q, k), np.float32)
+    idx = pkg.DeviceArray((Q, k), np.uint32)
+    pkg.check(dsx.dsx_knn_search(d_items.ptr, rows_padded, padding, D, d_q.ptr, Q, k, scores.ptr, idx.ptr, None, 0, None))
+    path = dsx.dsx_knn_last_search_path()
+    s, i = scores.numpy(), idx.numpy()
+    say("cfg5: %d queries x %d items x %d, k = %d, search path %d" % (Q, M, D, k, path))
+    assert path == 1, "the search was expected to run with candidate lists (path 1), ran path %d" % path
+    # every query: order, range, distinct, and the reported score is the dot product with the reported item
+    assert np.all(i < M)
+    d = np.diff(s.astype(np.float64), axis=1)
+    assert np.all(d <= 0)
+    if (d == 0).any():
+        assert np.all(np.diff(i.astype(np.int64), axis=1)[d == 0] > 0)
+    srt = np.sort(i, axis=1)
+    assert np.all(srt[:, 1:] != srt[:, :-1])
+    for q0 in range(0, Q, 256):
+        dots = np.einsum("qkd,qd->qk", p.items[i[q0:q0 + 256]].astype(np.float64), p.queries[q0:q0 + 256].astype(np.float64))
+        assert np.abs(dots - s[q0:q0 + 256]).max() < 2e-6, "a reported score is not the dot product with the reported item"
+    # sampled queries against the oracle's exact search over all items
+    picks = np.array(sorted({0, Q - 1} | {int(x) for x in np.linspace(0, Q - 1, 18)[1:-1]}), dtype=np.int64)
+    rs, ri = orc.knn_search(table, rows_padded, padding, D, p.queries[picks], k)
+    mism = i[picks] != ri
+    if mism.any():   # only inside near-ties of the oracle's own scores
+        gap = np.abs(s[picks][mism].astype(np.float64) - rs[mism].astype(np.float64))
+        assert gap.max() < 1e-5, "KNN indexes differ from the oracle outside near-ties (gap %g)" % gap.max()
+    assert_close(s[picks], rs, "cfg5 scores of the sampled queries", rel=1e-4)
+    say("cfg5: sampled queries agree with the oracle (%d tie-equivalent index differences)" % int(mism.sum()))
+    # fp16 storage on the same table: same checks against fp16-rounded operands for the sampled queries
+    f16_bytes = dsx.dsx_knn_f16_table_bytes(rows_padded, D)
+    t16 = pkg.DeviceArray((f16_bytes,), np.uint8)
+    pkg.check(dsx.dsx_knn_f16_convert_items(d_items.ptr, rows_padded, padding, D, t16.ptr))
+    pkg.check(dsx.dsx_knn_search_f16(t16.ptr, rows_padded, padding, D, d_q.ptr, Q, k, scores.ptr, idx.ptr, None, 0, None))
+    s16, i16 = scores.numpy(), idx.numpy()
+    assert np.all(i16 < M) and np.all(np.diff(s16.astype(np.float64), axis=1) <= 0)
+    tq = p.queries[picks].astype(np.float16).astype(np.float32)
+    table16 = table.astype(np.float16).astype(np.float32)
+    rs16, ri16 = orc.knn_search(table16, rows_padded, padding, D, tq, k)
+    mism = i16[picks] != ri16
+    if mism.any():
+        gap = np.abs(s16[picks][mism].astype(np.float64) - rs16[mism].astype(np.float64))
+        assert gap.max() < 1e-5, "fp16 KNN indexes differ from the oracle outside near-ties (gap %g)" % gap.max()
+    assert_close(s16[picks], rs16, "cfg5 fp16-storage scores of the sampled queries", rel=1e-4)
