@@ -63,6 +63,7 @@ SIGNATURES = {
     "dsx_sync": [],
     "dsx_set_lane": [_int],
     "dsx_get_lane": [],
+    "dsx_sync_lane": [_int],
     "dsx_memcpy_d2h_lane": [_int, _vp, _vp, _sz],
     "dsx_memcpy_d2h_pair": [_vp, _vp, _sz, _vp, _vp, _sz],
     "dsx_memcpy_h2d_unordered": [_vp, _vp, _sz],

@@ -86,8 +86,8 @@ __device__ __forceinline__ uint32_t candidate_bound_prefetch(const CandArgs& c, 
 // lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32): the tile is only compared with the rows' admission bounds.  A bound is the key
 // of a score that k items seen earlier reach, so a lane usually ends after its MI * NI * 16 compares.  The bounds of the
 // tile's 32*MI*WM rows are staged in LDS as floats (`lds`: kCandLdsBytes of workgroup memory that is free by now), four
-// consecutive rows per 128-bit read; "not (x < bound)" also lets NaN scores and a few scores whose key is below the bound's
-// through, which the merge of the lists sorts out.  A wavefront with survivors first gathers them in a list in LDS and
+// consecutive rows per 128-bit read; "x >= bound" as floats lets a few scores through whose key is below the bound's (-0.0
+// against +0.0), which the merge of the lists sorts out, and keeps NaN scores out, as the scanning top-K does.  A wavefront with survivors first gathers them in a list in LDS and
 // then appends the whole list to the rows' global lists, one atomic per survivor but all of them in flight together: asked
 // for one by one, each atomic's round trip (thousands of cycles) would be waited for separately.
 // bound_key is what candidate_bound_prefetch returned to this lane.  Every lane of the workgroup must call this.
@@ -101,7 +101,8 @@ __device__ __forceinline__ void candidate_epilogue(const floatx16 (&acc)[MI][NI]
 {
     constexpr int BM = 32 * MI * WM;   // at most as many rows as the workgroup has lanes
     float* sBound = lds;
-    if (tid < BM) sBound[tid] = (row0 + tid < batch) ? key_score(bound_key) : __builtin_inff();
+    // key 0: no bound yet (fewer than k items seen), every score that is a number is admitted
+    if (tid < BM) sBound[tid] = (row0 + tid < batch) ? (bound_key ? key_score(bound_key) : -__builtin_inff()) : __builtin_inff();
     __syncthreads();
     float bf[MI][4][4];
 #pragma unroll
@@ -121,7 +122,7 @@ __device__ __forceinline__ void candidate_epilogue(const floatx16 (&acc)[MI][NI]
         for (int j = 0; j < NI; j++) {
             uint64_t m = 0;
 #pragma unroll
-            for (int v = 0; v < 16; v++) m |= __builtin_amdgcn_ballot_w64(!(acc[i][j][v] < bf[i][v / 4][v % 4]));
+            for (int v = 0; v < 16; v++) m |= __builtin_amdgcn_ballot_w64(acc[i][j][v] >= bf[i][v / 4][v % 4]);
             block_mask[i][j] = m;
             any_mask |= m;
         }
@@ -160,7 +161,7 @@ __device__ __forceinline__ void candidate_epilogue(const floatx16 (&acc)[MI][NI]
             for (int v = 0; v < 16; v++) {
                 float x = acc[i][j][v];
                 asm volatile("" : "+v"(x));   // compared afresh: results kept from the pass above would cost more than they save
-                const uint64_t mask = __builtin_amdgcn_ballot_w64(!(x < bf[i][v / 4][v % 4]) && col_ok);
+                const uint64_t mask = __builtin_amdgcn_ballot_w64(x >= bf[i][v / 4][v % 4] && col_ok);
                 if (mask == 0) continue;
                 const bool cand = (mask >> lane) & 1;
                 const uint32_t r = row0 + wm * 32 * MI + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);

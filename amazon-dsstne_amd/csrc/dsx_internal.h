@@ -20,6 +20,17 @@ struct Context {
 };
 
 Context& ctx();
+
+// Device memory the library allocates for itself (split top-K lists, KNN workspace): grown on demand, counted by
+// dsx_get_memory_usage, released by dsx_shutdown.
+struct LibScratch {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+    bool listed = false;
+};
+// Makes s hold at least `bytes` (contents are not preserved when it grows; the selected lane is waited for before the old
+// block is freed).
+int lib_scratch_reserve(LibScratch& s, size_t bytes, const char* what);
 int current_lane();   // 0 or 1: which of the two in-order streams ctx().stream is (scratch buffers are kept per lane)
 int set_error(int code, const char* fmt, ...);
 

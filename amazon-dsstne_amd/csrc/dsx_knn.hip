@@ -8,8 +8,8 @@
 // the query's best list and raises its bound.  Results are exact for any input: a list that fills up (items sorted by
 // score, say) raises a flag that the host reads at the end, and the search is then redone block by block — GEMM into the
 // scratch matrix, scanning top-K into packed partial lists with the running bound, one merge — which is also the path
-// taken while the stream is being captured into a graph (no host read-back there) and for operands that are not 16-byte
-// aligned.  With fp16 storage (dsx_knn_search_f16) the scores come from the f16 MFMA kernel of dsx_knn_f16.hip instead, through
+// taken while the stream is being captured into a graph (no host read-back there; the caller then passes its own workspace,
+// the library's would have to be allocated inside the capture) and for operands that are not 16-byte aligned.  With fp16 storage (dsx_knn_search_f16) the scores come from the f16 MFMA kernel of dsx_knn_f16.hip instead, through
 // the same three steps.
 #include <algorithm>
 #include <hip/hip_runtime.h>
@@ -18,8 +18,7 @@
 
 namespace dsx {
 
-static void* g_knn_ws_of[2] = {nullptr, nullptr};   // per lane
-static size_t g_knn_ws_bytes_of[2] = {0, 0};
+static LibScratch g_knn_ws_of[2];   // per lane
 
 static uint32_t g_knn_block_columns = 0;   // 0: sized by the rule below
 static int g_knn_last_path = 0;            // how the last search ran: DSX_KNN_PATH_*
@@ -36,7 +35,7 @@ static uint32_t knn_block_columns(uint32_t rows_padded, uint32_t num_queries)
 
 static inline size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 
-// a fill kernel rather than hipMemsetAsync: callers may record the search into a HIP graph
+// a fill kernel rather than hipMemsetAsync (memset nodes of a captured graph are not trusted on this hardware pool)
 __global__ __launch_bounds__(256) void knn_clear_kernel(uint32_t* p, uint32_t n)
 {
     const uint32_t i = blockIdx.x * 256 + threadIdx.x;
@@ -115,7 +114,7 @@ struct KnnTimer {
     }
 };
 
-// Block by block through the scratch score matrix; exact for any input, usable under stream capture.
+// Block by block through the scratch score matrix; exact for any input, no host read-back.
 static int knn_search_blocks(const KnnWorkspace& w, const KnnOperands& op, uint32_t M, uint32_t num_queries, uint32_t k, float* scores,
                              uint32_t* indexes, KnnTimer& t)
 {
@@ -232,20 +231,9 @@ static int knn_search_common(KnnOperands& op, uint32_t padding, uint32_t num_que
         DSX_CHECK_ARG(workspace_bytes >= need, "dsx_knn_search: workspace of %zu bytes, %zu needed", workspace_bytes, need);
         DSX_CHECK_ARG(((uintptr_t)workspace % 256) == 0, "dsx_knn_search: workspace is not 256-byte aligned");
     } else {
-        void*& g_knn_ws = g_knn_ws_of[current_lane()];
-        size_t& g_knn_ws_bytes = g_knn_ws_bytes_of[current_lane()];
-        if (g_knn_ws_bytes < need) {
-            if (g_knn_ws) {
-                DSX_HIP(hipStreamSynchronize(ctx().stream));
-                DSX_HIP(hipFree(g_knn_ws));
-                g_knn_ws = nullptr;
-                g_knn_ws_bytes = 0;
-            }
-            hipError_t e = hipMalloc(&g_knn_ws, need);
-            if (e != hipSuccess) return set_error(DSX_ENOMEM, "dsx_knn_search: cannot allocate %zu bytes of workspace: %s", need, hipGetErrorString(e));
-            g_knn_ws_bytes = need;
-        }
-        workspace = g_knn_ws;
+        LibScratch& ws = g_knn_ws_of[current_lane()];
+        if (int rc = lib_scratch_reserve(ws, need, "dsx_knn_search workspace")) return rc;
+        workspace = ws.ptr;
     }
     const KnnWorkspace w = knn_layout(workspace, op.rows_padded, num_queries, k, op.f16, op.dim);
     const uint32_t M = op.rows_padded - padding;

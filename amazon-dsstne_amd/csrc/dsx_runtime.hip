@@ -2,6 +2,7 @@
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <vector>
 #include "dsx_internal.h"
 
 namespace dsx {
@@ -26,6 +27,42 @@ int set_error(int code, const char* fmt, ...)
 static std::mutex g_alloc_mutex;
 static std::map<void*, size_t> g_device_allocs;
 static std::map<void*, size_t> g_host_allocs;
+
+static std::vector<LibScratch*> g_lib_scratch;
+
+int lib_scratch_reserve(LibScratch& s, size_t bytes, const char* what)
+{
+    if (bytes <= s.bytes) return DSX_OK;
+    std::lock_guard<std::mutex> lock(g_alloc_mutex);
+    if (s.ptr) {
+        DSX_HIP(hipStreamSynchronize(ctx().stream));
+        DSX_HIP(hipFree(s.ptr));
+        ctx().gpu_bytes -= s.bytes;
+        s.ptr = nullptr;
+        s.bytes = 0;
+    }
+    hipError_t e = hipMalloc(&s.ptr, bytes);
+    if (e != hipSuccess) {
+        s.ptr = nullptr;
+        return set_error(DSX_ENOMEM, "%s: cannot allocate %zu bytes: %s", what, bytes, hipGetErrorString(e));
+    }
+    s.bytes = bytes;
+    ctx().gpu_bytes += bytes;
+    if (!s.listed) {
+        s.listed = true;
+        g_lib_scratch.push_back(&s);
+    }
+    return DSX_OK;
+}
+
+static void lib_scratch_release()
+{
+    for (LibScratch* s : g_lib_scratch) {
+        if (s->ptr) hipFree(s->ptr);
+        s->ptr = nullptr;
+        s->bytes = 0;
+    }
+}
 
 }  // namespace dsx
 
@@ -181,6 +218,7 @@ int dsx_shutdown(void)
     upload_ring_release();
     {
         std::lock_guard<std::mutex> lock(g_alloc_mutex);
+        lib_scratch_release();
         for (auto& kv : g_device_allocs) hipFree(kv.first);
         for (auto& kv : g_host_allocs) hipHostFree(kv.first);
         g_device_allocs.clear();
@@ -455,6 +493,15 @@ int dsx_sync(void)
     DSX_REQUIRE_INIT();
     if (other_lane_stream()) DSX_HIP(hipStreamSynchronize(other_lane_stream()));
     DSX_HIP(hipStreamSynchronize(ctx().stream));
+    return DSX_OK;
+}
+
+int dsx_sync_lane(int lane)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(lane == 0 || lane == 1, "dsx_sync_lane: lane %d (0 or 1)", lane);
+    hipStream_t s = g_lane_stream[lane] ? g_lane_stream[lane] : ctx().stream;
+    DSX_HIP(hipStreamSynchronize(s));
     return DSX_OK;
 }
 

@@ -383,7 +383,7 @@ int dsx_load_sparse_input_unit(uint32_t attributes, uint32_t data_type, uint32_t
     if (!(attributes & DSX_ATTR_INDEXED)) index = nullptr;
     if (!(attributes & DSX_ATTR_WEIGHTED)) data_weight = nullptr;
     hipStream_t s = ctx().stream;
-    // zero fill by kernel (not hipMemsetAsync) so the call can be recorded into a HIP graph
+    // zero fill by kernel rather than hipMemsetAsync (memset nodes of a captured graph are not trusted on this hardware pool)
     uint64_t size = (uint64_t)batch * stride;
     hipLaunchKernelGGL(clear_unit_kernel, dim3(grid_for(size, 256, 4)), dim3(256), 0, s, unit, nullptr, nullptr, nullptr, nullptr, 0u,
                        stride, size);

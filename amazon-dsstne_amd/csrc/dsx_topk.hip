@@ -904,25 +904,13 @@ __global__ __launch_bounds__(256) void topk_gather_kernel(const V* in_values, V*
     values[pos] = (j < width) ? in_values[(uint64_t)b * width + col] : (V)0;
 }
 
-static uint64_t* g_partial_of[2] = {nullptr, nullptr};   // per lane: two lanes may run a split top-K at the same time
-static size_t g_partial_bytes_of[2] = {0, 0};
+static LibScratch g_partial_of[2];   // per lane: two lanes may run a split top-K at the same time
 
 static int ensure_partial(size_t bytes, uint64_t** out)
 {
-    uint64_t*& buf = g_partial_of[current_lane()];
-    size_t& have = g_partial_bytes_of[current_lane()];
-    if (bytes > have) {
-        if (buf) {
-            DSX_HIP(hipStreamSynchronize(ctx().stream));
-            DSX_HIP(hipFree(buf));
-            buf = nullptr;
-            have = 0;
-        }
-        hipError_t e = hipMalloc((void**)&buf, bytes);
-        if (e != hipSuccess) return set_error(DSX_ENOMEM, "top-K: cannot allocate %zu bytes for partial lists: %s", bytes, hipGetErrorString(e));
-        have = bytes;
-    }
-    *out = buf;
+    LibScratch& buf = g_partial_of[current_lane()];
+    if (int rc = lib_scratch_reserve(buf, bytes, "top-K partial lists")) return rc;
+    *out = static_cast<uint64_t*>(buf.ptr);
     return DSX_OK;
 }
 

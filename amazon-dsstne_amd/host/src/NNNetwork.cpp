@@ -470,6 +470,11 @@ NNFloat* NNNetwork::GetUnitBuffer(const string& layer)
     }
     // the caller gets a writable device pointer: the segment maxima of the batch may not describe the units any longer
     itr->second->_segWidth = 0;
+    // The reference's callers follow this call with a plain cudaMemcpy or a kernel of their own
+    // (utils/NNRecsGenerator.cpp:83, java/src/main/native/com_amazon_dsstne_Dsstne.cpp:366), which the default stream ordered
+    // after the forward pass.  The lanes' streams are not ordered against the null stream, so the batch that filled this
+    // buffer is waited for here; a batch in flight on the other lane keeps running.
+    dsxFatal(dsx_sync_lane((int)_lane), "NNNetwork::GetUnitBuffer");
     return itr->second->GetUnitBuffer();
 }
 

@@ -404,6 +404,15 @@ int dsstne_get_units(dsstne_context* c, const char* layer, float* units, size_t 
     CAPI_CATCH(-1)
 }
 
+void* dsstne_get_unit_buffer(dsstne_context* c, const char* layer)
+{
+    CAPI_TRY
+    NNFloat* p = c->net()->GetUnitBuffer(layer);
+    if (!p) fail("dsstne_get_unit_buffer: layer %s is unknown or has no unit buffer", layer);
+    return (void*)p;
+    CAPI_CATCH(NULL)
+}
+
 int dsstne_set_units(dsstne_context* c, const char* layer, const float* units, size_t count)
 {
     CAPI_TRY

@@ -29,6 +29,7 @@ SIGNATURES = {
     "dsstne_get_topk": ([_vp, _cp, _u32, _u32, _vp, _vp], _int),
     "dsstne_predict": ([_vp, _cp, _u32, _cp, _vp, _vp], _int),
     "dsstne_get_units": ([_vp, _cp, _vp, _sz], _int),
+    "dsstne_get_unit_buffer": ([_vp, _cp], _vp),
     "dsstne_set_units": ([_vp, _cp, _vp, _sz], _int),
     "dsstne_sync": ([], _int),
     "dsstne_timer_start": ([], _int),
@@ -159,6 +160,13 @@ class Network:
         out = np.empty((rows, width), dtype=np.float32)
         _check(self.lib.dsstne_get_units(self.ctx, layer.encode(), out.ctypes.data, out.size))
         return out
+
+    def unit_buffer(self, layer="Output"):
+        """Device address of the layer's activations of the batch predicted last (NNNetwork::GetUnitBuffer)."""
+        ptr = self.lib.dsstne_get_unit_buffer(self.ctx, layer.encode())
+        if not ptr:
+            raise DsxError("dsstne_get_unit_buffer failed: %s" % self.lib.dsstne_last_error().decode())
+        return ptr
 
     def set_units(self, values, layer="Output"):
         values = np.ascontiguousarray(values, dtype=np.float32)

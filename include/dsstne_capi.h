@@ -91,6 +91,11 @@ int dsstne_set_lanes(dsstne_context* ctx, uint32_t lanes);
 int dsstne_predict(dsstne_context* ctx, const char* layer, uint32_t k, const char* filter_dataset, float* scores, uint32_t* indexes);
 /* NNLayer::GetUnits: the layer's [batch][width] activations. */
 int dsstne_get_units(dsstne_context* ctx, const char* layer, float* units, size_t count);
+/* NNNetwork::GetUnitBuffer (engine/NNNetwork.cpp:2006-2020): device address of the layer's [batch][stride] activations of the
+ * batch predicted last, as the reference's JNI predict takes it (Dsstne.cpp:366).  The call returns once that batch's
+ * forward pass has finished on the device, so the caller may read the memory with any copy or kernel of its own; the
+ * address changes from batch to batch with two lanes (fetch it per batch, as the reference's callers do).  NULL on failure. */
+void* dsstne_get_unit_buffer(dsstne_context* ctx, const char* layer);
 /* NNLayer::SetUnits (engine/NNLayer.cpp:318-368 group): overwrites the layer's unit buffer (batch x stride values) from the host. */
 int dsstne_set_units(dsstne_context* ctx, const char* layer, const float* units, size_t count);
 int dsstne_sync(void);

@@ -3,8 +3,13 @@
  *
  * Plain pointers and sizes only.  Every pointer named "device" is an address in HBM obtained from dsx_malloc (or any
  * other HIP allocation of the same process).  All functions return 0 on success and a negative DSX_E* code on failure;
- * dsx_last_error() then returns a message for the calling thread.  Kernels are enqueued on one library-owned HIP
- * stream and return without waiting; dsx_sync() (or any dsx_memcpy_d2h) waits for them.
+ * dsx_last_error() then returns a message for the calling thread.  Kernels are enqueued on a library-owned HIP stream
+ * (created non-blocking: work on the null stream is NOT ordered against it) and return without waiting; dsx_sync() (or any
+ * dsx_memcpy_d2h) waits for them.  A caller that touches device memory with its own kernels or copies calls dsx_sync (or
+ * dsx_sync_lane) first.
+ *
+ * Thread safety: like the reference's GpuContext, the library keeps one context per process (selected lane, staging ring,
+ * scratch buffers) without locks around it; calls must come from one thread at a time.  Only dsx_last_error is per thread.
  *
  * Each entry point cites the function of the reference (paths relative to the reference root,
  * engine/ = src/amazon/dsstne/engine/, knn/ = src/amazon/dsstne/knn/, utils/ = src/amazon/dsstne/utils/)
@@ -121,6 +126,7 @@ int dsx_sync(void);                                                          /* 
  * themselves, dsx_memcpy_d2h and dsx_sync wait for both, dsx_memcpy_d2h_lane for one lane only. */
 int dsx_set_lane(int lane);
 int dsx_get_lane(void);
+int dsx_sync_lane(int lane);   /* waits for everything queued on one lane (before the second lane exists: on the only stream) */
 int dsx_memcpy_d2h_lane(int lane, void* host_dst, const void* device_src, size_t bytes);
 /* For data that arrives batch by batch (no counterpart in the reference, whose uploads block).  dsx_memcpy_h2d_unordered is
  * dsx_memcpy_h2d on the selected lane only: the other lane is neither waited for nor told to wait, so the copy overlaps with

@@ -653,6 +653,40 @@ def test_knn_search_full_candidate_list_falls_back(pkg, dsx, orc, rng, small_knn
     assert got_i[0].min() >= items - 2 * k and got_i[1].max() < 2 * k
 
 
+def test_knn_search_nan_scores_never_returned_on_either_path(pkg, dsx, orc, synth):
+    """Items with a NaN component score NaN against every query.  The scanning top-K drops NaN; the candidate lists must do the
+    same, so both ways of running the search give the same bits and never name such an item."""
+    p = synth.knn_config(seed=11, items=20000, queries=24, dim=32, k=50)
+    bad = np.arange(7, 20000, 13)
+    p.items[bad, 5] = np.nan
+    dsx.dsx_knn_set_block_columns(1024)
+    try:
+        cs, ci, _, _, _ = knn_case(pkg, dsx, orc, p.items, p.queries, 50)
+        assert dsx.dsx_knn_last_search_path() == 1
+    finally:
+        dsx.dsx_knn_set_block_columns(0)
+    bs, bi, _, _, _ = knn_case(pkg, dsx, orc, p.items, p.queries, 50)
+    assert dsx.dsx_knn_last_search_path() == 0
+    assert np.array_equal(ci, bi) and np.array_equal(cs.view(np.uint32), bs.view(np.uint32))
+    assert not np.isin(ci, bad).any() and not np.isnan(cs).any()
+
+
+def test_library_scratch_is_counted_and_released(pkg, dsx, rng):
+    """Memory the library allocates for itself (here the partial lists of a split top-K) shows up in dsx_get_memory_usage."""
+    g0, g1 = C.c_int(), C.c_int()
+    scores = pkg.DeviceArray.from_numpy(rng.random((3, 1 << 20), dtype=np.float32))
+    keys = pkg.DeviceArray((3, 256), np.float32)
+    vals = pkg.DeviceArray((3, 256), np.uint32)
+    pkg.check(dsx.dsx_get_memory_usage(C.byref(g0), None))
+    for lane in (0, 1):
+        pkg.check(dsx.dsx_set_lane(lane))
+        pkg.check(dsx.dsx_topk(scores.ptr, keys.ptr, vals.ptr, 3, 1 << 20, 256))
+    pkg.check(dsx.dsx_set_lane(0))
+    pkg.check(dsx.dsx_sync())
+    pkg.check(dsx.dsx_get_memory_usage(C.byref(g1), None))
+    assert g1.value >= g0.value            # lists of this size may already exist from an earlier test; never less
+
+
 def test_knn_search_unaligned_dim_takes_block_path(pkg, dsx, orc, synth, small_knn_blocks):
     p = synth.knn_config(seed=9, items=5000, queries=17, dim=30, k=20)      # 30 floats per row: no 128-bit loads
     got_s, got_i, ref_s, ref_i, _ = knn_case(pkg, dsx, orc, p.items, p.queries, 20)

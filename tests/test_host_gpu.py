@@ -444,3 +444,35 @@ def test_two_lanes_keep_batches_apart(pkg, dsx, orc, synth, config, batches):
         assert_topk_parity(gk, gi, want[0][1], want[0][2], want[0][3], p.name + " back on two lanes")
     finally:
         net.close()
+
+
+def test_unit_buffer_read_with_a_bare_hipmemcpy(pkg, dsx, orc, synth):
+    """The reference's callers follow PredictBatch with GetUnitBuffer and a plain cudaMemcpy on the default stream
+    (utils/NNRecsGenerator.cpp:83, java/src/main/native/com_amazon_dsstne_Dsstne.cpp:366).  The same pattern with hipMemcpy from the
+    HIP runtime itself, not through this library: every batch read this way must be that batch's finished activations, on two
+    lanes (the pointer alternates between two buffers) and on one."""
+    import ctypes as C
+    from amazon_dsstne_amd import host_api
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+    hip.hipMemcpy.restype = C.c_int
+    p = synth.config(2, batches=3)
+    N = p.widths[-1]
+    refs = [orc.forward(p, pos, p.batch, filtered=False, want_unit=True, want_topk=False)[1] for pos in (0, p.batch, 2 * p.batch)]
+    net = host_api.Network(p, max_k=p.k)
+    try:
+        net.bind_input()
+        for lanes in (2, 1):
+            net.set_lanes(lanes)
+            seen = set()
+            for rep in range(2):
+                for n, pos in enumerate((0, p.batch, 2 * p.batch)):
+                    net.predict_batch(pos)
+                    ptr = net.unit_buffer("Output")
+                    seen.add(ptr)
+                    got = np.empty((p.batch, N), dtype=np.float32)
+                    assert hip.hipMemcpy(got.ctypes.data, ptr, got.nbytes, 2) == 0     # hipMemcpyDeviceToHost, null stream
+                    assert_close(got, refs[n], "units of batch %d read with hipMemcpy (%d lanes)" % (n, lanes), rel=1e-4, abs_floor=1e-3)
+            assert len(seen) == lanes
+    finally:
+        net.close()
