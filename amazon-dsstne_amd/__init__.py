@@ -91,6 +91,11 @@ SIGNATURES = {
     "dsx_topk_filtered": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp],
     "dsx_topk_filtered_static": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp],
     "dsx_topk_guided": [_vp, _vp, _vp, _u32, _u32, _u32, _vp, _u32, _u32, _vp, _vp, _vp, _vp, _vp],
+    "dsx_fc_topk": [_vp, _u32, _vp, _vp, _u32, _u32, _u32, _u32, C.POINTER(ActParams), _u32, _vp, _vp, _u32, _vp, _vp, _vp, _vp],
+    "dsx_fc_topk_supported": [_u32, _vp, _u32, C.POINTER(ActParams), _vp],
+    "dsx_fc_topk_flagged": [_int],
+    "dsx_fc_topk_set_first_columns": [_u32],
+    "dsx_fc_topk_set_candidate_capacity": [_u32],
     "dsx_knn_search": [_vp, _u32, _u32, _u32, _vp, _u32, _u32, _vp, _vp, _vp, _sz, C.POINTER(_f32)],
     "dsx_knn_set_block_columns": [_u32],
     "dsx_knn_f16_convert_items": [_vp, _u32, _u32, _u32, _vp],

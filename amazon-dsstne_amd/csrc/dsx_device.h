@@ -70,7 +70,53 @@ struct CandArgs {
     uint32_t cand_cap;
     uint32_t col_offset;
     uint32_t* overflow;
+    // Layer mode (template flag PRE of candidate_epilogue): the accumulators hold pre-activation sums z (bias included), the
+    // bounds are keys of activated scores; see preactivation_bound.
+    uint32_t act;
+    float slope, alpha, lambda;
 };
+
+// Layer mode of the candidate epilogue.  The k-th best score B of a row is known as an activated value, the tile holds
+// pre-activation sums z.  For a non-decreasing activation every z with act(z) >= B lies above any point zb with
+// act(zb) < B, so "z >= zb" admits a superset of what "act(z) >= B" admits, and only the few survivors are activated.  zb is
+// found by inverting the activation a little below B and stepping down until the activation, evaluated exactly as the
+// survivors' scores are (activate_rt), is at most B less eight units in the last place: the hardware's exp and reciprocal are
+// good to about one such unit each, so no rounding wobble of theirs can lift a lower z to B.  Where the activation is flat at
+// B (a ReLU's zero, a saturated sigmoid) the result falls to the start of the flat part or to -inf: everything that ties is
+// admitted.  Supported: sigmoid, tanh, ReLU, leaky ReLU with a positive slope, linear.
+__device__ __forceinline__ float preactivation_bound(uint32_t key, uint32_t act, float slope, float alpha, float lambda)
+{
+    if (key == 0) return -__builtin_inff();   // no bound yet: fewer than k scores seen
+    const float B = key_score(key);
+    if (act == DSX_ACT_LINEAR) return B;
+    const float target = B - fabsf(B) * 1e-6f - 1e-37f;
+    float z;
+    switch (act) {
+    case DSX_ACT_SIGMOID:
+        if (target <= 0.0f) return -__builtin_inff();
+        z = (target < 1.0f) ? logf(target / (1.0f - target)) : 20.0f;
+        break;
+    case DSX_ACT_TANH:
+        if (target <= -1.0f) return -__builtin_inff();
+        z = (target < 1.0f) ? 0.5f * logf((1.0f + target) / (1.0f - target)) : 10.0f;
+        break;
+    case DSX_ACT_RELU:
+        if (target < 0.0f) return -__builtin_inff();
+        z = target;
+        break;
+    case DSX_ACT_LRELU:
+        z = (target > 0.0f) ? target : target / slope;
+        break;
+    default: return -__builtin_inff();
+    }
+    float delta = fmaxf(fabsf(z), 1.0f) * 9.5367431640625e-7f;   // 2^-20
+    for (int it = 0; it < 64; it++) {
+        if (activate_rt(z, act, slope, alpha, lambda) <= target) return z;
+        z -= delta;
+        delta *= 2.0f;
+    }
+    return -__builtin_inff();
+}
 
 // The epilogue below needs the admission bounds of the tile's rows.  Lane t < 32*MI*WM asks for row t's bound here, at the start
 // of the kernel: asked for in the epilogue, the load's latency would sit at the end of every tile.
@@ -94,7 +140,7 @@ __device__ __forceinline__ uint32_t candidate_bound_prefetch(const CandArgs& c, 
 constexpr int kCandWaveList = 256;   // survivors a wavefront gathers before it appends them
 template <int MI, int WM = 2, int WN = 2> constexpr int kCandLdsBytes = 32 * MI * WM * 4 + WM * WN * kCandWaveList * 12;
 
-template <int MI, int NI, int WM = 2, int WN = 2>
+template <int MI, int NI, int WM = 2, int WN = 2, bool PRE = false>
 __device__ __forceinline__ void candidate_epilogue(const floatx16 (&acc)[MI][NI], float* lds, const CandArgs& c, uint32_t bound_key,
                                                    uint32_t row0, uint32_t col0, uint32_t batch, uint32_t n, int tid, int wm, int wn, int l32,
                                                    int lhi)
@@ -102,7 +148,14 @@ __device__ __forceinline__ void candidate_epilogue(const floatx16 (&acc)[MI][NI]
     constexpr int BM = 32 * MI * WM;   // at most as many rows as the workgroup has lanes
     float* sBound = lds;
     // key 0: no bound yet (fewer than k items seen), every score that is a number is admitted
-    if (tid < BM) sBound[tid] = (row0 + tid < batch) ? (bound_key ? key_score(bound_key) : -__builtin_inff()) : __builtin_inff();
+    if (tid < BM) {
+        float bound = __builtin_inff();   // rows beyond the batch admit nothing
+        if (row0 + tid < batch) {
+            if constexpr (PRE) bound = preactivation_bound(bound_key, c.act, c.slope, c.alpha, c.lambda);
+            else bound = bound_key ? key_score(bound_key) : -__builtin_inff();
+        }
+        sBound[tid] = bound;
+    }
     __syncthreads();
     float bf[MI][4][4];
 #pragma unroll
@@ -169,7 +222,9 @@ __device__ __forceinline__ void candidate_epilogue(const floatx16 (&acc)[MI][NI]
                 if (listed + count > (uint32_t)kCandWaveList) append_all();
                 if (cand) {
                     const uint32_t slot = listed + __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
-                    sWord[slot] = ((uint64_t)score_key(x) << 32) | (uint32_t)~(c.col_offset + col);
+                    float score = x;
+                    if constexpr (PRE) score = activate_rt(x, c.act, c.slope, c.alpha, c.lambda);
+                    sWord[slot] = ((uint64_t)score_key(score) << 32) | (uint32_t)~(c.col_offset + col);
                     sRow[slot] = (r < batch) ? r : 0xffffffffu;   // (rows beyond the batch have an infinite bound: never taken)
                 }
                 listed += count;

@@ -147,7 +147,10 @@ __device__ __forceinline__ void fc_epilogue(floatx16 (&acc)[MI][NI], const FcArg
 
 // MI, NI: 32x32 MFMA blocks per wavefront in M and N.  XV / WV: vector width (floats) of the global loads of X / W.
 // TRANS: W is stored [n][k].
-template <int MI, int NI, int BK, int XV, int WV, bool TRANS, int ACT, bool CAND = false>
+// CAND: 0 = the result is stored (epilogue above); 1 = candidate mode, scores compared with score bounds (exact KNN);
+// 2 = candidate mode of a layer: the accumulators start from the bias, pre-activation sums are compared with bounds derived
+// from activated scores, and the survivors are activated (candidate_epilogue, PRE).
+template <int MI, int NI, int BK, int XV, int WV, bool TRANS, int ACT, int CAND = 0>
 __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_kernel(FcArgs a)
 {
     constexpr int BM = 64 * MI, BN = 64 * NI;
@@ -180,11 +183,17 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
 
     floatx16 acc[MI][NI];
 #pragma unroll
-    for (int i = 0; i < MI; i++)
+    for (int j = 0; j < NI; j++) {
+        float start = 0.0f;
+        if constexpr (CAND == 2) {   // every register of a lane belongs to column l32 of its block: the sums start from the bias
+            const uint32_t c = col0 + wn * 32 * NI + j * 32 + l32;
+            if (a.bias && c < a.n) start = a.bias[c];
+        }
 #pragma unroll
-        for (int j = 0; j < NI; j++)
+        for (int i = 0; i < MI; i++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+            for (int v = 0; v < 16; v++) acc[i][j][v] = start;
+    }
 
     float ra[A_ELEMS], rb[B_ELEMS];
     uint32_t bound_key = 0;
@@ -424,7 +433,7 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
     if constexpr (CAND) {
         static_assert(sizeof(sA) >= kCandLdsBytes<MI>, "the epilogue reuses the X tile's LDS");
         // (the k-loop ended with a barrier: every wavefront is done with sA)
-        candidate_epilogue<MI, NI>(acc, &sA[0][0][0], a.cand, bound_key, row0, col0, a.batch, a.n, tid, wm, wn, l32, lhi);
+        candidate_epilogue<MI, NI, 2, 2, CAND == 2>(acc, &sA[0][0][0], a.cand, bound_key, row0, col0, a.batch, a.n, tid, wm, wn, l32, lhi);
         return;
     }
 
@@ -598,8 +607,36 @@ int fc_candidates_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw
     a.tiles_n = (n + 127) / 128;
     const uint32_t total = a.tiles_m * a.tiles_n;
     const uint32_t grid = ((total + kXcds - 1) / kXcds) * kXcds;
-    hipLaunchKernelGGL((fc_gemm_kernel<2, 2, 16, 4, 4, false, DSX_ACT_LINEAR, true>), dim3(grid), dim3(kFcThreads), 0, ctx().stream, a);
+    hipLaunchKernelGGL((fc_gemm_kernel<2, 2, 16, 4, 4, false, DSX_ACT_LINEAR, 1>), dim3(grid), dim3(kFcThreads), 0, ctx().stream, a);
     DSX_LAUNCH_CHECK("fc_gemm_kernel (candidates)");
+    return DSX_OK;
+}
+
+// The same for a layer: Z = act(bias + X.W) is not stored; cand.act / slope / alpha / lambda describe the activation and
+// cand.row_bound holds keys of activated scores.  X must be 16-byte aligned with a pitch that is a multiple of four floats; W may
+// be aligned to 16, 8 or 4 bytes (a 27,278-wide row-major matrix is 8-byte aligned).
+int fc_layer_candidates_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, const float* bias, uint32_t batch, uint32_t k,
+                            uint32_t n, const CandArgs& cand)
+{
+    FcArgs a{};
+    a.X = X; a.W = W; a.bias = bias;
+    a.ldx = ldx; a.ldw = ldw;
+    a.batch = batch; a.k = k; a.n = n;
+    a.act = DSX_ACT_LINEAR;
+    a.fast32 = ((uint64_t)(batch + 128) * ldx * 4 < (1ull << 32)) && ((32ull * ldw + n + 128) * 4 < (1ull << 32));
+    a.cand = cand;
+    a.tiles_m = (batch + 127) / 128;
+    a.tiles_n = (n + 127) / 128;
+    const uint32_t total = a.tiles_m * a.tiles_n;
+    const dim3 grid(((total + kXcds - 1) / kXcds) * kXcds);
+    hipStream_t s = ctx().stream;
+    if (((uintptr_t)W % 16) == 0 && (ldw % 4) == 0)
+        hipLaunchKernelGGL((fc_gemm_kernel<2, 2, 16, 4, 4, false, DSX_ACT_LINEAR, 2>), grid, dim3(kFcThreads), 0, s, a);
+    else if (((uintptr_t)W % 8) == 0 && (ldw % 2) == 0)
+        hipLaunchKernelGGL((fc_gemm_kernel<2, 2, 16, 4, 2, false, DSX_ACT_LINEAR, 2>), grid, dim3(kFcThreads), 0, s, a);
+    else
+        hipLaunchKernelGGL((fc_gemm_kernel<2, 2, 16, 4, 1, false, DSX_ACT_LINEAR, 2>), grid, dim3(kFcThreads), 0, s, a);
+    DSX_LAUNCH_CHECK("fc_gemm_kernel (layer candidates)");
     return DSX_OK;
 }
 

@@ -87,6 +87,35 @@ int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int trans
 struct CandArgs;
 int fc_candidates_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, uint32_t batch, uint32_t k, uint32_t n,
                       const CandArgs& cand);
+// The same for a layer (pre-activation sums compared with bounds derived from activated scores, bias folded in).
+int fc_layer_candidates_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, const float* bias, uint32_t batch, uint32_t k,
+                            uint32_t n, const CandArgs& cand);
+// Output layer fused with its top-K (dsx_topk.hip): folds every row's candidates, minus the columns its filter lists, into its
+// best list and raises its bound; with keys != NULL (last column range) writes the result instead.  A row whose candidate list
+// overflowed is flagged, and recomputed from X, W and bias in the last range's call.
+struct LayerRefresh {
+    uint64_t* best;
+    const uint64_t* cand;
+    uint32_t* cand_count;
+    uint32_t cap, k;
+    uint32_t* row_bound;
+    uint32_t* row_flag;
+    uint32_t* flagged_total;
+    uint32_t position;
+    const uint32_t* index;
+    const uint64_t* fstart;
+    const uint64_t* fend;
+    const uint32_t* fidx;
+    float* keys;
+    uint32_t* values;
+    const float* X;
+    const float* W;
+    const float* bias;
+    uint32_t ldx, ldw, kdim, n;
+    uint32_t act;
+    float slope, alpha, lambda;
+};
+int layer_refresh_run(const LayerRefresh& r, uint32_t batch);
 // fp16 storage of the KNN operands (dsx_knn_f16.hip): padded row-major layout, conversion, and the score kernel in store mode
 // (cand == NULL: Z[batch][ldz]) or candidate mode.
 uint32_t knn_f16_ld(uint32_t dim);

@@ -1059,6 +1059,214 @@ int knn_refresh(uint64_t* best, const uint64_t* cand, uint32_t* cand_count, uint
     return DSX_OK;
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// Output layer fused with its top-K (dsx_fc_topk): the row's best list so far (k packed words) is merged with the candidates
+// the layer's last column range appended, minus the columns the row's filter lists (multiplier 0: the sample's own items).
+// One wavefront per row.  The filter is applied by hashing the candidates' columns into an LDS table (at most half full,
+// linear probing), striking out every listed column found there, and then offering only the candidates still present.
+// A row whose candidate list filled up is flagged; the refresh after the last range recomputes flagged rows from scratch,
+// without any list that could fill up: act(bias + x . W) 256 columns at a time (lane = column, k in order), the listed columns
+// marked in a bitmap that covers 262,144 columns at a time.  Slow (the whole matrix is read for one row) and exact.
+constexpr uint32_t kLayerTableSlots = 8192;   // twice the candidate capacity the layer search uses; as a bitmap: 262,144 columns
+constexpr uint32_t kLayerEmpty = 0xffffffffu, kLayerStruck = 0xfffffffeu;   // (no column has these numbers: widths stay below 2^32 - 2)
+
+struct LayerRefreshArgs {
+    uint64_t* best;            // [batch][k] packed words, best first, 0 = empty
+    const uint64_t* cand;      // [batch][cap]
+    uint32_t* cand_count;      // [batch], reset to 0 here
+    uint32_t cap;
+    uint32_t k;
+    uint32_t* row_bound;       // [batch] key of the row's k-th best score, raised here
+    uint32_t* row_flag;        // [batch] != 0: the row's list overflowed in this or an earlier range
+    uint32_t* flagged_total;   // host-visible word that is set to 1 when a row is flagged (may be NULL)
+    uint32_t position;
+    const uint32_t* index;
+    const uint64_t* fstart;
+    const uint64_t* fend;
+    const uint32_t* fidx;      // NULL: no filter
+    float* keys;               // final range only (else NULL): [batch][k] results
+    uint32_t* values;
+    // the layer itself, for flagged rows (final range only)
+    const float* X;
+    const float* W;
+    const float* bias;
+    uint32_t ldx, ldw, kdim, n;
+    uint32_t act;
+    float slope, alpha, lambda;
+};
+
+__device__ __forceinline__ uint32_t layer_hash(uint32_t col, uint32_t shift) { return (col * 2654435761u) >> shift; }
+
+template <int R>
+__device__ __forceinline__ void layer_recompute_row(WaveTopK<R>& list, const LayerRefreshArgs& a, uint32_t b, uint32_t lane, uint64_t fs,
+                                                    uint64_t fe, uint32_t* sBits)
+{
+    constexpr uint32_t kSpan = kLayerTableSlots * 32;
+    const float* x = a.X + (uint64_t)b * a.ldx;
+    for (uint32_t C0 = 0; C0 < a.n; C0 += kSpan) {
+        for (uint32_t i = lane; i < kLayerTableSlots; i += kWave) sBits[i] = 0;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        for (uint64_t t = fs + lane; t < fe; t += kWave) {
+            const uint32_t c = a.fidx[t];
+            if (c >= C0 && c - C0 < kSpan) atomicOr(&sBits[(c - C0) >> 5], 1u << ((c - C0) & 31));
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const uint32_t C1 = (a.n - C0 < kSpan) ? a.n : C0 + kSpan;
+        for (uint32_t c0 = C0; c0 < C1; c0 += 4 * kWave) {
+            float sum[4];
+            uint32_t col[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                col[j] = c0 + j * kWave + lane;
+                sum[j] = (a.bias && col[j] < C1) ? a.bias[col[j]] : 0.0f;
+            }
+            for (uint32_t kk = 0; kk < a.kdim; kk++) {
+                const float xk = x[kk];
+                const float* w = a.W + (uint64_t)kk * a.ldw;
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (col[j] < C1) sum[j] = fmaf(xk, w[col[j]], sum[j]);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float y = activate_rt(sum[j], a.act, a.slope, a.alpha, a.lambda);
+                const uint32_t off = col[j] - C0;
+                const bool ok = col[j] < C1 && y == y && !((sBits[off >> 5] >> (off & 31)) & 1u);
+                list.offer(ok, pack_score(y, col[j]));
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+template <int R>
+__global__ __launch_bounds__(kWave) void layer_refresh_kernel(LayerRefreshArgs a)
+{
+    __builtin_amdgcn_s_setprio(3);   // short kernels issue ahead of a GEMM's wavefronts that share their SIMD
+    using List = WaveTopK<R>;
+    __shared__ uint64_t sStage[List::kStageWords];
+    __shared__ uint32_t sTable[kLayerTableSlots];
+    const uint32_t b = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    const uint32_t count = a.cand_count[b];
+    bool flagged = a.row_flag[b] != 0;
+    __builtin_amdgcn_wave_barrier();
+    if (lane == 0) a.cand_count[b] = 0;
+    if (!flagged && count > a.cap) {
+        flagged = true;
+        if (lane == 0) {
+            a.row_flag[b] = 1;
+            if (a.flagged_total) *(volatile uint32_t*)a.flagged_total = 1u;
+        }
+    }
+    const bool final_range = a.keys != nullptr;
+    if (flagged && !final_range) return;
+    uint64_t fs = 0, fe = 0;
+    if (a.fidx && (count > 0 || flagged)) {
+        uint32_t r = a.position + b;
+        if (a.index) r = a.index[r];
+        fs = a.fstart[r];
+        fe = a.fend[r];
+    }
+    List list;
+    list.init(sStage, lane, a.k);
+    if (flagged) {
+        layer_recompute_row<R>(list, a, b, lane, fs, fe, sTable);
+        list.finish();
+        write_final<R>(list.q, lane, a.k, 0, a.keys + (uint64_t)b * a.k, a.values + (uint64_t)b * a.k);
+        return;
+    }
+    const uint64_t* src = a.cand + (uint64_t)b * a.cap;
+    const bool filtering = fe > fs && count > 0;   // wave-uniform
+    // table size: a power of two, at least twice the candidates
+    uint32_t bits = 7;
+    while ((1u << bits) < 2 * count) bits++;
+    const uint32_t mask = (1u << bits) - 1, shift = 32 - bits;
+    if (filtering) {
+        for (uint32_t i = lane; i <= mask; i += kWave) sTable[i] = kLayerEmpty;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        for (uint32_t p = lane; p < count; p += kWave) {
+            const uint32_t col = ~(uint32_t)src[p];
+            uint32_t h = layer_hash(col, shift);
+            while (atomicCAS(&sTable[h], kLayerEmpty, col) != kLayerEmpty) h = (h + 1) & mask;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        for (uint64_t t = fs + lane; t < fe; t += kWave) {
+            const uint32_t col = a.fidx[t];
+            uint32_t h = layer_hash(col, shift);
+            for (;;) {
+                const uint32_t v = sTable[h];
+                if (v == kLayerEmpty) break;
+                if (v == col) {
+                    sTable[h] = kLayerStruck;
+                    break;
+                }
+                h = (h + 1) & mask;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+    uint64_t* mine = a.best + (uint64_t)b * a.k;
+    for (uint32_t p0 = 0; p0 < a.k; p0 += kWave) {
+        const uint32_t p = p0 + lane;
+        const uint64_t word = (p < a.k) ? mine[p] : 0ull;
+        list.offer(word != 0, word);
+    }
+    for (uint32_t p0 = 0; p0 < count; p0 += kWave) {
+        const uint32_t p = p0 + lane;
+        const uint64_t word = (p < count) ? src[p] : 0ull;
+        bool live = word != 0;
+        if (filtering && live) {
+            const uint32_t col = ~(uint32_t)word;
+            uint32_t h = layer_hash(col, shift);
+            for (;;) {
+                const uint32_t v = sTable[h];
+                if (v == col) break;
+                if (v == kLayerEmpty) {   // struck out: the chain ends without the column
+                    live = false;
+                    break;
+                }
+                h = (h + 1) & mask;
+            }
+        }
+        list.offer(live, word);
+    }
+    list.finish();
+    if (final_range) {
+        write_final<R>(list.q, lane, a.k, 0, a.keys + (uint64_t)b * a.k, a.values + (uint64_t)b * a.k);
+        return;
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const uint32_t p = r * kWave + lane;
+        if (p < a.k) mine[p] = list.q[r];
+        if (p == a.k - 1 && list.q[r] != 0) a.row_bound[b] = max(a.row_bound[b], (uint32_t)(list.q[r] >> 32));
+    }
+}
+
+int layer_refresh_run(const LayerRefresh& r, uint32_t batch)
+{
+    if (2 * r.cap > kLayerTableSlots) return set_error(DSX_EINVAL, "layer_refresh: candidate capacity %u exceeds %u", r.cap, kLayerTableSlots / 2);
+    LayerRefreshArgs a{};
+    a.best = r.best; a.cand = r.cand; a.cand_count = r.cand_count; a.cap = r.cap; a.k = r.k;
+    a.row_bound = r.row_bound; a.row_flag = r.row_flag; a.flagged_total = r.flagged_total;
+    a.position = r.position; a.index = r.index; a.fstart = r.fstart; a.fend = r.fend; a.fidx = r.fidx;
+    a.keys = r.keys; a.values = r.values;
+    a.X = r.X; a.W = r.W; a.bias = r.bias; a.ldx = r.ldx; a.ldw = r.ldw; a.kdim = r.kdim; a.n = r.n;
+    a.act = r.act; a.slope = r.slope; a.alpha = r.alpha; a.lambda = r.lambda;
+    hipStream_t s = ctx().stream;
+    if (a.k <= 64) hipLaunchKernelGGL((layer_refresh_kernel<1>), dim3(batch), dim3(kWave), 0, s, a);
+    else if (a.k <= 128) hipLaunchKernelGGL((layer_refresh_kernel<2>), dim3(batch), dim3(kWave), 0, s, a);
+    else hipLaunchKernelGGL((layer_refresh_kernel<4>), dim3(batch), dim3(kWave), 0, s, a);
+    DSX_LAUNCH_CHECK("layer_refresh_kernel");
+    return DSX_OK;
+}
+
 // Guided top-K when it applies (k <= 64, 64-column segments, at most kGuidedMaxSegs of them), the scan otherwise.
 int topk_guided_run(const float* in, uint32_t width, uint32_t batch, uint32_t k, float* keys, uint32_t* values, const float* seg_max,
                     uint32_t seg_width, uint32_t position, const uint32_t* index, const uint64_t* fstart, const uint64_t* fend,

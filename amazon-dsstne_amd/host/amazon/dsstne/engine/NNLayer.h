@@ -71,11 +71,21 @@ private:
     unique_ptr<GpuBuffer<NNFloat>> _pbSegMaxOther;
     uint32_t _segWidthOther = 0;
     uint32_t _lanes = 1;
+    // A wide output layer that feeds nothing but a top-K is not computed by the forward pass: NNNetwork::CalculateTopK /
+    // CalculateFilteredTopK then run the layer and the top-K in one call that never stores the layer's result (dsx_fc_topk), and
+    // whoever asks for the units themselves (NNNetwork::GetUnitBuffer, GetUnits) has them computed at that moment (Materialise).
+    // _deferred: the units of the current batch have not been computed yet; _deferredBatch: its rows.
+    bool _bDeferOutput = true;   // NNNetwork::SetDeferredOutput
+    bool _deferred = false, _deferredOther = false;
+    uint32_t _deferredBatch = 0, _deferredBatchOther = 0;
+    void Materialise();
     void SwapLane()
     {
         _pbUnit.swap(_pbUnitOther);
         _pbSegMax.swap(_pbSegMaxOther);
         std::swap(_segWidth, _segWidthOther);
+        std::swap(_deferred, _deferredOther);
+        std::swap(_deferredBatch, _deferredBatchOther);
     }
     int32_t _priority;
 

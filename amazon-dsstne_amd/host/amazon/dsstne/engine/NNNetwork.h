@@ -53,6 +53,8 @@ private:
     void LoadBatch();
     void RefreshState();
     void ClearUpdates() {}
+    void LayerWithTopK(NNLayer* pLayer, uint32_t k, uint32_t batch, const uint32_t* pIndex, const uint64_t* pFilterStart,
+                       const uint64_t* pFilterEnd, const uint32_t* pFilterIndex, NNFloat* pKey, uint32_t* pValue);
 
 public:
     ~NNNetwork();
@@ -76,6 +78,10 @@ public:
     // with those of the batch before it.  Everything read back through this API waits as needed; a device pointer obtained
     // from GetUnitBuffer belongs to the batch predicted last.  One lane restores single buffers.
     bool SetLanes(uint32_t lanes);
+    // No counterpart in the reference.  By default a wide output layer that feeds nothing else is not computed by PredictBatch
+    // but together with the CalculateTopK / CalculateFilteredTopK that follows, without storing its result; GetUnitBuffer and
+    // GetUnits compute it on demand.  SetDeferredOutput(false) makes PredictBatch store every layer, as the reference does.
+    bool SetDeferredOutput(bool bDefer);
     uint32_t GetLanes() const { return _lanes; }
     uint32_t GetLane() const { return _lane; }
     void Randomize();                           // every connection back to its starting values (engine/NNNetwork.cpp:675-679)

@@ -131,6 +131,12 @@ void NNLayer::ForwardPropagate(uint32_t position, uint32_t batch, bool bTraining
 
 // Narrower layers are cheap to scan in full.
 static const uint32_t kSegMaxMinWidth = 8192;
+// From this width on the output layer is not stored but computed together with its top-K.  What the GEMM kernel's epilogue
+// then does per 32 x 32 block depends on how many scores of the block reach the row's running k-th score: about
+// 1024 * (k / columns seen so far + the filter's density).  In a 27,278-wide catalogue with top-10 and 144 own items per sample
+// that is ten per block, every block takes the slow path and the fused call is no faster than storing the layer (measured:
+// 95 us against 76 us for the GEMM alone); in a 1,000,000-wide one it is one block in three, and 16 GB of stores and loads go away.
+static const uint32_t kDeferMinWidth = 131072;
 
 void NNLayer::ForwardPropagateFullyConnected(uint32_t position, uint32_t batch, bool bTraining)
 {
@@ -145,6 +151,7 @@ void NNLayer::ForwardPropagateFullyConnected(uint32_t position, uint32_t batch, 
     dsx_act_params params = {_RELUSlope, _ELUAlpha, _SELULambda};
     NNFloat* pUnit = GetIncomingUnitBuffer();
     _segWidth = 0;   // whatever described the previous batch no longer holds
+    _deferred = false;
 
     // One source, no skips, elementwise activation: a single fused kernel.
     if (nIn == 1 && _vIncomingSkip.empty() && _activation != SoftMax) {
@@ -155,13 +162,23 @@ void NNLayer::ForwardPropagateFullyConnected(uint32_t position, uint32_t batch, 
             src->_pDataSet->CalculateSparseLayer(position, batch, _stride, wsrc->_pbWeight->_pDevData, w->_pbBias->_pDevData, _activation,
                                                  _RELUSlope, _ELUAlpha, _SELULambda, pUnit);
         } else if (_kind == Output && _localStride >= kSegMaxMinWidth) {
-            // wide output layer: the kernel also leaves segment maxima for the top-K that usually follows
-            const size_t need = (size_t)_batch * ((_localStride + 63) / 64);
-            if (!_pbSegMax || _pbSegMax->_length < need) _pbSegMax.reset(new GpuBuffer<NNFloat>(need));
-            dsxFatal(dsx_fc_forward_segmax(src->GetUnitBuffer(), src->_stride, wsrc->_pbWeight->_pDevData, w->_bTransposed ? 1 : 0,
-                                           w->_pbBias->_pDevData, pUnit, _stride, batch, src->_stride, _localStride, (uint32_t)_activation,
-                                           &params, _pbSegMax->_pDevData, &_segWidth),
-                     "NNLayer::ForwardPropagate: GEMM failure");
+            // Wide output layer that feeds no other layer: what usually follows is a top-K, which can run together with the layer
+            // without the layer's result ever being stored.  The layer is computed when somebody asks for it.
+            if (_bDeferOutput && _localStride >= kDeferMinWidth && !w->_bTransposed && _vOutgoingLayer.empty() && _vOutgoingSkip.empty() &&
+                dsx_fc_topk_supported(src->_stride, src->GetUnitBuffer(), (uint32_t)_activation, &params, NULL)) {
+                if (dsx_fc_topk_flagged(0)) {
+                    // rows whose survivor lists filled up had to be recomputed one by one: this data (thousands of scores tied at the
+                    // top of a row) is served better by the stored layer and the scanning top-K
+                    printf("NNLayer::ForwardPropagate: scores of layer %s tie in their thousands; its result is stored from now on.\n", _name.c_str());
+                    _bDeferOutput = false;
+                } else {
+                    _deferred = true;
+                    _deferredBatch = batch;
+                    return;
+                }
+            }
+            _deferredBatch = batch;
+            Materialise();
         } else {
             dsxFatal(dsx_fc_forward(src->GetUnitBuffer(), src->_stride, wsrc->_pbWeight->_pDevData, w->_bTransposed ? 1 : 0,
                                     w->_pbBias->_pDevData, pUnit, _stride, batch, src->_stride, _localStride, 0, (uint32_t)_activation, &params),
@@ -189,6 +206,22 @@ void NNLayer::ForwardPropagateFullyConnected(uint32_t position, uint32_t batch, 
     CalculateActivation(batch);
 }
 
+// The wide output layer's own kernel: stores the layer's result and leaves segment maxima for the top-K that usually follows.
+void NNLayer::Materialise()
+{
+    _deferred = false;
+    NNLayer* src = _vIncomingLayer[0];
+    NNWeight* w = _vIncomingWeight[0];
+    NNWeight* wsrc = w->_bShared ? w->_pSharedWeight : w;
+    dsx_act_params params = {_RELUSlope, _ELUAlpha, _SELULambda};
+    const size_t need = (size_t)_batch * ((_localStride + 63) / 64);
+    if (!_pbSegMax || _pbSegMax->_length < need) _pbSegMax.reset(new GpuBuffer<NNFloat>(need));
+    dsxFatal(dsx_fc_forward_segmax(src->GetUnitBuffer(), src->_stride, wsrc->_pbWeight->_pDevData, w->_bTransposed ? 1 : 0,
+                                   w->_pbBias->_pDevData, GetIncomingUnitBuffer(), _stride, _deferredBatch, src->_stride, _localStride,
+                                   (uint32_t)_activation, &params, _pbSegMax->_pDevData, &_segWidth),
+             "NNLayer::ForwardPropagate: GEMM failure");
+}
+
 void NNLayer::CalculateActivation(uint32_t batch)
 {
     dsx_act_params params = {_RELUSlope, _ELUAlpha, _SELULambda};
@@ -211,6 +244,7 @@ bool NNLayer::GetUnits(vector<NNFloat>& vUnit)
         printf("NNLayer::GetUnits: Unit data not yet allocated.\n");
         return false;
     }
+    if (_deferred) Materialise();
     // the whole [batch][stride] buffer comes back (the reference sizes the vector to one row only and then overruns it)
     if (vUnit.size() < _pbUnit->_length) vUnit.resize(_pbUnit->_length);
     _pbUnit->Download(vUnit.data());
@@ -227,6 +261,7 @@ bool NNLayer::GetUnits(NNFloat* pUnit)
         printf("NNLayer::GetUnits: Download pointer invalid.\n");
         return false;
     }
+    if (_deferred) Materialise();
     _pbUnit->Download(pUnit);
     return true;
 }
@@ -243,5 +278,6 @@ bool NNLayer::SetUnits(const vector<NNFloat>& vUnit)
     }
     _pbUnit->Upload(vUnit.data());
     _segWidth = 0;
+    _deferred = false;
     return true;
 }

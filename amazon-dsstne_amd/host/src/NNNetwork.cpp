@@ -307,6 +307,29 @@ bool NNNetwork::SetLanes(uint32_t lanes)
     return true;
 }
 
+// The deferred output layer and its top-K in one call; the layer's result is not stored.
+void NNNetwork::LayerWithTopK(NNLayer* pLayer, uint32_t k, uint32_t batch, const uint32_t* pIndex, const uint64_t* pFilterStart,
+                              const uint64_t* pFilterEnd, const uint32_t* pFilterIndex, NNFloat* pKey, uint32_t* pValue)
+{
+    NNLayer* src = pLayer->_vIncomingLayer[0];
+    NNWeight* w = pLayer->_vIncomingWeight[0];
+    NNWeight* wsrc = w->_bShared ? w->_pSharedWeight : w;
+    dsx_act_params params = {pLayer->_RELUSlope, pLayer->_ELUAlpha, pLayer->_SELULambda};
+    dsxFatal(dsx_fc_topk(src->GetUnitBuffer(), src->_stride, wsrc->_pbWeight->_pDevData, w->_pbBias->_pDevData, batch, src->_stride,
+                         pLayer->_localStride, (uint32_t)pLayer->_activation, &params, k, pKey, pValue, _position, pIndex, pFilterStart,
+                         pFilterEnd, pFilterIndex),
+             "NNNetwork::CalculateTopK: output layer with top-K");
+}
+
+bool NNNetwork::SetDeferredOutput(bool bDefer)
+{
+    for (auto l : _vLayer) {
+        if (!bDefer && l->_deferred) l->Materialise();
+        l->_bDeferOutput = bDefer;
+    }
+    return true;
+}
+
 void NNNetwork::CalculateTopK(const string& layer, uint32_t k, GpuBuffer<NNFloat>* pbKey, GpuBuffer<uint32_t>* pbValue)
 {
     auto it = _mLayer.find(layer);
@@ -329,7 +352,9 @@ void NNNetwork::CalculateTopK(const string& layer, uint32_t k, GpuBuffer<NNFloat
     }
     uint32_t batch = _batch;
     if (_position + batch > _examples) batch = _examples - _position;
-    if (pLayer->_segWidth != 0 && pLayer->_pbSegMax)
+    if (pLayer->_deferred)
+        LayerWithTopK(pLayer, k, batch, NULL, NULL, NULL, NULL, pbKey->_pDevData, pbValue->_pDevData);
+    else if (pLayer->_segWidth != 0 && pLayer->_pbSegMax)
         dsxFatal(dsx_topk_guided(pLayer->_pbUnit->_pDevData, pbKey->_pDevData, pbValue->_pDevData, batch, pLayer->_localStride, k,
                                  pLayer->_pbSegMax->_pDevData, pLayer->_segWidth, 0, NULL, NULL, NULL, NULL, NULL),
                  "NNNetwork::CalculateTopK");
@@ -368,6 +393,14 @@ void NNNetwork::CalculateFilteredTopK(const string& layer, uint32_t k, NNDataSet
     }
     pFilter->NoteSparseRead();
     const uint32_t* pIndex = (pFilter->_attributes & NNDataSetEnums::Indexed) ? pFilter->_pbIndex->_pDevData : NULL;
+    if (pLayer->_deferred) {
+        if (pMul == NULL) {
+            LayerWithTopK(pLayer, k, batch, pIndex, pFilter->_pbSparseStart->_pDevData, pFilter->_pbSparseEnd->_pDevData,
+                          pFilter->_pbSparseIndex->_pDevData, pbKey->_pDevData, pbValue->_pDevData);
+            return;
+        }
+        pLayer->Materialise();   // multipliers other than 0 need the listed items' scores
+    }
     // with segment maxima of the current batch (left by the layer's dense kernel) only the segments that can hold a result are read
     const NNFloat* pSegMax = (pLayer->_segWidth != 0 && pLayer->_pbSegMax) ? pLayer->_pbSegMax->_pDevData : NULL;
     dsxFatal(dsx_topk_guided(pLayer->_pbUnit->_pDevData, pbKey->_pDevData, pbValue->_pDevData, batch, pLayer->_localStride, k, pSegMax,
@@ -391,6 +424,13 @@ void NNNetwork::CalculateFilteredTopK(const string& layer, uint32_t k, const uin
     }
     uint32_t batch = _batch;
     if (_position + batch > _examples) batch = _examples - _position;
+    if (pLayer->_deferred) {
+        if (pFilterMul == NULL) {
+            LayerWithTopK(pLayer, k, batch, NULL, pFilterStart, pFilterEnd, pFilterIndex, pKey, pValue);
+            return;
+        }
+        pLayer->Materialise();
+    }
     const NNFloat* pSegMax = (pLayer->_segWidth != 0 && pLayer->_pbSegMax) ? pLayer->_pbSegMax->_pDevData : NULL;
     dsxFatal(dsx_topk_guided(pLayer->_pbUnit->_pDevData, pKey, pValue, batch, pLayer->_localStride, k, pSegMax, pLayer->_segWidth, _position,
                              NULL, pFilterStart, pFilterEnd, pFilterIndex, pFilterMul),
@@ -468,6 +508,7 @@ NNFloat* NNNetwork::GetUnitBuffer(const string& layer)
         printf("NNNetwork::GetUnitBuffer: Unknown layer %s.\n", layer.c_str());
         return NULL;
     }
+    if (itr->second->_deferred) itr->second->Materialise();
     // the caller gets a writable device pointer: the segment maxima of the batch may not describe the units any longer
     itr->second->_segWidth = 0;
     // The reference's callers follow this call with a plain cudaMemcpy or a kernel of their own

@@ -381,6 +381,13 @@ int dsstne_set_lanes(dsstne_context* c, uint32_t lanes)
     CAPI_CATCH(-1)
 }
 
+int dsstne_set_deferred_output(dsstne_context* c, int defer)
+{
+    CAPI_TRY
+    return c->net()->SetDeferredOutput(defer != 0) ? 0 : fail("dsstne_set_deferred_output failed");
+    CAPI_CATCH(-1)
+}
+
 int dsstne_predict(dsstne_context* c, const char* layer, uint32_t k, const char* filter_dataset, float* scores, uint32_t* indexes)
 {
     int rc = dsstne_predict_batch(c, 0);

@@ -87,6 +87,11 @@ int dsstne_get_topk(dsstne_context* ctx, const char* layer, uint32_t rows, uint3
  * dsstne_set_lanes(ctx, 1) goes back to one set of buffers and one stream. */
 int dsstne_get_topk_previous(dsstne_context* ctx, const char* layer, uint32_t rows, uint32_t k, float* scores, uint32_t* indexes);
 int dsstne_set_lanes(dsstne_context* ctx, uint32_t lanes);
+/* No counterpart in the reference (NNNetwork::SetDeferredOutput).  By default a wide output layer that feeds nothing else is
+ * computed together with the dsstne_topk that follows dsstne_predict_batch, in one pass that never stores the layer's
+ * [batch x width] result; dsstne_get_units / dsstne_get_unit_buffer compute it when asked.  defer == 0: every layer is stored
+ * by dsstne_predict_batch, as in the reference. */
+int dsstne_set_deferred_output(dsstne_context* ctx, int defer);
 /* Dsstne.predict in one call: position 0, predict, unfiltered (filter_dataset NULL) or filtered top-k, copy back. */
 int dsstne_predict(dsstne_context* ctx, const char* layer, uint32_t k, const char* filter_dataset, float* scores, uint32_t* indexes);
 /* NNLayer::GetUnits: the layer's [batch][width] activations. */

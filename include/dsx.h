@@ -262,6 +262,30 @@ int dsx_topk_guided(const float* in, float* keys, uint32_t* values, uint32_t bat
                     uint32_t seg_width, uint32_t position, const uint32_t* index, const uint64_t* filter_start,
                     const uint64_t* filter_end, const uint32_t* filter_index, const float* filter_mul);
 
+/* Output layer and recommendations in one call: the forward GEMM of NNLayer::ForwardPropagateFullyConnected (bias, product,
+ * activation; engine/NNLayer.cpp:994-1167) on the output layer, followed by NNRecsGenerator::generateRecs' filtered
+ * kCalculateTopK (utils/NNRecsGenerator.cpp:83-150) over its result, without ever storing the [batch x n] result:
+ *   keys/values[b] = top-k over columns j of act(bias[j] + sum_i X[b][i] * W[i][j]), the columns listed in row b's filter dropped
+ * (filter arguments as dsx_topk_filtered with filter_mul == NULL; filter_index == NULL: no filter).  W is [k_dim x n]
+ * row-major.  Only the first few thousand columns are produced as a matrix (library scratch) and scanned; every later column
+ * range is compared with the rows' running k-th scores inside the GEMM kernel's registers and only the survivors are kept.
+ * Results are exact under the same total order as dsx_topk (score descending, column ascending); a score here and the same
+ * score from dsx_fc_forward may differ in the last place (the bias enters the sum first instead of last).  A row whose
+ * survivor list fills up (thousands of scores tied at the top) is recomputed on the device, slowly; dsx_fc_topk_flagged tells
+ * a caller that this has happened, so that it can go back to dsx_fc_forward + dsx_topk_filtered for such data.
+ * Returns DSX_EUNSUPPORTED (dsx_fc_topk_supported() == 0) unless the activation is non-decreasing (sigmoid, tanh, ReLU, leaky
+ * ReLU with a positive slope, linear) and X is 16-byte aligned with ldx a multiple of 4. */
+int dsx_fc_topk(const float* X, uint32_t ldx, const float* W, const float* bias, uint32_t batch, uint32_t k_dim, uint32_t n,
+                uint32_t activation, const dsx_act_params* params, uint32_t k, float* keys, uint32_t* values, uint32_t position,
+                const uint32_t* index, const uint64_t* filter_start, const uint64_t* filter_end, const uint32_t* filter_index);
+int dsx_fc_topk_supported(uint32_t ldx, const float* X, uint32_t activation, const dsx_act_params* params, const float* filter_mul);
+/* 1 if any row of any dsx_fc_topk call so far had to be recomputed (reset != 0 clears the mark). */
+int dsx_fc_topk_flagged(int reset);
+/* Tuning knobs, used by the tests to reach every path with small inputs: width of the first column block (0: default 2,048) and
+ * survivor words per row and column range (0: default 4,096, the maximum). */
+int dsx_fc_topk_set_first_columns(uint32_t columns);
+int dsx_fc_topk_set_candidate_capacity(uint32_t words);
+
 /* ---- KNN ------------------------------------------------------------------------------------------------------------- */
 /* Device part of KnnExactGpu::search (knn/KnnExactGpu.cu:99-148): scores = queries . items^T (cublasSgemmEx) followed by
  * the padded top-K.  items is column-major [rows_padded x dim] as KnnData::load builds it (knn/KnnData.cpp:197-207),

@@ -133,6 +133,23 @@ def test_cfg4_full_size(pkg, dsx, orc, synth):
     rk, ri = orc.topk(unit, p.k)
     assert np.array_equal(ui[picks], ri) and np.array_equal(uk[picks].view(np.uint32), rk.view(np.uint32)), "unfiltered top-100 differs"
     check_batch_properties(p, uk, ui, filtered_rows=False)
+    # the output layer and the filtered top-100 in one call that stores no scores: same recommendations
+    fk = pkg.DeviceArray((p.batch, p.k), np.float32)
+    fi = pkg.DeviceArray((p.batch, p.k), np.uint32)
+    dsx.dsx_fc_topk_flagged(1)
+    pkg.check(dsx.dsx_fc_topk(pipe.units[0].ptr, p.widths[1], pipe.W[1].ptr, pipe.b[1].ptr, p.batch, p.widths[1], p.widths[2], p.acts[1],
+                              C.byref(pipe.params), p.k, fk.ptr, fi.ptr, 0, None, pipe.start.ptr, pipe.end.ptr, pipe.sidx.ptr))
+    gk, gi = fk.numpy(), fi.numpy()
+    say("cfg4 fused: %d of %d indexes differ from the stored path, rows recomputed: %d" % (int((gi != idx).sum()), gi.size, dsx.dsx_fc_topk_flagged(0)))
+    check_batch_properties(p, gk, gi)
+    assert_close(gk, keys, "cfg4 fused scores vs stored path", rel=1e-5)
+    mism = gi != idx
+    assert mism.mean() < 1e-3          # last-place differences of the sums may swap neighbours in a near-tie, nothing else
+    if mism.any():
+        assert np.abs(gk[mism].astype(np.float64) - keys[mism].astype(np.float64)).max() < 1e-5
+    _, ref_scores, ref_keys, ref_idx = oracle_rows(orc, p, picks, p.k)
+    assert_topk_parity(gk[picks], gi[picks], ref_keys, ref_idx, ref_scores, "cfg4 fused vs oracle")
+    assert dsx.dsx_fc_topk_flagged(1) == 0
 
 
 def test_cfg5_knn_full_size(pkg, dsx, orc, synth):
