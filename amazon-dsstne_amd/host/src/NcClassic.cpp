@@ -70,6 +70,7 @@ struct Cursor {
     std::ifstream& in;
     int version;
     const std::string& fname;
+    uint64_t fileSize;   // no count in the header can exceed what the file holds
 
     void bytes(void* dst, size_t n)
     {
@@ -92,7 +93,7 @@ struct Cursor {
     std::string name()
     {
         uint64_t n = count();
-        if (n > (1u << 20)) throw Error(fname + ": implausible name length");
+        if (n > (1u << 20) || n > fileSize) throw Error(fname + ": implausible name length");
         std::string s((size_t)n, '\0');
         if (n) bytes(&s[0], (size_t)n);
         skipPad(n);
@@ -111,7 +112,7 @@ struct Cursor {
         a.type = (int)u32();
         a.count = count();
         size_t es = typeSize(a.type);
-        if (a.count > (1ull << 32)) throw Error(fname + ": implausible attribute length");
+        if (a.count > fileSize / es) throw Error(fname + ": an attribute claims more values than the file holds");
         a.raw.resize((size_t)(a.count * es));
         if (!a.raw.empty()) bytes(a.raw.data(), a.raw.size());
         skipPad(a.count * es);
@@ -147,14 +148,26 @@ Reader::Reader(const std::string& fname) : _fname(fname), _version(0)
     char magic[4] = {0};
     in.read(magic, 4);
     if (!in || magic[0] != 'C' || magic[1] != 'D' || magic[2] != 'F' || (magic[3] != 1 && magic[3] != 2 && magic[3] != 5)) {
-        if (isHdf5File(fname))
-            throw Error(fname + ": this is a NetCDF-4 (HDF5) file; convert it with `nccopy -k cdf5 " + fname + " out.nc` (this build reads the classic CDF-1/2/5 containers)");
-        throw Error(fname + ": not a classic NetCDF file");
+        if (isHdf5File(fname)) {
+            in.close();
+            _version = 4;
+            parseHdf5(fname, _dims, _dimByName, _atts, _attOrder, _vars, _varByName);
+            return;
+        }
+        throw Error(fname + ": neither a classic NetCDF file nor a NetCDF-4 (HDF5) one");
     }
     _version = magic[3];
-    Cursor c{in, _version, _fname};
+    in.seekg(0, std::ios::end);
+    const uint64_t fileSize = (uint64_t)in.tellg();
+    in.seekg(4);
+    Cursor c{in, _version, _fname, fileSize};
     c.count();   // numrecs: no record variables are used
-    uint64_t ndims = c.listHeader(0x0A);
+    // (a list of n entries takes at least 8 n bytes of header)
+    auto plausible = [&](uint64_t n, const char* what) {
+        if (n > fileSize / 8) throw Error(_fname + ": the header claims more " + what + " than the file could hold");
+        return n;
+    };
+    uint64_t ndims = plausible(c.listHeader(0x0A), "dimensions");
     for (uint64_t i = 0; i < ndims; i++) {
         Dimension d;
         d.name = c.name();
@@ -162,24 +175,27 @@ Reader::Reader(const std::string& fname) : _fname(fname), _version(0)
         _dimByName[d.name] = _dims.size();
         _dims.push_back(d);
     }
-    uint64_t natts = c.listHeader(0x0C);
+    uint64_t natts = plausible(c.listHeader(0x0C), "attributes");
     for (uint64_t i = 0; i < natts; i++) {
         Attribute a = c.attribute();
+        if (!_atts.count(a.name)) _attOrder.push_back(a.name);
         _atts[a.name] = a;
     }
-    uint64_t nvars = c.listHeader(0x0B);
+    uint64_t nvars = plausible(c.listHeader(0x0B), "variables");
     for (uint64_t i = 0; i < nvars; i++) {
         Variable v;
         v.name = c.name();
-        uint64_t nd = c.count();
+        uint64_t nd = plausible(c.count(), "dimensions of a variable");
         v.count = 1;
         for (uint64_t j = 0; j < nd; j++) {
             uint64_t id = _version == 5 ? c.u64() : c.u32();
             if (id >= _dims.size()) throw Error(_fname + ": variable " + v.name + " uses an unknown dimension");
             v.dimIds.push_back((uint32_t)id);
-            v.count *= _dims[(size_t)id].length;
+            const uint64_t len = _dims[(size_t)id].length;
+            if (len != 0 && v.count > (1ull << 62) / len) throw Error(_fname + ": variable " + v.name + " has an implausible size");
+            v.count *= len;
         }
-        uint64_t nva = c.listHeader(0x0C);
+        uint64_t nva = plausible(c.listHeader(0x0C), "attributes of a variable");
         for (uint64_t j = 0; j < nva; j++) c.attribute();
         v.type = (int)c.u32();
         c.count();   // vsize
@@ -212,14 +228,39 @@ const Variable& Reader::var(const std::string& name) const
 
 void Reader::readRaw(const Variable& v, std::vector<uint8_t>& raw) const
 {
+    if (!v.unsupported.empty()) throw Error(_fname + ": variable " + v.name + " cannot be read: " + v.unsupported);
     std::ifstream in(_fname, std::ios::binary);
     if (!in) throw Error(_fname + ": cannot open");
+    in.seekg(0, std::ios::end);
+    const uint64_t fileSize = (uint64_t)in.tellg();
     size_t es = typeSize(v.type);
-    raw.resize((size_t)(v.count * es));
-    in.seekg((std::streamoff)v.begin);
-    if (!raw.empty()) in.read((char*)raw.data(), (std::streamsize)raw.size());
-    if (!in) throw Error(_fname + ": variable " + v.name + " is truncated");
-    swapInPlace(raw.data(), es, v.count);
+    if (v.count > (fileSize + v.inlineData.size() + 8) / es && !(v.hdf5 && (v.chunked || v.begin == ~0ull)))
+        throw Error(_fname + ": variable " + v.name + " claims more data than the file holds");
+    raw.assign((size_t)(v.count * es), 0);
+    auto readAt = [&](uint64_t offset, uint8_t* dst, uint64_t bytes) {
+        if (offset > fileSize || bytes > fileSize - offset) throw Error(_fname + ": variable " + v.name + " is truncated");
+        in.seekg((std::streamoff)offset);
+        if (bytes) in.read((char*)dst, (std::streamsize)bytes);
+        if (!in) throw Error(_fname + ": variable " + v.name + " is truncated");
+    };
+    if (!v.hdf5) {
+        readAt(v.begin, raw.data(), raw.size());
+        swapInPlace(raw.data(), es, v.count);
+        return;
+    }
+    if (v.compact) {
+        if (v.inlineData.size() < raw.size()) throw Error(_fname + ": variable " + v.name + " is truncated");
+        memcpy(raw.data(), v.inlineData.data(), raw.size());
+    } else if (v.chunked) {
+        for (const Variable::Extent& e : v.extents) {
+            if (e.first >= v.count) continue;
+            const uint64_t n = std::min(e.count, v.count - e.first);   // the last chunk may reach beyond the variable
+            readAt(e.offset, raw.data() + e.first * es, n * es);
+        }
+    } else if (v.begin != ~0ull) {
+        readAt(v.begin, raw.data(), raw.size());
+    }
+    if (!v.littleEndian) swapInPlace(raw.data(), es, v.count);
 }
 
 template <typename T> void Reader::read(const std::string& name, std::vector<T>& out) const

@@ -1,0 +1,72 @@
+// nc_dump — prints everything ncc::Reader finds in a NetCDF file (classic or NetCDF-4) in a canonical text form: dimensions,
+// global attributes with their values, variables with type, element count and every value.  The tests compare the dumps of a
+// classic file and of the same content in NetCDF-4 containers of several layouts.
+#include <cinttypes>
+#include <cstdio>
+#include <cstring>
+#include <algorithm>
+#include <string>
+#include <vector>
+
+#include "NcClassic.h"
+
+static void printValues(int type, const uint8_t* p, uint64_t count)
+{
+    for (uint64_t i = 0; i < count; i++) {
+        switch (type) {
+        case ncc::NC_BYTE: printf(" %d", ((const int8_t*)p)[i]); break;
+        case ncc::NC_UBYTE: printf(" %u", p[i]); break;
+        case ncc::NC_SHORT: { int16_t v; memcpy(&v, p + 2 * i, 2); printf(" %d", v); break; }
+        case ncc::NC_USHORT: { uint16_t v; memcpy(&v, p + 2 * i, 2); printf(" %u", v); break; }
+        case ncc::NC_INT: { int32_t v; memcpy(&v, p + 4 * i, 4); printf(" %d", v); break; }
+        case ncc::NC_UINT: { uint32_t v; memcpy(&v, p + 4 * i, 4); printf(" %u", v); break; }
+        case ncc::NC_INT64: { int64_t v; memcpy(&v, p + 8 * i, 8); printf(" %" PRId64, v); break; }
+        case ncc::NC_UINT64: { uint64_t v; memcpy(&v, p + 8 * i, 8); printf(" %" PRIu64, v); break; }
+        case ncc::NC_FLOAT: { uint32_t v; memcpy(&v, p + 4 * i, 4); printf(" f%08x", v); break; }
+        case ncc::NC_DOUBLE: { uint64_t v; memcpy(&v, p + 8 * i, 8); printf(" d%016" PRIx64, v); break; }
+        default: printf(" ?"); break;
+        }
+    }
+}
+
+int main(int argc, char** argv)
+{
+    if (argc < 2) {
+        fprintf(stderr, "usage: nc_dump file.nc\n");
+        return 2;
+    }
+    try {
+        ncc::Reader nc(argv[1]);
+        fprintf(stderr, "container %d\n", nc.version());
+        std::vector<ncc::Dimension> dims = nc.dims();
+        std::sort(dims.begin(), dims.end(), [](const ncc::Dimension& a, const ncc::Dimension& b) { return a.name < b.name; });
+        for (const auto& d : dims) printf("dim %s %" PRIu64 "\n", d.name.c_str(), d.length);
+        std::vector<std::string> names = nc.attNames();
+        std::sort(names.begin(), names.end());
+        for (const auto& n : names) {
+            const ncc::Attribute& a = nc.att(n);
+            if (a.type == ncc::NC_CHAR)
+                printf("att %s text \"%s\"\n", n.c_str(), a.asString().c_str());
+            else {
+                printf("att %s type %d count %" PRIu64 ":", n.c_str(), a.type, a.count);
+                printValues(a.type, a.raw.data(), a.count);
+                printf("\n");
+            }
+        }
+        std::vector<std::string> vnames;
+        for (const auto& v : nc.vars()) vnames.push_back(v.name);
+        std::sort(vnames.begin(), vnames.end());
+        for (const auto& n : vnames) {
+            const ncc::Variable& v = nc.var(n);
+            std::vector<uint8_t> raw;
+            nc.readBytes(n, raw);
+            printf("var %s type %d count %" PRIu64 ":", n.c_str(), v.type, v.count);
+            printValues(v.type, raw.data(), v.count);
+            printf("\n");
+        }
+    } catch (const std::exception& e) {
+        printf("error: %s\n", e.what());
+        return 1;
+    }
+    return 0;
+}

@@ -476,3 +476,31 @@ def test_unit_buffer_read_with_a_bare_hipmemcpy(pkg, dsx, orc, synth):
             assert len(seen) == lanes
     finally:
         net.close()
+
+
+def test_network_file_in_netcdf4_container_predicts(pkg, dsx, orc, synth, tmp_path):
+    """LoadNeuralNetworkNetCDF on NetCDF-4 (HDF5) network files, the container the reference writes: the fixtures of
+    tests/golden/nc4 (written by the HDF5 library, old and new file-format generations, contiguous and chunked) through the
+    native embedding example (DsstneContext -> PredictBatch -> kCalculateTopK) must print what the classic file prints, and
+    that must be what the oracle predicts for the same weights."""
+    nc4 = os.path.join(ROOT, "tests", "golden", "nc4")
+    p = synth.autoencoder("small-nc4", 4242, 256, [32], 16, 5, 1, 1.0, 12, 0.5, (1, 40), bias_std=0.3)   # as make_fixtures.py builds it
+    inputs = tmp_path / "inputs.txt"
+    with open(inputs, "w") as f:
+        for r in range(p.batch):
+            f.write(" ".join(str(int(i)) for i in p.sparse_index[int(p.start[r]):int(p.end[r])]) + "\n")
+    outs = {}
+    for name in ("small.classic.nc", "small.earliest.nc", "small.v18.c1000.nc"):
+        rc, out = run_exe("predict_main", os.path.join(nc4, name), inputs, p.batch, p.k)
+        assert rc == 0, out[-3000:]
+        outs[name] = [l for l in out.splitlines() if l and l[0].isdigit() and "\t" in l]
+        assert len(outs[name]) == p.batch, out[-2000:]
+    assert outs["small.earliest.nc"] == outs["small.classic.nc"] and outs["small.v18.c1000.nc"] == outs["small.classic.nc"]
+    idx = np.zeros((p.batch, p.k), dtype=np.uint32)
+    keys = np.zeros((p.batch, p.k), dtype=np.float32)
+    for r, line in enumerate(outs["small.v18.c1000.nc"]):
+        for j, c in enumerate(c for c in line.split("\t")[1].split(",") if c):
+            i, s = c.split(":")
+            idx[r, j], keys[r, j] = int(i), float(s)
+    _, ref_unit, ref_keys, ref_idx = orc.forward(p, filtered=False, want_unit=True)
+    assert_topk_parity(keys, idx, ref_keys, ref_idx, ref_unit, "network from a NetCDF-4 file")
