@@ -26,18 +26,23 @@ import __graft_entry__ as entry  # noqa: E402
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP32_MFMA_PEAK_TF = 157.3    # MI355X dense fp32 matrix, published
 
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), scaled by what the same counters
-# read for a plain 256 MiB device-to-device copy (FETCH_SIZE reads half of the bytes, factor 2.0; WRITE_SIZE factor 1.0).
-# Measured on the cfg2 workload; the summary with the commands is profiles/pmc_cfg2_hbm_traffic.md.
-MEASURED_TRAFFIC = {
-    "cfg2-catalogue-27278": {
-        "sparse_z_kernel": {"fetch": 15080 * 1024 * 2.0, "write": 512 * 1024 * 1.0},
-        "fc_small_kernel[1024x128x128]": {"fetch": 1107 * 1024 * 2.0, "write": 512 * 1024 * 1.0},
-        "fc_gemm_kernel[1024x128x27278]": {"fetch": 11470 * 1024 * 2.0, "write": 147200 * 1024 * 1.0},
-        "topk_scan_kernel": {"fetch": 58540 * 1024 * 2.0, "write": 128 * 1024 * 1.0},
-        "topk_guided_kernel": {"fetch": 10610 * 1024 * 2.0, "write": 128 * 1024 * 1.0},
-    },
-}
+# HBM bytes per launch, measured: profiles/pmc_hbm_traffic.json holds, per workload and kernel, what rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE read (KiB per dispatch) and the calibration factors from a plain 256 MiB device-to-device copy in the same runs; the
+# summary beside it (profiles/pmc_cfg2_hbm_traffic.md) is made from the same file and gives the commands.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "pmc_hbm_traffic.json")
+BATCHES = 8                  # distinct batches resident in HBM that the timed loop cycles over
+WINDOWS = 5                  # timed windows of --steps steps each; the median is reported
+
+
+def measured_traffic(workload):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            t = json.load(f)
+    except OSError:
+        return {}
+    w = t.get("workloads", {}).get(workload, {})
+    ff, wf = t.get("fetch_factor", 1.0), t.get("write_factor", 1.0)
+    return {k: {"read": int(v["fetch_kib"] * 1024 * ff), "write": int(v["write_kib"] * 1024 * wf)} for k, v in w.items()}
 
 
 class StdoutToStderr:
@@ -82,56 +87,85 @@ def time_launches(pkg, lib, fn, reps):
     return ms.value / reps
 
 
+def timed_windows(step, sync, steps, windows):
+    """`windows` regions of exactly `steps` calls of step(i), each bracketed by sync(); milliseconds per step of every region."""
+    out = []
+    n = 0
+    for _ in range(windows):
+        sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step(n)
+            n += 1
+        sync()
+        out.append((time.perf_counter() - t0) * 1e3 / steps)
+    return out
+
+
 def network_bench(args, pkg, lib):
     from amazon_dsstne_amd import ATTR_BOOLEAN, ATTR_INDEXED, synth
     from amazon_dsstne_amd.pipeline import DevicePipeline
 
     from amazon_dsstne_amd.host_api import Network
 
-    p = synth.config(args.config)
+    batches = 1 if args.config == 4 else BATCHES      # config 4's generator takes seconds per batch; its step is 33 ms of GEMM
+    p = synth.config(args.config, batches=batches)
     B, H, N, K = p.batch, p.widths[1], p.widths[-1], p.k
     nnzB = p.batch_nnz()
+    nnz_mean = p.nnz / batches
 
     # The timed step goes through the C++ host layer, as a DSSTNE caller would: NNNetwork::PredictBatch on the resident input
     # dataset, then NNNetwork::CalculateFilteredTopK with the sample's own items as the filter.  Inputs, weights and
-    # results stay in HBM.
+    # results stay in HBM; consecutive steps take consecutive batches of the resident dataset.
     net = Network(p)
     net.bind_input()
 
-    def step():
-        net.predict_batch(0)
+    def step(i=0):
+        net.predict_batch((i % batches) * B)
         net.topk(K, filter_dataset=net.dataset)
+
+    # From idle the clocks of this part ramp up over tens of milliseconds: what a caller sees who sends a burst after a pause.
+    net.sync()
+    time.sleep(2.5)
+    for i in range(args.warmup):
+        step(i)
+    ms_cold = timed_windows(step, net.sync, args.steps, 1)[0]
+
     settle(pkg, lib, step)
-    for _ in range(args.warmup):
-        step()
-    net.sync()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    net.sync()
-    t1 = time.perf_counter()
-    ms_step = (t1 - t0) * 1e3 / args.steps
+    for i in range(args.warmup):
+        step(i)
+    windows = timed_windows(step, net.sync, args.steps, WINDOWS)
+    ms_step = float(np.median(windows))
 
     # The step above runs as NNNetwork does by default: consecutive batches alternate between two lanes (two sets of unit
     # buffers on two streams), so one batch's input layers and top-K overlap with the next one's GEMM.  The same on one
     # lane — the reference's single set of buffers, one batch's kernels strictly after the other's — for comparison.
     net.set_lanes(1)
     settle(pkg, lib, step)
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    net.sync()
-    ms_one_lane = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_one_lane = float(np.median(timed_windows(step, net.sync, args.steps, 3)))
     net.set_lanes(2)
-    step()
+    # ... and with the output layer stored by PredictBatch as the reference does, instead of computed together with the top-K
+    # (NNNetwork::SetDeferredOutput; only layers of 131,072 units or more are deferred, so this differs for config 4 alone)
+    net.set_deferred_output(False)
+    settle(pkg, lib, step)
+    ms_stored = float(np.median(timed_windows(step, net.sync, args.steps, 3)))
+    net.set_deferred_output(True)
     net.sync()
+    net.close()
 
     # The same step when the batch's CSR arrays are handed over as host buffers every time (NNDataSet::LoadSparseData, as the
-    # reference's JNI predict does): never `value`, reported beside it.
+    # reference's JNI predict does): never `value`, reported beside it.  (A second network whose dataset holds one batch.)
+    p1 = synth.config(args.config)
+    net = Network(p1)
+    net.bind_input()
+
+    def step1():
+        net.predict_batch(0)
+        net.topk(K, filter_dataset=net.dataset)
     up_steps = max(5, min(200, args.steps))
     def upload_step():
-        net.load_sparse(p.start, p.end, p.sparse_data, p.sparse_index)
-        step()
+        net.load_sparse(p1.start, p1.end, p1.sparse_data, p1.sparse_index)
+        step1()
     # untimed: the first uploads allocate the pinned staging buffers
     settle(pkg, lib, upload_step)
     # (median of four runs of up_steps: somewhere in its first thousand queued copies the HIP runtime grows its pools once, a
@@ -150,39 +184,47 @@ def network_bench(args, pkg, lib):
     rt = []
     for n in range(up_steps + 5):
         t0 = time.perf_counter()
-        net.load_sparse(p.start, p.end, p.sparse_data, p.sparse_index)
-        step()
+        net.load_sparse(p1.start, p1.end, p1.sparse_data, p1.sparse_index)
+        step1()
         net.get_topk(B)
         if n >= 5:
             rt.append(time.perf_counter() - t0)
     ms_request = float(np.median(rt)) * 1e3
+    net.close()
 
-    # The same kernels one at a time on the same shapes (raw C ABI of the kernel library, same stream).
+    # The same kernels one at a time on the first batch (raw C ABI of the kernel library, same stream): HIP events around
+    # back-to-back launches of one kernel, clocks settled.
     pipe = DevicePipeline(p, lib)
     pipe.step()
     pkg.check(lib.dsx_sync())
-
-    # per-kernel figures (HIP events around back-to-back launches of one kernel)
     reps = max(10, min(100, args.steps))
     params = C.byref(pipe.params)
     ptr = pkg.ptr
     kernels = {}
+    traffic = measured_traffic(p.name)
 
     def k_sparse():
         pkg.check(lib.dsx_sparse_layer_forward(p.attributes, p.data_type, 0, B, H, ptr(pipe.W[0]), ptr(pipe.index), ptr(pipe.start),
                                                ptr(pipe.end), ptr(pipe.sidx), ptr(pipe.dw), ptr(pipe.sdata), ptr(pipe.b[0]),
                                                p.acts[0], params, ptr(pipe.units[0])))
     val_bytes = 0 if (p.attributes & ATTR_BOOLEAN) else p.sparse_data.dtype.itemsize
-    spmm_bytes = nnzB * (4 * H + 4 + val_bytes) + B * (16 + (4 if (p.attributes & ATTR_INDEXED) else 0)) + 4 * H + 4 * B * H
+    fixed = B * (16 + (4 if (p.attributes & ATTR_INDEXED) else 0)) + 4 * H + 4 * B * H
+    spmm_bytes = nnzB * (4 * H + 4 + val_bytes) + fixed
+    rows0 = np.arange(B) if p.index is None else p.index[:B]
+    touched = np.unique(np.concatenate([p.sparse_index[int(p.start[r]):int(p.end[r])] for r in rows0])).size
+    compulsory = touched * 4 * H + nnzB * (4 + val_bytes) + fixed     # every distinct weight row once
     ms = time_launches(pkg, lib, k_sparse, reps)
     kernels["sparse_z_kernel"] = {"bound": "hbm", "ms": ms, "achieved": spmm_bytes / ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                  "algorithmic_bytes": spmm_bytes}
+                                  "algorithmic_bytes": spmm_bytes, "compulsory_bytes": compulsory,
+                                  "compulsory_gbs": compulsory / ms / 1e6,
+                                  "note": "algorithmic = every non-zero gathers its weight row (no reuse); compulsory = every distinct weight row of the batch once"}
 
-    # the dense layers as the timed step runs them: the last one also leaves segment maxima for the guided top-K
+    # the dense layers as the stored-output step runs them: the last one also leaves segment maxima for the guided top-K
     gp = DevicePipeline(p, lib, guided=True)
     gp.step()
     pkg.check(lib.dsx_sync())
     last = len(pipe.W) - 1
+    flops_step = 0.0
     for l in range(1, len(pipe.W)):
         kk, n = p.widths[l], p.widths[l + 1]
 
@@ -194,11 +236,13 @@ def network_bench(args, pkg, lib):
                 pkg.check(lib.dsx_fc_forward(ptr(pipe.units[l - 1]), kk, ptr(pipe.W[l]), 0, ptr(pipe.b[l]), ptr(pipe.units[l]), n, B, kk, n, 0,
                                              p.acts[l], params))
         flops = 2.0 * B * kk * n
+        flops_step += flops
         ms = time_launches(pkg, lib, k_fc, reps)
         small = (kk in (128, 256)) and B * n <= (1 << 20)
         name = "%s[%dx%dx%d]" % ("fc_small_kernel" if small else "fc_gemm_kernel", B, kk, n)
         kernels[name] = {"bound": "mfma", "ms": ms, "achieved": flops / ms / 1e9, "peak": FP32_MFMA_PEAK_TF, "unit": "TFLOP/s",
                          "algorithmic_flops": flops}
+    gemm_name = name
 
     def k_topk():
         pipe.topk()
@@ -206,23 +250,47 @@ def network_bench(args, pkg, lib):
     ms = time_launches(pkg, lib, k_topk, reps)
     kernels["topk_scan_kernel"] = {"bound": "hbm", "ms": ms, "achieved": topk_bytes / ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                    "algorithmic_bytes": topk_bytes}
-    if gp.seg_width.value:
-        # what the timed step runs when the output layer left segment maxima; priced with the scan's algorithmic bytes (it reads
-        # a fraction of them, so the figure can exceed the roofline: it measures the work avoided, not bandwidth)
-        ms = time_launches(pkg, lib, lambda: gp.topk(), reps)
-        kernels["topk_guided_kernel"] = {"bound": "hbm", "ms": ms, "achieved": topk_bytes / ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                         "algorithmic_bytes": topk_bytes, "note": "reads only the segments that can hold a result"}
     for v in kernels.values():
         v["frac"] = v["achieved"] / v["peak"]
+    if gp.seg_width.value:
+        # what the step runs when the output layer left segment maxima: it reads the maxima and the few segments that can hold a
+        # result, so it is a chain of dependent loads, not a stream.  Its figure is the bandwidth of what it really moves.
+        ms = time_launches(pkg, lib, lambda: gp.topk(), reps)
+        moved = traffic.get("topk_guided_kernel")
+        g = {"bound": "latency", "ms": ms, "replaces_scan_of_bytes": topk_bytes,
+             "note": "reads the segment maxima and the segments that can hold a result instead of scanning the row"}
+        if moved:
+            g.update({"achieved": (moved["read"] + moved["write"]) / ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s"})
+            g["frac"] = g["achieved"] / g["peak"]
+        kernels["topk_guided_kernel"] = g
+    deferred = N >= 131072      # NNLayer defers output layers from this width on
+    if deferred:
+        keys = pkg.DeviceArray((B, K), np.float32)
+        vals = pkg.DeviceArray((B, K), np.uint32)
 
-    for n, t in MEASURED_TRAFFIC.get(p.name, {}).items():
+        def k_fused():
+            pkg.check(lib.dsx_fc_topk(ptr(pipe.units[last - 1]), p.widths[last], ptr(pipe.W[last]), ptr(pipe.b[last]), B, p.widths[last], N,
+                                      p.acts[last], params, K, keys.ptr, vals.ptr, 0, ptr(pipe.index), ptr(pipe.start), ptr(pipe.end),
+                                      ptr(pipe.sidx)))
+        flops = 2.0 * B * p.widths[last] * N
+        ms = time_launches(pkg, lib, k_fused, max(5, reps // 4))
+        kernels["dsx_fc_topk (output layer + filtered top-K, nothing stored)"] = {
+            "bound": "mfma", "ms": ms, "achieved": flops / ms / 1e9, "peak": FP32_MFMA_PEAK_TF, "unit": "TFLOP/s",
+            "algorithmic_flops": flops, "frac": flops / ms / 1e9 / FP32_MFMA_PEAK_TF,
+            "note": "what the timed step runs for this layer: first column block stored and scanned, the rest compared in registers"}
+
+    for n, t in traffic.items():
         if n in kernels:
-            kernels[n]["traffic"] = int(t["fetch"] + t["write"])
+            kernels[n]["traffic"] = t["read"] + t["write"]
+            kernels[n]["traffic_read"] = t["read"]
+            kernels[n]["traffic_write"] = t["write"]
 
-    dominant = max(kernels, key=lambda n: kernels[n]["ms"])
+    candidates = [n for n in kernels if "frac" in kernels[n] and not (deferred and n in (gemm_name, "topk_scan_kernel"))]
+    dominant = max(candidates, key=lambda n: kernels[n]["ms"])
     d = kernels[dominant]
     roofline = {"kernel": dominant, "bound": d["bound"], "achieved": round(d["achieved"], 3), "peak": d["peak"], "unit": d["unit"],
-                "frac": round(d["frac"], 4), "traffic": d.get("traffic"), "avg_launch_ms": round(d["ms"], 5)}
+                "frac": round(d["frac"], 4), "traffic": d.get("traffic"), "avg_launch_ms": round(d["ms"], 5),
+                "note": "isolated back-to-back launches, clocks settled; `pipeline` below prices the whole timed step"}
     if args.calibrate_copy:
         # plain device-to-device copy of known size: what FETCH_SIZE / WRITE_SIZE read for it calibrates the counters
         nbytes = args.calibrate_copy << 20
@@ -249,9 +317,11 @@ def network_bench(args, pkg, lib):
         cpu = {"value": round(rows * nb / secs, 1), "unit": "samples/s", "cores": cores, "kind": "port",
                "sample": "%d passes over the first %d rows of one batch of %d of the same workload (%s), %.1f s" % (nb, rows, B, p.name, secs)}
 
+    def rate(ms):
+        return round(B / (ms / 1e3), 1)
     out = {
         "metric": "predicted samples/sec (sparse-in -> filtered top-K) at batch %d" % B,
-        "value": round(B / (ms_step / 1e3), 1),
+        "value": rate(ms_step),
         "unit": "samples/s",
         "n_gpus": 1,
         "steps": args.steps,
@@ -263,16 +333,26 @@ def network_bench(args, pkg, lib):
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": p.name, "batch": B, "input_width": p.widths[0], "layers": p.widths[1:], "top_k": K, "filtered": True,
-                   "batch_nnz": nnzB},
+                   "resident_batches": batches, "batch_nnz": nnzB, "mean_batch_nnz": round(nnz_mean, 1)},
+        "windows": {"count": WINDOWS, "steps_each": args.steps, "ms_per_step": [round(w, 5) for w in windows],
+                    "min": round(min(windows), 5), "median": round(ms_step, 5), "max": round(max(windows), 5),
+                    "note": "value is the median window; the timed steps cycle over the resident batches"},
         "roofline": roofline,
+        "pipeline": {"gemm_flops_per_step": flops_step, "achieved": round(flops_step / ms_step / 1e9, 3), "peak": FP32_MFMA_PEAK_TF,
+                     "unit": "TFLOP/s", "frac": round(flops_step / ms_step / 1e9 / FP32_MFMA_PEAK_TF, 4),
+                     "note": "all dense-layer flops of a step over the timed step itself (two lanes, every kernel of the step included): the fraction of the fp32 MFMA peak the whole path sustains"},
         "kernels": {n: {k: (round(v, 5) if isinstance(v, float) else v) for k, v in kv.items()} for n, kv in kernels.items()},
         "cpu_baseline": cpu,
         "clock_settle_ms": SETTLE_SECONDS * 1e3,
-        "one_lane": {"ms_per_step": round(ms_one_lane, 5), "value": round(B / (ms_one_lane / 1e3), 1), "unit": "samples/s",
+        "cold_clock": {"ms_per_step": round(ms_cold, 5), "value": rate(ms_cold), "unit": "samples/s",
+                       "note": "the same %d steps started after 2.5 s of idling, no settling load: the clocks are still ramping up" % args.steps},
+        "one_lane": {"ms_per_step": round(ms_one_lane, 5), "value": rate(ms_one_lane), "unit": "samples/s",
                      "note": "NNNetwork::SetLanes(1): one set of buffers, one stream, batches strictly one after the other"},
-        "with_input_upload": {"ms_per_step": round(ms_upload, 5), "value": round(B / (ms_upload / 1e3), 1), "unit": "samples/s",
+        "stored_output": {"ms_per_step": round(ms_stored, 5), "value": rate(ms_stored), "unit": "samples/s",
+                          "note": "NNNetwork::SetDeferredOutput(false): PredictBatch stores the output layer, the top-K reads it back (the same as the default below 131,072 output units)"},
+        "with_input_upload": {"ms_per_step": round(ms_upload, 5), "value": rate(ms_upload), "unit": "samples/s",
                               "note": "the batch's CSR arrays handed over as host memory before every step (NNDataSet::LoadSparseData; PCIe-inclusive): uploads go to alternating sets of device arrays on the lane of the batch they belong to"},
-        "request_round_trip": {"ms": round(ms_request, 5), "value": round(B / (ms_request / 1e3), 1), "unit": "samples/s",
+        "request_round_trip": {"ms": round(ms_request, 5), "value": rate(ms_request), "unit": "samples/s",
                                "note": "median over requests served one at a time: upload, predict, filtered top-K, results read back"},
     }
     return out

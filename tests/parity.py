@@ -58,3 +58,43 @@ def check_topk_invariants(scores, keys, idx, k, width=None):
         masked = scores[:, :width].copy()
         masked[rows, idx[:, :m]] = -np.inf
         assert np.all(masked.max(axis=1) <= keys[:, m - 1]), "an unselected score beats the k-th key"
+
+
+def forward_f64(p, rows):
+    """The chain network of a synth.Problem in float64 for the given batch positions (numpy only): the ground truth that both
+    the fp32 oracle and the GPU approximate."""
+    sig = lambda z: 1.0 / (1.0 + np.exp(-z))
+    acts = {0: sig, 1: np.tanh, 2: lambda z: np.maximum(z, 0.0), 3: lambda z: z}
+    out = []
+    for b in rows:
+        r = int(p.index[b]) if p.index is not None else int(b)
+        s, e = int(p.start[r]), int(p.end[r])
+        cols = p.sparse_index[s:e]
+        vals = np.ones(e - s) if p.sparse_data is None else p.sparse_data[s:e].astype(np.float64)
+        h = p.biases[0].astype(np.float64) + vals @ p.weights[0][cols].astype(np.float64)
+        h = acts[p.acts[0]](h)
+        for l in range(1, len(p.weights)):
+            h = acts[p.acts[l]](p.biases[l].astype(np.float64) + h @ p.weights[l].astype(np.float64))
+        out.append(h)
+    return np.asarray(out)
+
+
+def assert_units_close(got, ref, p, position=0, what="activations", rel=REL_TOL, abs_floor=1e-3, positions=None):
+    """Layer outputs against the fp32 oracle: within `rel` of it, or — where deep sums cancel and two fp32 summation orders part
+    by more than that — at least as close to the float64 ground truth as the oracle itself is (row by row: the largest deviation
+    from the truth at most twice the oracle's, plus one part in 10^6 of the row's largest value).  Row i of got / ref is batch position `position + i`, or positions[i]."""
+    got64, ref64 = np.asarray(got, dtype=np.float64), np.asarray(ref, dtype=np.float64)
+    err = np.abs(got64 - ref64) / np.maximum(np.abs(ref64), abs_floor)
+    bad_rows = np.nonzero((err > rel).any(axis=1))[0]
+    if bad_rows.size == 0:
+        return float(err.max()) if err.size else 0.0
+    assert bad_rows.size <= max(4, got.shape[0] // 20), "%s: %d rows differ from the oracle by more than %.0e" % (what, bad_rows.size, rel)
+    truth = forward_f64(p, (position + bad_rows) if positions is None else np.asarray(positions)[bad_rows])
+    e_got = np.abs(got64[bad_rows] - truth)
+    e_ref = np.abs(ref64[bad_rows] - truth)
+    # rounding errors fall on different elements in the two computations: compare their levels row by row
+    level_got, level_ref = e_got.max(axis=1), e_ref.max(axis=1)
+    worse = level_got > 2.0 * level_ref + 1e-6 * np.abs(truth).max(axis=1) + 1e-9
+    assert not worse.any(), "%s: %d rows are further from the float64 result than the fp32 oracle is (worst %.3g vs oracle %.3g)" % (
+        what, int(worse.sum()), float(level_got.max()), float(level_ref.max()))
+    return float(err.max())

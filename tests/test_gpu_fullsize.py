@@ -14,7 +14,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from parity import assert_close, assert_topk_parity
+from parity import assert_close, assert_topk_parity, assert_units_close
 
 pytestmark = pytest.mark.gpu
 
@@ -89,7 +89,7 @@ def run_network_config(pkg, dsx, orc, p, guided):
     check_batch_properties(p, keys, idx)
     ref_unit, ref_scores, ref_keys, ref_idx = oracle_rows(orc, p, picks, k)
     unit = download_rows(pkg, dsx, pipe.units[-1], N, picks)
-    assert_close(unit, ref_unit, "%s output activations of the sampled rows" % p.name, rel=1e-4, abs_floor=1e-3)
+    assert_units_close(unit, ref_unit, p, what="%s output activations of the sampled rows" % p.name, positions=picks)
     assert np.array_equal(unit[np.arange(len(picks))[:, None], idx[picks]], keys[picks]), "score is not the activation at the reported index"
     n = assert_topk_parity(keys[picks], idx[picks], ref_keys, ref_idx, ref_scores, p.name)
     say("%s: sampled rows agree with the oracle (%d tie-equivalent index differences)" % (p.name, n))

@@ -4,7 +4,7 @@ import os
 import numpy as np
 import pytest
 
-from parity import assert_close, assert_topk_parity
+from parity import assert_close, assert_topk_parity, assert_units_close
 
 pytestmark = pytest.mark.gpu
 
@@ -21,7 +21,7 @@ def run_and_compare(pkg, dsx, orc, p, position=0, batch=None, filtered=True, gui
     unit = pipe.output_unit(batch)
     _, ref_unit, _, _ = orc.forward(p, position, batch, filtered=False, want_unit=True, want_topk=False)
     _, _, ref_keys, ref_idx = orc.forward(p, position, batch, filtered=filtered)
-    assert_close(unit, ref_unit, "%s output activations" % p.name, rel=1e-4, abs_floor=1e-3)
+    assert_units_close(unit, ref_unit, p, position, "%s output activations" % p.name)
     ref_scores = ref_unit.copy()
     if filtered:
         b = p.batch if batch is None else batch

@@ -6,7 +6,7 @@ import subprocess
 import numpy as np
 import pytest
 
-from parity import assert_close, assert_topk_parity
+from parity import assert_close, assert_topk_parity, assert_units_close
 
 pytestmark = pytest.mark.gpu
 
@@ -46,7 +46,7 @@ def host_forward(pkg, dsx, orc, p, filtered=True, boolean=None, position=0):
         net.close()
     _, ref_unit, _, _ = orc.forward(p, position, rows, filtered=False, want_unit=True, want_topk=False)
     _, _, ref_keys, ref_idx = orc.forward(p, position, rows, filtered=filtered)
-    assert_close(unit, ref_unit, p.name + " units via NNNetwork", rel=1e-4, abs_floor=1e-3)
+    assert_units_close(unit, ref_unit, p, position, p.name + " units via NNNetwork")
     ref_scores = ref_unit.copy()
     if filtered:
         orc.lib().orc_apply_filter(ref_scores.ctypes.data, rows, ref_scores.shape[1], 0, position,
@@ -422,7 +422,7 @@ def test_two_lanes_keep_batches_apart(pkg, dsx, orc, synth, config, batches):
         net.predict_batch(positions[1])
         unit = net.units(rows=p.batch)
         _, ref_unit, _, _ = orc.forward(p, positions[1], p.batch, filtered=False, want_unit=True, want_topk=False)
-        assert_close(unit, ref_unit, p.name + " units on two lanes", rel=1e-4, abs_floor=1e-3)
+        assert_units_close(unit, ref_unit, p, positions[1], p.name + " units on two lanes")
         net.load_sparse(p.start, p.end, p.sparse_data, p.sparse_index)
         net.predict_batch(positions[0])
         net.topk(p.k, filter_dataset="input")
