@@ -509,10 +509,12 @@ __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kern
                 }
             }
         };
+        // With the default multiplier (every listed column is multiplied by 0) the listed scores are only of interest to a
+        // wavefront whose k-th score is not above 0 by the end of the scan: they are then read at that point, not up here.
 #pragma unroll
         for (int u = 0; u < kFU; u++) {
             fv[u] = 0.0f;
-            if (fcol[u] >= lo && fcol[u] < hi) fv[u] = row[fcol[u]];
+            if (a.fmul && fcol[u] >= lo && fcol[u] < hi) fv[u] = row[fcol[u]];
             mark(fcol[u]);
         }
         for (uint64_t t = fs + (uint64_t)kFU * kTopkThreads + threadIdx.x; t < fe; t += kTopkThreads) mark(a.fidx[t]);
@@ -623,16 +625,21 @@ __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kern
     // owns it (a column listed twice is injected once).  The bitmap is no longer consulted after the barrier.
     if constexpr (FILTERED) {
         __syncthreads();
-        for (uint64_t base = fs; base < fe; base += (uint64_t)kFU * kTopkThreads) {
-            if (base != fs) {
+        // A listed column multiplied by 0 scores 0 (or nothing at all, if its score is not finite): it cannot enter the list of
+        // a wavefront that already holds k scores above 0, and the final k-th score is at least that wavefront's.
+        const bool zeros_matter = a.fmul != nullptr || !(list.thr_key > 0.0f);   // wave-uniform
+        for (uint64_t base = fs; base < fe && zeros_matter; base += (uint64_t)kFU * kTopkThreads) {
+            if (base != fs || !a.fmul) {
+                if (base != fs) {
 #pragma unroll
-                for (int u = 0; u < kFU; u++) {
-                    const uint64_t t = base + (uint64_t)u * kTopkThreads + threadIdx.x;
-                    fcol[u] = 0xffffffffu;
-                    fm[u] = 0.0f;
-                    if (t < fe) {
-                        fcol[u] = a.fidx[t];
-                        if (a.fmul) fm[u] = a.fmul[t];
+                    for (int u = 0; u < kFU; u++) {
+                        const uint64_t t = base + (uint64_t)u * kTopkThreads + threadIdx.x;
+                        fcol[u] = 0xffffffffu;
+                        fm[u] = 0.0f;
+                        if (t < fe) {
+                            fcol[u] = a.fidx[t];
+                            if (a.fmul) fm[u] = a.fmul[t];
+                        }
                     }
                 }
 #pragma unroll
