@@ -504,3 +504,50 @@ def test_network_file_in_netcdf4_container_predicts(pkg, dsx, orc, synth, tmp_pa
             idx[r, j], keys[r, j] = int(i), float(s)
     _, ref_unit, ref_keys, ref_idx = orc.forward(p, filtered=False, want_unit=True)
     assert_topk_parity(keys, idx, ref_keys, ref_idx, ref_unit, "network from a NetCDF-4 file")
+
+
+def test_wide_output_layer_is_deferred_and_materialised_on_demand(pkg, dsx, orc, synth):
+    """An output layer of 131,072 units or more is not stored by PredictBatch: CalculateFilteredTopK / CalculateTopK run it
+    together with the top-K (dsx_fc_topk), GetUnits computes it when asked, and SetDeferredOutput(false) stores it as the
+    reference does.  All three must agree with the oracle, batch after batch on two lanes (the deferred state travels with the
+    lane's buffers), the last batch being short."""
+    from amazon_dsstne_amd import host_api
+    p = synth.autoencoder("wide-140k", 31, 140000, [64], 48, 20, batches=3, zipf_s=1.1, nnz_mean=30, nnz_sigma=0.8, nnz_clip=(1, 400))
+    short = 11
+    p.examples -= short
+    p.unique_examples -= short
+    p.start, p.end = p.start[:p.examples], p.end[:p.examples]
+    positions = list(range(0, p.examples, p.batch))
+    want = reference_batches(orc, p, positions)
+    dsx.dsx_fc_topk_flagged(1)
+    net = host_api.Network(p, max_k=p.k)
+    try:
+        net.bind_input()
+        for deferred in (True, False):
+            net.set_deferred_output(deferred)
+            got = []
+            for n, pos in enumerate(positions):
+                net.predict_batch(pos)
+                net.topk(p.k, filter_dataset="input")
+                if n > 0:
+                    got.append(net.get_topk_previous(want[n - 1][0]))
+            got.append(net.get_topk(want[-1][0]))
+            for n, ((rows, keys, idx, scores), (gk, gi)) in enumerate(zip(want, got)):
+                assert_topk_parity(gk, gi, keys, idx, scores, "%s batch %d, deferred=%s" % (p.name, n, deferred))
+        # unfiltered top-K of a deferred layer, then its units on demand, then the top-K again from the stored units
+        net.set_deferred_output(True)
+        net.predict_batch(positions[1])
+        net.topk(p.k, filter_dataset=None)
+        k1, i1 = net.get_topk(p.batch)
+        _, ref_unit, ref_keys, ref_idx = orc.forward(p, positions[1], p.batch, filtered=False, want_unit=True)
+        assert_topk_parity(k1, i1, ref_keys, ref_idx, ref_unit, "deferred, unfiltered")
+        unit = net.units(rows=p.batch)
+        assert_units_close(unit, ref_unit, p, positions[1], "units of a deferred layer, computed on demand")
+        net.topk(p.k, filter_dataset=None)
+        k2, i2 = net.get_topk(p.batch)
+        assert_topk_parity(k2, i2, ref_keys, ref_idx, ref_unit, "after the units were asked for")
+        rows = np.arange(p.batch)[:, None]
+        assert np.array_equal(unit[rows, i2], k2)          # now the scores are the stored units, bit for bit
+        assert dsx.dsx_fc_topk_flagged(0) == 0
+    finally:
+        net.close()
