@@ -814,13 +814,15 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
     }
     __syncthreads();
 
-    // One lane per column of a segment, four segments in flight per wave.
+    // One lane per column of a segment, eight segments in flight per wave: the usual dozen or two of segments are then one
+    // round trip, and a row full of ties (every segment reaches the bound) a few dozen instead of a hundred.
     const uint32_t count = sListCount;
-    for (uint32_t i0 = wave * 4; i0 < count; i0 += kTopkWaves * 4) {
-        float v[4];
-        uint32_t col[4];
+    constexpr int kSegsInFlight = 8;
+    for (uint32_t i0 = wave * kSegsInFlight; i0 < count; i0 += kTopkWaves * kSegsInFlight) {
+        float v[kSegsInFlight];
+        uint32_t col[kSegsInFlight];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < kSegsInFlight; u++) {
             v[u] = __uint_as_float(0x7fc00000u);   // NaN fails the compare below
             col[u] = 0;
             if (i0 + u < count) {
@@ -829,11 +831,12 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
             }
         }
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
+        for (int u = 0; u < kSegsInFlight; u++) {
             bool ok = v[u] >= list.thr_key;
             if (__ballot(ok) == 0) continue;
             if (ok) ok = !filtered_out(col[u]);
             list.stage_only(ok, pack_score(v[u], col[u]));
+            if ((u & 3) == 3) list.drain();   // at most four stagings of 64 words between two checks of the fill level
         }
         list.drain();
     }
