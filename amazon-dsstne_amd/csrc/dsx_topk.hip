@@ -145,6 +145,8 @@ template <int R> struct WaveTopK {
     uint64_t q[R];        // sorted descending over position r*64 + lane; 0 = empty slot
     uint64_t thr;         // current k-th word: candidates must be strictly larger
     float thr_key;        // its score: cheap first test is score >= thr_key
+    float thr_above;      // the next score above thr_key
+    uint32_t thr_col;     // the k-th word's column (0xffffffff while the threshold is a bare score bound)
     uint32_t count;       // staged candidates (wave-uniform)
     bool flushed;         // the register list holds something
     uint64_t* stage;      // LDS, kStageWords words, private to this wave
@@ -157,6 +159,8 @@ template <int R> struct WaveTopK {
         for (int r = 0; r < R; r++) q[r] = 0;
         thr = 0;
         thr_key = -__builtin_inff();
+        thr_above = -__builtin_inff();
+        thr_col = 0xffffffffu;
         count = 0;
         flushed = false;
         stage = stage_;
@@ -209,7 +213,17 @@ template <int R> struct WaveTopK {
             uint32_t col;
             unpack_score(t, key, col);
             thr_key = key;
+            thr_above = key_score((uint32_t)(t >> 32) + 1u);   // above +inf this is NaN, which nothing reaches
+            thr_col = col;
         }
+    }
+
+    // Lowest score a column at or beyond first_col needs.  A score equal to the k-th one wins only with a smaller column, so once
+    // the k-th word's column lies before first_col, ties are out: in a row of saturated scores (thousands of columns at exactly
+    // 1.0) the scan then skips every group with one compare, like any other row.
+    __device__ __forceinline__ float admission_score(uint32_t first_col) const
+    {
+        return (thr_col < first_col) ? thr_above : thr_key;
     }
 
     // Every word whose score key is below t can no longer reach the top k (t must be the key of a real score).
@@ -219,6 +233,7 @@ template <int R> struct WaveTopK {
         if (w > thr) {
             thr = w;
             thr_key = key_score(t);
+            thr_col = 0xffffffffu;
         }
     }
 
@@ -586,7 +601,7 @@ __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kern
         const uint32_t gbase = span + threadIdx.x;
         uint32_t hot = 0;
         {
-            const float t = list.thr_key;
+            const float t = list.admission_score(head + 4 * span);   // every column of this span and after is at or beyond that
 #pragma unroll
             for (int u = 0; u < CH; u++) {
                 const float m = fmaxf(fmaxf(cur[u].x, cur[u].y), fmaxf(cur[u].z, cur[u].w));
@@ -687,10 +702,11 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
     __shared__ uint64_t sStage[kTopkWaves][List::kStageWords];
     __shared__ uint32_t sPrime[kTopkWaves][kGuidedMaxK];
     __shared__ uint32_t sListCount;
-    extern __shared__ uint32_t sDyn[];   // segments to read [nseg] | best listed score per segment [nseg] | bitmap of listed columns
+    extern __shared__ uint32_t sDyn[];   // segments to read [nseg] | their maxima [nseg] | best listed score per segment [nseg] | bitmap of listed columns
     uint32_t* sList = sDyn;
-    uint32_t* sFiltMax = sDyn + a.nseg;
-    uint32_t* sBitmap = sDyn + 2 * a.nseg;
+    uint32_t* sListKey = sDyn + a.nseg;
+    uint32_t* sFiltMax = sDyn + 2 * a.nseg;
+    uint32_t* sBitmap = sDyn + 3 * a.nseg;
 
     const uint32_t b = blockIdx.x;
     const uint32_t wave = threadIdx.x / kWave;
@@ -810,12 +826,17 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
         uint32_t base = 0;
         if (lane == 0) base = atomicAdd(&sListCount, (uint32_t)__popcll(m));
         base = (uint32_t)__builtin_amdgcn_readfirstlane((int)base);
-        if (flagged) sList[base + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u))] = idx;
+        if (flagged) {
+            const uint32_t pos = base + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+            sList[pos] = idx;
+            sListKey[pos] = mk[e];
+        }
     }
     __syncthreads();
 
-    // One lane per column of a segment, eight segments in flight per wave: the usual dozen or two of segments are then one
-    // round trip, and a row full of ties (every segment reaches the bound) a few dozen instead of a hundred.
+    // One lane per column of a segment, eight segments in flight per wave: the usual dozen or two of segments are one round
+    // trip.  A segment whose maximum no longer reaches what its columns need is not read: in a row of saturated scores every
+    // segment reaches the bound, but once a wavefront holds k of them, later segments that only tie are out.
     const uint32_t count = sListCount;
     constexpr int kSegsInFlight = 8;
     for (uint32_t i0 = wave * kSegsInFlight; i0 < count; i0 += kTopkWaves * kSegsInFlight) {
@@ -826,8 +847,11 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
             v[u] = __uint_as_float(0x7fc00000u);   // NaN fails the compare below
             col[u] = 0;
             if (i0 + u < count) {
-                col[u] = sList[i0 + u] * kGuidedSegWidth + lane;
-                if (col[u] < a.width) v[u] = row[col[u]];
+                const uint32_t first = sList[i0 + u] * kGuidedSegWidth;
+                if (key_score(sListKey[i0 + u]) >= list.admission_score(first)) {   // wave-uniform
+                    col[u] = first + lane;
+                    if (col[u] < a.width) v[u] = row[col[u]];
+                }
             }
         }
 #pragma unroll
@@ -1284,7 +1308,7 @@ int topk_guided_run(const float* in, uint32_t width, uint32_t batch, uint32_t k,
 {
     const bool filtered = fidx != nullptr;
     const uint32_t nseg = (width + kGuidedSegWidth - 1) / kGuidedSegWidth;
-    size_t lds = (size_t)nseg * 4;
+    size_t lds = (size_t)nseg * 8;
     if (filtered) lds += (size_t)nseg * 4 + ((size_t)(width + 31) / 32) * 4;
     if (!seg_max || seg_width != kGuidedSegWidth || k > kGuidedMaxK || nseg > kGuidedMaxSegs || lds > 40 * 1024)
         return topk_run(in, width, width, batch, k, keys, values, position, index, fstart, fend, fidx, fmul, 0, nullptr, 0, 0, 0);
