@@ -123,5 +123,12 @@ uint64_t knn_f16_rows(uint64_t rows);
 int knn_to_f16(const float* src, bool colmajor, uint64_t src_ld, uint32_t rows_valid, uint32_t dim, void* dst, uint32_t rows_out);
 int knn_f16_scores_run(const void* queries16, const void* items16, uint32_t ld, uint32_t batch, uint32_t n, float* Z, uint32_t ldz,
                        const CandArgs* cand);
-int knn_refresh(uint64_t* best, const uint64_t* cand, uint32_t* cand_count, uint32_t cap, uint32_t k, uint32_t* row_bound, uint32_t batch);
+int knn_refresh(uint64_t* best, const uint64_t* cand, uint32_t* cand_count, uint32_t cap, uint32_t k, uint32_t* row_bound, uint32_t batch,
+                const uint64_t* seg = nullptr, uint32_t* seg_count = nullptr, uint32_t chunks = 0, uint32_t seg_cap = 0);
+// fp16 storage, long column ranges: every workgroup sweeps a chunk of the range and keeps (row, chunk) lists of its own
+// (seg [queries][chunks][seg_cap], seg_count [queries][64]); full lists spill into cand's shared ones.
+uint32_t knn_f16_sweep_chunks(uint32_t batch);
+bool knn_f16_sweep_applies(uint32_t batch, uint32_t n);
+int knn_f16_sweep_run(const void* queries16, const void* items16, uint32_t ld, uint32_t batch, uint32_t n, const CandArgs& cand, uint64_t* seg,
+                      uint32_t* seg_count, uint32_t seg_cap);
 }  // namespace dsx

@@ -22,6 +22,7 @@ static LibScratch g_knn_ws_of[2];   // per lane
 
 static uint32_t g_knn_block_columns = 0;   // 0: sized by the rule below
 static int g_knn_last_path = 0;            // how the last search ran: DSX_KNN_PATH_*
+static int g_knn_f16_sweep = 1;            // fp16 storage: 0 never sweeps, 1 sweeps long column ranges (knn_f16_sweep_kernel), 2 every range it can
 
 static uint32_t knn_block_columns(uint32_t rows_padded, uint32_t num_queries)
 {
@@ -52,6 +53,8 @@ struct KnnWorkspace {
     uint32_t* overflow;     // [1] (+ padding)
     uint64_t* cand;         // [queries][kCandCap]
     void* queries16;        // fp16 storage only: the query batch, [queries rounded up to 256][ld] halves
+    uint64_t* seg;          // fp16 storage only: [queries][chunks][kCandCap / chunks], the lists of a sweep (knn_f16_sweep_run)
+    uint32_t* seg_count;    // fp16 storage only: [queries][64]
     size_t bytes;
 };
 
@@ -72,7 +75,15 @@ static KnnWorkspace knn_layout(void* base, uint32_t rows_padded, uint32_t num_qu
     w.cand = (uint64_t*)p;
     p += align256((size_t)num_queries * kCandCap * sizeof(uint64_t));
     w.queries16 = p;
-    if (f16) p += align256((size_t)knn_f16_rows(num_queries) * knn_f16_ld(dim) * 2);
+    w.seg = nullptr;
+    w.seg_count = nullptr;
+    if (f16) {
+        p += align256((size_t)knn_f16_rows(num_queries) * knn_f16_ld(dim) * 2);
+        w.seg = (uint64_t*)p;
+        p += align256((size_t)num_queries * kCandCap * sizeof(uint64_t));
+        w.seg_count = (uint32_t*)p;
+        p += align256((size_t)num_queries * 64 * sizeof(uint32_t));
+    }
     w.bytes = (size_t)(p - (char*)base);
     return w;
 }
@@ -91,8 +102,13 @@ struct KnnOperands {
         if (f16) return knn_f16_scores_run(queries16, items16 + (uint64_t)c0 * ld16 * 2, ld16, num_queries, ncols, Z, ldz, nullptr);
         return fc_run(queries, dim, items + c0, rows_padded, 0, nullptr, Z, ldz, num_queries, dim, ncols, 0, DSX_ACT_LINEAR, nullptr);
     }
-    int into_candidates(uint32_t c0, uint32_t ncols, uint32_t num_queries, const CandArgs& cand) const
+    int into_candidates(uint32_t c0, uint32_t ncols, uint32_t num_queries, const CandArgs& cand, uint64_t* seg, uint32_t* seg_count) const
     {
+        const bool sweep = g_knn_f16_sweep == 2 ? (ncols + 127) / 128 >= knn_f16_sweep_chunks(num_queries)
+                                                : (g_knn_f16_sweep == 1 && knn_f16_sweep_applies(num_queries, ncols));
+        if (f16 && seg && sweep)
+            return knn_f16_sweep_run(queries16, items16 + (uint64_t)c0 * ld16 * 2, ld16, num_queries, ncols, cand, seg, seg_count,
+                                     kCandCap / knn_f16_sweep_chunks(num_queries));
         if (f16) return knn_f16_scores_run(queries16, items16 + (uint64_t)c0 * ld16 * 2, ld16, num_queries, ncols, nullptr, 0, &cand);
         return fc_candidates_run(queries, dim, items + c0, rows_padded, num_queries, dim, ncols, cand);
     }
@@ -149,6 +165,8 @@ static int knn_search_candidates(const KnnWorkspace& w, const KnnOperands& op, u
     const uint32_t cb = knn_block_columns(op.rows_padded, num_queries);
     const uint32_t clear_words = 2 * num_queries + 64;
     hipLaunchKernelGGL(knn_clear_kernel, dim3((clear_words + 255) / 256), dim3(256), 0, s, w.row_bound, clear_words);
+    if (w.seg_count) hipLaunchKernelGGL(knn_clear_kernel, dim3((num_queries * 64 + 255) / 256), dim3(256), 0, s, w.seg_count, num_queries * 64);
+    const uint32_t chunks = w.seg ? knn_f16_sweep_chunks(num_queries) : 0;
     uint32_t done = std::min(cb, M);
     t.start(s);
     int rc = op.into_matrix(0, done, num_queries, w.block_scores, cb);
@@ -164,11 +182,12 @@ static int knn_search_candidates(const KnnWorkspace& w, const KnnOperands& op, u
         const uint32_t ncols = (uint32_t)std::min<uint64_t>((uint64_t)M - done, (uint64_t)done * 4 / 128 * 128);
         t.start(s);
         const CandArgs cand{w.row_bound, w.cand, w.cand_count, kCandCap, done, w.overflow};
-        rc = op.into_candidates(done, ncols, num_queries, cand);
+        rc = op.into_candidates(done, ncols, num_queries, cand, w.seg, w.seg_count);
         if (rc) return rc;
         t.stop(s, t.gemm);
         t.start(s);
-        rc = knn_refresh(w.partial, w.cand, w.cand_count, kCandCap, k, w.row_bound, num_queries);
+        rc = knn_refresh(w.partial, w.cand, w.cand_count, kCandCap, k, w.row_bound, num_queries, w.seg, w.seg_count, chunks,
+                         chunks ? kCandCap / chunks : 0);
         if (rc) return rc;
         t.stop(s, t.topk);
         done += ncols;
@@ -197,6 +216,13 @@ int dsx_knn_set_block_columns(uint32_t columns)
 }
 
 int dsx_knn_last_search_path(void) { return g_knn_last_path; }
+
+int dsx_knn_f16_set_sweep(int mode)
+{
+    DSX_CHECK_ARG(mode >= 0 && mode <= 2, "dsx_knn_f16_set_sweep: mode %d (0, 1 or 2)", mode);
+    g_knn_f16_sweep = mode;
+    return DSX_OK;
+}
 
 size_t dsx_knn_workspace_bytes(uint32_t rows_padded, uint32_t dim, uint32_t num_queries, uint32_t k)
 {

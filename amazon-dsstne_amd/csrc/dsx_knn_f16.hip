@@ -147,6 +147,194 @@ __global__ __launch_bounds__(64 * WM * WN) __attribute__((amdgpu_waves_per_eu(WP
     }
 }
 
+// Candidate mode for long column ranges: a workgroup keeps its 128 queries and sweeps a contiguous chunk of the range's item
+// tiles, one after the other.  What a tile costs beyond its multiplications then shrinks to the compares:
+//  * the operand stream never stops at a tile boundary — the loads of the next tile's first two steps are in flight while
+//    the current tile's last steps are multiplied, so no tile waits for its first operands;
+//  * the rows' bounds are read once per workgroup, not once per tile;
+//  * survivors go to lists that belong to this (row, chunk) alone, a[row][chunk][seg_cap], whose fill counts live in LDS:
+//    no atomic on device memory (thousands of cycles of round trip per tile in knn_f16_kernel), only a plain store.  The
+//    counts are published when the sweep ends.  A (row, chunk) list that is full spills into the row's shared list, the one
+//    knn_f16_kernel appends to (CandArgs), so clustered items cost time, not exactness.
+// The 80-byte LDS rows of the operand tiles have 16 bytes of padding each; row r of the first query buffer keeps row r's
+// fill count and bound there, so the kernel needs no LDS beyond the operand buffers and four workgroups still share a CU.
+constexpr uint32_t kSweepCountStride = 64;   // seg_count is [queries][64]; chunks <= 64
+
+struct KnnF16SweepArgs {
+    const _Float16* A;      // queries [rows rounded up to 256][ld]
+    const _Float16* B;      // items of this column range [columns rounded up to 256][ld]
+    uint32_t ld;
+    uint32_t batch, n;
+    uint32_t tiles_m, tiles_n;
+    uint32_t chunks, tiles_per_chunk;
+    uint64_t* seg;          // [queries][chunks][seg_cap]
+    uint32_t* seg_count;    // [queries][kSweepCountStride]
+    uint32_t seg_cap;
+    CandArgs cand;          // bounds, column offset, and the shared lists a full (row, chunk) list spills into
+};
+
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void knn_f16_sweep_kernel(KnnF16SweepArgs a)
+{
+    constexpr int MI = 2, NI = 2, WN = 2, BM = 128, BN = 128, BK = 32, PITCH = BK + 8, RS = 64;
+    __shared__ __attribute__((aligned(16))) _Float16 sA[2][BM][PITCH];
+    __shared__ __attribute__((aligned(16))) _Float16 sB[2][BN][PITCH];
+
+    // Workgroups that sweep the same chunk (the same item tiles, different queries) sit on the same XCD and advance at the
+    // same rate: an item tile comes from HBM once and from that XCD's L2 for the others.
+    const uint32_t total = a.tiles_m * a.chunks;
+    uint32_t wg = blockIdx.x;
+    {
+        const uint32_t per_xcd = (total + kF16Xcds - 1) / kF16Xcds;
+        const uint32_t xcd = wg % kF16Xcds, local = wg / kF16Xcds;
+        wg = xcd * per_xcd + local;
+        if (local >= per_xcd || wg >= total) return;
+    }
+    const uint32_t tm = wg % a.tiles_m, chunk = wg / a.tiles_m;
+    const uint32_t row0 = tm * BM;
+    const uint32_t t0 = chunk * a.tiles_per_chunk;
+    const uint32_t t1 = min(t0 + a.tiles_per_chunk, a.tiles_n);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int l32 = lane & 31, lhi = lane >> 5;
+    if (t0 >= t1) {   // more chunks than tiles: an empty list
+        if (tid < BM && row0 + tid < a.batch) a.seg_count[(uint64_t)(row0 + tid) * kSweepCountStride + chunk] = 0;
+        return;
+    }
+    // row r's state: [0] fill count of its list, [1] its bound as a float (key 0: no bound yet, everything that is a number passes)
+    auto row_state = [&](int r) __attribute__((always_inline)) { return reinterpret_cast<uint32_t*>(&sA[0][r][BK]); };
+    if (tid < BM) {
+        float bound = __builtin_inff();   // rows beyond the batch admit nothing
+        if (row0 + tid < a.batch) {
+            const uint32_t key = a.cand.row_bound[row0 + tid];
+            bound = key ? key_score(key) : -__builtin_inff();
+        }
+        row_state(tid)[0] = 0;
+        row_state(tid)[1] = __float_as_uint(bound);
+    }
+
+    floatx16 acc[MI][NI];
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < NI; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    // The operand stream: step after step of 32 components, tile after tile.  The cursor stops at the chunk's last tile (what
+    // is requested beyond the end is that tile again and never used).
+    const int srow = tid >> 2, spart = tid & 3;
+    const uint32_t nk = a.ld / BK;   // a multiple of 2
+    const uint32_t rstep = RS * (a.ld / 8);
+    const uint64_t tile_step = (uint64_t)BN * (a.ld / 8);
+    const uint4* gA = reinterpret_cast<const uint4*>(a.A + (uint64_t)(row0 + srow) * a.ld) + spart;
+    const uint4* gB = reinterpret_cast<const uint4*>(a.B + ((uint64_t)t0 * BN + srow) * a.ld) + spart;
+    uint32_t cur_kt = 0, cur_t = t0;
+#define F16_LOAD(S)                                \
+    do {                                           \
+        const uint32_t o_ = cur_kt * (BK / 8);     \
+        S##a0 = gA[o_];                            \
+        S##a1 = gA[o_ + rstep];                    \
+        S##b0 = gB[o_];                            \
+        S##b1 = gB[o_ + rstep];                    \
+        if (++cur_kt == nk) {                      \
+            cur_kt = 0;                            \
+            if (cur_t + 1 < t1) {                  \
+                cur_t++;                           \
+                gB += tile_step;                   \
+            }                                      \
+        }                                          \
+    } while (0)
+#define F16_STORE(S, BUF)                                                         \
+    do {                                                                          \
+        *reinterpret_cast<uint4*>(&sA[BUF][srow][spart * 8]) = S##a0;             \
+        *reinterpret_cast<uint4*>(&sA[BUF][srow + RS][spart * 8]) = S##a1;        \
+        *reinterpret_cast<uint4*>(&sB[BUF][srow][spart * 8]) = S##b0;             \
+        *reinterpret_cast<uint4*>(&sB[BUF][srow + RS][spart * 8]) = S##b1;        \
+    } while (0)
+    auto multiply = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ks++) {
+            half8 av[MI], bv[NI];
+#pragma unroll
+            for (int i = 0; i < MI; i++) av[i] = *reinterpret_cast<const half8*>(&sA[buf][wm * 32 * MI + i * 32 + l32][ks * 16 + lhi * 8]);
+#pragma unroll
+            for (int j = 0; j < NI; j++) bv[j] = *reinterpret_cast<const half8*>(&sB[buf][wn * 32 * NI + j * 32 + l32][ks * 16 + lhi * 8]);
+#pragma unroll
+            for (int i = 0; i < MI; i++)
+#pragma unroll
+                for (int j = 0; j < NI; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[j], acc[i][j], 0, 0, 0);
+        }
+    };
+
+    uint4 s0a0, s0a1, s0b0, s0b1, s1a0, s1a1, s1b0, s1b1;
+    F16_LOAD(s0);
+    F16_LOAD(s1);
+    F16_STORE(s0, 0);
+    __syncthreads();   // also publishes the rows' state
+    for (uint32_t t = t0; t < t1; t++) {
+        __builtin_amdgcn_s_setprio(3);   // multiplying wavefronts first, comparing ones in the issue slots that are left
+        for (uint32_t kt = 0; kt < nk; kt += 2) {
+            F16_LOAD(s0);
+            multiply(0);
+            F16_STORE(s1, 1);
+            __syncthreads();
+            F16_LOAD(s1);
+            multiply(1);
+            F16_STORE(s0, 0);   // after a tile's last step: the next tile's first
+            __syncthreads();
+        }
+        __builtin_amdgcn_s_setprio(0);
+        // The tile against the rows' bounds: one compare per score; a 32 x 32 block without survivors costs nothing else.
+        const uint32_t colbase = t * BN + wn * 32 * NI;
+#pragma unroll
+        for (int i = 0; i < MI; i++) {
+            float bf[16];
+#pragma unroll
+            for (int v = 0; v < 16; v++) bf[v] = __uint_as_float(row_state(wm * 32 * MI + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4))[1]);
+#pragma unroll
+            for (int j = 0; j < NI; j++) {
+                uint64_t any = 0;
+#pragma unroll
+                for (int v = 0; v < 16; v++) any |= __builtin_amdgcn_ballot_w64(acc[i][j][v] >= bf[v]);
+                if (any != 0) {
+                    const uint32_t col = colbase + j * 32 + l32;
+                    const bool col_ok = col < a.n;   // columns beyond the range hold sums over zero padding
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        float x = acc[i][j][v];
+                        asm volatile("" : "+v"(x));
+                        const bool pass = x >= bf[v] && col_ok;
+                        if (__builtin_amdgcn_ballot_w64(pass) == 0) continue;
+                        if (pass) {
+                            // (the row is made opaque so that the list addresses of all 64 registers are worked out here, where one
+                            // is needed, and not kept in registers across the sweep)
+                            uint32_t rl = wm * 32 * MI + i * 32 + 8 * (v / 4) + 4 * lhi + (v % 4);
+                            asm volatile("" : "+v"(rl));
+                            const uint32_t r = row0 + rl;
+                            const uint64_t word = ((uint64_t)score_key(x) << 32) | (uint32_t)~(a.cand.col_offset + col);
+                            const uint32_t pos = atomicAdd(&row_state(rl)[0], 1u);
+                            if (pos < a.seg_cap) {
+                                a.seg[((uint64_t)r * a.chunks + chunk) * a.seg_cap + pos] = word;
+                            } else {   // this (row, chunk) list is full: the row's shared list
+                                const uint32_t p2 = atomicAdd(&a.cand.cand_count[r], 1u);
+                                if (p2 < a.cand.cand_cap) a.cand.cand[(uint64_t)r * a.cand.cand_cap + p2] = word;
+                                else *a.cand.overflow = 1u;
+                            }
+                        }
+                    }
+                }
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+            }
+        }
+    }
+#undef F16_LOAD
+#undef F16_STORE
+    __syncthreads();
+    if (tid < BM && row0 + tid < a.batch)
+        a.seg_count[(uint64_t)(row0 + tid) * kSweepCountStride + chunk] = min(row_state(tid)[0], a.seg_cap);
+}
+
 // fp32 -> fp16, round to nearest even (__float2half), into the padded row-major layout.  src is either column-major
 // (items: src[d * src_ld + row]) or row-major (queries: src[row * src_ld + d]); rows >= rows_valid and components >= dim
 // become zero.  One lane per 8 output halves.
@@ -227,6 +415,48 @@ int knn_f16_scores_run(const void* queries16, const void* items16, uint32_t ld, 
     // 256 x 256 tiles with eight wavefronts (6.6 ms vs 6.0), three workgroups per CU (6.3 ms).
     launch_f16<2, 2, 2, 2, 4>(a, cand);
     DSX_LAUNCH_CHECK("knn_f16_kernel");
+    return DSX_OK;
+}
+
+// Chunks per row tile for a search of `batch` queries: enough workgroups to fill every CU four times, at most 64.
+uint32_t knn_f16_sweep_chunks(uint32_t batch)
+{
+    const uint32_t tiles_m = (batch + 127) / 128;
+    const uint32_t want = 4 * (uint32_t)ctx().num_cus;
+    uint32_t chunks = (want + tiles_m - 1) / tiles_m;
+    if (chunks > kSweepCountStride) chunks = kSweepCountStride;
+    return chunks;
+}
+
+// Whether a range of n columns is worth a sweep: workgroups for every CU, and at least four tiles in every chunk.
+bool knn_f16_sweep_applies(uint32_t batch, uint32_t n)
+{
+    const uint32_t tiles_m = (batch + 127) / 128, tiles_n = (n + 127) / 128;
+    const uint32_t chunks = knn_f16_sweep_chunks(batch);
+    return tiles_m * chunks >= 2 * (uint32_t)ctx().num_cus && tiles_n >= 4 * chunks;
+}
+
+int knn_f16_sweep_run(const void* queries16, const void* items16, uint32_t ld, uint32_t batch, uint32_t n, const CandArgs& cand, uint64_t* seg,
+                      uint32_t* seg_count, uint32_t seg_cap)
+{
+    KnnF16SweepArgs a{};
+    a.A = (const _Float16*)queries16;
+    a.B = (const _Float16*)items16;
+    a.ld = ld;
+    a.batch = batch;
+    a.n = n;
+    a.tiles_m = (batch + 127) / 128;
+    a.tiles_n = (n + 127) / 128;
+    a.chunks = knn_f16_sweep_chunks(batch);
+    a.tiles_per_chunk = (a.tiles_n + a.chunks - 1) / a.chunks;
+    a.seg = seg;
+    a.seg_count = seg_count;
+    a.seg_cap = seg_cap;
+    a.cand = cand;
+    const uint32_t total = a.tiles_m * a.chunks;
+    const uint32_t grid = ((total + kF16Xcds - 1) / kF16Xcds) * kF16Xcds;
+    hipLaunchKernelGGL(knn_f16_sweep_kernel, dim3(grid), dim3(256), 0, ctx().stream, a);
+    DSX_LAUNCH_CHECK("knn_f16_sweep_kernel");
     return DSX_OK;
 }
 

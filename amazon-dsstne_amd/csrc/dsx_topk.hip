@@ -1046,13 +1046,16 @@ int topk_merge(const uint64_t* partial, uint32_t slots, uint32_t k, float* keys,
 
 // Exact KNN with candidate lists: merges a row's running best list (k packed words, best first) with the candidates the last
 // column range left behind, writes the best k back, raises the row's bound to their k-th key and empties the candidate
-// list.  One wavefront per row.
+// lists.  One wavefront per row.  The candidates are the row's shared list (cand, cand_count) and, after a sweep
+// (knn_f16_sweep_kernel), its `chunks` private lists seg[row][chunk][seg_cap] with fill counts seg_count[row][64].
 template <int R>
 __global__ __launch_bounds__(kWave) void knn_refresh_kernel(uint64_t* best, const uint64_t* cand, uint32_t* cand_count, uint32_t cap,
-                                                            uint32_t k, uint32_t* row_bound)
+                                                            uint32_t k, uint32_t* row_bound, const uint64_t* seg, uint32_t* seg_count,
+                                                            uint32_t chunks, uint32_t seg_cap)
 {
     using List = WaveTopK<R>;
     __shared__ uint64_t sStage[List::kStageWords];
+    __shared__ uint32_t sStart[kWave + 1];
     const uint32_t b = blockIdx.x;
     const uint32_t lane = threadIdx.x;
     List list;
@@ -1070,6 +1073,38 @@ __global__ __launch_bounds__(kWave) void knn_refresh_kernel(uint64_t* best, cons
         const uint64_t word = (p < n) ? src[p] : 0ull;
         list.offer(word != 0, word);
     }
+    if (seg) {
+        // entry e of the chunks' lists laid end to end: lane c holds where chunk c starts
+        uint32_t* counts = seg_count + (uint64_t)b * kWave;
+        const uint32_t mine_count = (lane < chunks) ? min(counts[lane], seg_cap) : 0u;
+        uint32_t incl = mine_count;
+#pragma unroll
+        for (int d = 1; d < kWave; d *= 2) {
+            const uint32_t below = __shfl_up(incl, d);
+            if (lane >= (uint32_t)d) incl += below;
+        }
+        if (lane == 0) sStart[0] = 0;
+        sStart[lane + 1] = incl;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const uint32_t total = sStart[kWave];
+        const uint64_t* lists = seg + (uint64_t)b * chunks * seg_cap;
+        for (uint32_t e0 = 0; e0 < total; e0 += kWave) {
+            const uint32_t e = e0 + lane;
+            uint64_t word = 0;
+            if (e < total) {
+                uint32_t lo = 0, hi = kWave;   // the last chunk that starts at or before e (empty chunks start where the next one does)
+                while (hi - lo > 1) {
+                    const uint32_t mid = (lo + hi) / 2;
+                    if (sStart[mid] <= e) lo = mid;
+                    else hi = mid;
+                }
+                word = lists[(uint64_t)lo * seg_cap + (e - sStart[lo])];
+            }
+            list.offer(word != 0, word);
+        }
+        if (lane < chunks) counts[lane] = 0;
+    }
     list.finish();
 #pragma unroll
     for (int r = 0; r < R; r++) {
@@ -1080,15 +1115,21 @@ __global__ __launch_bounds__(kWave) void knn_refresh_kernel(uint64_t* best, cons
     if (lane == 0) cand_count[b] = 0;
 }
 
-int knn_refresh(uint64_t* best, const uint64_t* cand, uint32_t* cand_count, uint32_t cap, uint32_t k, uint32_t* row_bound, uint32_t batch)
+int knn_refresh(uint64_t* best, const uint64_t* cand, uint32_t* cand_count, uint32_t cap, uint32_t k, uint32_t* row_bound, uint32_t batch,
+                const uint64_t* seg, uint32_t* seg_count, uint32_t chunks, uint32_t seg_cap)
 {
     hipStream_t s = ctx().stream;
+    if (seg && (chunks == 0 || chunks > (uint32_t)kWave || !seg_count))
+        return set_error(DSX_EINVAL, "knn_refresh: %u chunks (1..64)", chunks);
     if (k <= 64)
-        hipLaunchKernelGGL((knn_refresh_kernel<1>), dim3(batch), dim3(kWave), 0, s, best, cand, cand_count, cap, k, row_bound);
+        hipLaunchKernelGGL((knn_refresh_kernel<1>), dim3(batch), dim3(kWave), 0, s, best, cand, cand_count, cap, k, row_bound, seg, seg_count,
+                           chunks, seg_cap);
     else if (k <= 128)
-        hipLaunchKernelGGL((knn_refresh_kernel<2>), dim3(batch), dim3(kWave), 0, s, best, cand, cand_count, cap, k, row_bound);
+        hipLaunchKernelGGL((knn_refresh_kernel<2>), dim3(batch), dim3(kWave), 0, s, best, cand, cand_count, cap, k, row_bound, seg, seg_count,
+                           chunks, seg_cap);
     else
-        hipLaunchKernelGGL((knn_refresh_kernel<4>), dim3(batch), dim3(kWave), 0, s, best, cand, cand_count, cap, k, row_bound);
+        hipLaunchKernelGGL((knn_refresh_kernel<4>), dim3(batch), dim3(kWave), 0, s, best, cand, cand_count, cap, k, row_bound, seg, seg_count,
+                           chunks, seg_cap);
     DSX_LAUNCH_CHECK("knn_refresh_kernel");
     return DSX_OK;
 }

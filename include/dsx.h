@@ -320,6 +320,11 @@ int dsx_knn_set_block_columns(uint32_t columns);
 #define DSX_KNN_PATH_CANDIDATES 1         /* first block as above, then candidate lists */
 #define DSX_KNN_PATH_CANDIDATES_REDONE 2  /* a candidate list filled up: repeated block by block */
 int dsx_knn_last_search_path(void);
+/* No counterpart in the reference: how dsx_knn_search_f16 scores the column ranges after the first block.  1 (default): a
+ * range with enough item tiles is swept by workgroups that keep their queries and walk a chunk of the range each (private
+ * candidate lists, no atomics on device memory); 0: always one workgroup per tile; 2: sweep every range that has at least one
+ * tile per chunk (for tests at small sizes).  The results are the same in every mode. */
+int dsx_knn_f16_set_sweep(int mode);
 
 #ifdef __cplusplus
 }

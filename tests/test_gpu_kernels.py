@@ -723,17 +723,23 @@ def knn_case_f16(pkg, dsx, orc, items_m, queries_m, k):
     return scores.numpy(), idx.numpy(), ref_s, ref_i, it16, q16, table
 
 
+# sweep 0: one workgroup per tile of scores; 2: column ranges with at least a tile per chunk go through knn_f16_sweep_kernel
+# (with these few queries that is 64 chunks per row tile, so ranges from 8,192 columns on)
+@pytest.mark.parametrize("sweep", [0, 2])
 @pytest.mark.parametrize("items,queries,dim,k,blocks", [(1003, 9, 24, 10, 0), (50000, 64, 256, 100, 0), (30011, 70, 64, 100, 1024),
-                                                          (9000, 130, 250, 10, 1024), (26000, 33, 32, 200, 1024)])
-def test_knn_search_f16(pkg, dsx, orc, synth, items, queries, dim, k, blocks):
-    say("knn fp16 items=%d queries=%d dim=%d k=%d first block=%d" % (items, queries, dim, k, blocks))
+                                                          (9000, 130, 250, 10, 1024), (26000, 33, 32, 200, 1024),
+                                                          (70001, 300, 100, 100, 2048)])
+def test_knn_search_f16(pkg, dsx, orc, synth, items, queries, dim, k, blocks, sweep):
+    say("knn fp16 items=%d queries=%d dim=%d k=%d first block=%d sweep=%d" % (items, queries, dim, k, blocks, sweep))
     p = synth.knn_config(seed=21, items=items, queries=queries, dim=dim, k=k)
     dsx.dsx_knn_set_block_columns(blocks)
+    pkg.check(dsx.dsx_knn_f16_set_sweep(sweep))
     try:
         got_s, got_i, ref_s, ref_i, it16, q16, _ = knn_case_f16(pkg, dsx, orc, p.items, p.queries, k)
         assert dsx.dsx_knn_last_search_path() == (1 if blocks else 0)
     finally:
         dsx.dsx_knn_set_block_columns(0)
+        pkg.check(dsx.dsx_knn_f16_set_sweep(1))
     full = q16.astype(np.float64) @ it16.astype(np.float64).T
     assert got_i.max() < items
     mism = got_i != ref_i
@@ -742,6 +748,32 @@ def test_knn_search_f16(pkg, dsx, orc, synth, items, queries, dim, k, blocks):
         assert np.abs(full[r, got_i[r, c]] - full[r, ref_i[r, c]]).max() < 1e-5
     assert_close(got_s, np.take_along_axis(full, got_i.astype(np.int64), axis=1), "knn fp16 scores", rel=1e-4, abs_floor=0.05)
     assert (np.diff(got_s, axis=1) <= 0).all()
+
+
+def test_knn_search_f16_sweep_spills_clustered_items(pkg, dsx, orc, rng):
+    """300 neighbouring items that all beat a query's bound land in two or three chunks of a sweep, whose lists hold 64 words
+    each: the rest goes to the query's shared list, nothing is lost and the search is not redone."""
+    items, queries, dim, k = 40000, 70, 64, 100
+    it = rng.standard_normal((items, dim)).astype(np.float32)
+    q = rng.standard_normal((queries, dim)).astype(np.float32)
+    u = q[5] / np.linalg.norm(q[5])
+    for j in range(300):
+        it[21000 + j] = u * (40.0 + 0.25 * j)   # far above anything else for query 5, all different
+    dsx.dsx_knn_set_block_columns(1024)
+    pkg.check(dsx.dsx_knn_f16_set_sweep(2))
+    try:
+        got_s, got_i, ref_s, ref_i, it16, q16, _ = knn_case_f16(pkg, dsx, orc, it, q, k)
+        assert dsx.dsx_knn_last_search_path() == 1
+    finally:
+        dsx.dsx_knn_set_block_columns(0)
+        pkg.check(dsx.dsx_knn_f16_set_sweep(1))
+    assert set(got_i[5]) <= set(range(21000, 21300))
+    full = q16.astype(np.float64) @ it16.astype(np.float64).T
+    mism = got_i != ref_i
+    if mism.any():
+        r, c = np.nonzero(mism)
+        assert np.abs(full[r, got_i[r, c]] - full[r, ref_i[r, c]]).max() < 1e-5
+    assert_close(got_s, np.take_along_axis(full, got_i.astype(np.int64), axis=1), "knn fp16 scores", rel=1e-4, abs_floor=0.05)
 
 
 def test_knn_f16_table_layout_and_rounding(pkg, dsx, rng):
@@ -761,12 +793,15 @@ def test_knn_f16_table_layout_and_rounding(pkg, dsx, rng):
     assert (t[items:] == 0).all() and (t[:, dim:] == 0).all()
 
 
-def test_knn_search_f16_exact_ties_and_full_lists(pkg, dsx, orc, rng):
-    """Small integers are exact in fp16 too: bit-identical to the oracle, including the query whose candidates all tie."""
+@pytest.mark.parametrize("sweep", [0, 2])
+def test_knn_search_f16_exact_ties_and_full_lists(pkg, dsx, orc, rng, sweep):
+    """Small integers are exact in fp16 too: bit-identical to the oracle, including the query whose candidates all tie (with
+    the sweep: its 64-word lists per chunk fill up and spill into the shared list, which fills up as well)."""
     items, queries, dim, k = 21000, 40, 16, 100
     it = rng.integers(-2, 3, size=(items, dim)).astype(np.float32)
     q = rng.integers(-2, 3, size=(queries, dim)).astype(np.float32)
     dsx.dsx_knn_set_block_columns(1024)
+    pkg.check(dsx.dsx_knn_f16_set_sweep(sweep))
     try:
         got_s, got_i, ref_s, ref_i, _, _, _ = knn_case_f16(pkg, dsx, orc, it, q, k)
         assert dsx.dsx_knn_last_search_path() == 1
@@ -777,3 +812,4 @@ def test_knn_search_f16_exact_ties_and_full_lists(pkg, dsx, orc, rng):
         assert np.array_equal(got_s, ref_s) and np.array_equal(got_i, ref_i)
     finally:
         dsx.dsx_knn_set_block_columns(0)
+        pkg.check(dsx.dsx_knn_f16_set_sweep(1))
