@@ -125,10 +125,9 @@ int knn_f16_scores_run(const void* queries16, const void* items16, uint32_t ld, 
                        const CandArgs* cand);
 int knn_refresh(uint64_t* best, const uint64_t* cand, uint32_t* cand_count, uint32_t cap, uint32_t k, uint32_t* row_bound, uint32_t batch,
                 const uint64_t* seg = nullptr, uint32_t* seg_count = nullptr, uint32_t chunks = 0, uint32_t seg_cap = 0);
-// fp16 storage, long column ranges: every workgroup sweeps a chunk of the range and keeps (row, chunk) lists of its own
-// (seg [queries][chunks][seg_cap], seg_count [queries][64]); full lists spill into cand's shared ones.
-uint32_t knn_f16_sweep_chunks(uint32_t batch);
-bool knn_f16_sweep_applies(uint32_t batch, uint32_t n);
-int knn_f16_sweep_run(const void* queries16, const void* items16, uint32_t ld, uint32_t batch, uint32_t n, const CandArgs& cand, uint64_t* seg,
-                      uint32_t* seg_count, uint32_t seg_cap);
+// fp16 storage, candidate mode of a column range: one workgroup per tile, or (long ranges) workgroups that sweep a chunk of the
+// range each and keep (row, chunk) lists of their own (seg [queries][chunks][seg_words / chunks], seg_count [queries][64]); full
+// lists spill into cand's shared ones.  mode: see dsx_knn_f16_set_sweep.  *chunks_used is what knn_refresh needs to know.
+int knn_f16_candidates_run(const void* queries16, const void* items16, uint32_t ld, uint32_t batch, uint32_t n, const CandArgs& cand,
+                           uint64_t* seg, uint32_t* seg_count, uint32_t seg_words, int mode, uint32_t* chunks_used);
 }  // namespace dsx

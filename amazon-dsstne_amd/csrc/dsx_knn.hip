@@ -22,7 +22,7 @@ static LibScratch g_knn_ws_of[2];   // per lane
 
 static uint32_t g_knn_block_columns = 0;   // 0: sized by the rule below
 static int g_knn_last_path = 0;            // how the last search ran: DSX_KNN_PATH_*
-static int g_knn_f16_sweep = 1;            // fp16 storage: 0 never sweeps, 1 sweeps long column ranges (knn_f16_sweep_kernel), 2 every range it can
+static int g_knn_f16_sweep = 1;            // fp16 storage, see dsx_knn_f16_set_sweep
 
 static uint32_t knn_block_columns(uint32_t rows_padded, uint32_t num_queries)
 {
@@ -102,14 +102,14 @@ struct KnnOperands {
         if (f16) return knn_f16_scores_run(queries16, items16 + (uint64_t)c0 * ld16 * 2, ld16, num_queries, ncols, Z, ldz, nullptr);
         return fc_run(queries, dim, items + c0, rows_padded, 0, nullptr, Z, ldz, num_queries, dim, ncols, 0, DSX_ACT_LINEAR, nullptr);
     }
-    int into_candidates(uint32_t c0, uint32_t ncols, uint32_t num_queries, const CandArgs& cand, uint64_t* seg, uint32_t* seg_count) const
+    // *chunks_used: how many (row, chunk) lists of seg the range filled besides the shared lists (0: none)
+    int into_candidates(uint32_t c0, uint32_t ncols, uint32_t num_queries, const CandArgs& cand, uint64_t* seg, uint32_t* seg_count,
+                        uint32_t* chunks_used) const
     {
-        const bool sweep = g_knn_f16_sweep == 2 ? (ncols + 127) / 128 >= knn_f16_sweep_chunks(num_queries)
-                                                : (g_knn_f16_sweep == 1 && knn_f16_sweep_applies(num_queries, ncols));
-        if (f16 && seg && sweep)
-            return knn_f16_sweep_run(queries16, items16 + (uint64_t)c0 * ld16 * 2, ld16, num_queries, ncols, cand, seg, seg_count,
-                                     kCandCap / knn_f16_sweep_chunks(num_queries));
-        if (f16) return knn_f16_scores_run(queries16, items16 + (uint64_t)c0 * ld16 * 2, ld16, num_queries, ncols, nullptr, 0, &cand);
+        *chunks_used = 0;
+        if (f16)
+            return knn_f16_candidates_run(queries16, items16 + (uint64_t)c0 * ld16 * 2, ld16, num_queries, ncols, cand, seg, seg_count, kCandCap,
+                                          g_knn_f16_sweep, chunks_used);
         return fc_candidates_run(queries, dim, items + c0, rows_padded, num_queries, dim, ncols, cand);
     }
 };
@@ -166,7 +166,6 @@ static int knn_search_candidates(const KnnWorkspace& w, const KnnOperands& op, u
     const uint32_t clear_words = 2 * num_queries + 64;
     hipLaunchKernelGGL(knn_clear_kernel, dim3((clear_words + 255) / 256), dim3(256), 0, s, w.row_bound, clear_words);
     if (w.seg_count) hipLaunchKernelGGL(knn_clear_kernel, dim3((num_queries * 64 + 255) / 256), dim3(256), 0, s, w.seg_count, num_queries * 64);
-    const uint32_t chunks = w.seg ? knn_f16_sweep_chunks(num_queries) : 0;
     uint32_t done = std::min(cb, M);
     t.start(s);
     int rc = op.into_matrix(0, done, num_queries, w.block_scores, cb);
@@ -182,11 +181,12 @@ static int knn_search_candidates(const KnnWorkspace& w, const KnnOperands& op, u
         const uint32_t ncols = (uint32_t)std::min<uint64_t>((uint64_t)M - done, (uint64_t)done * 4 / 128 * 128);
         t.start(s);
         const CandArgs cand{w.row_bound, w.cand, w.cand_count, kCandCap, done, w.overflow};
-        rc = op.into_candidates(done, ncols, num_queries, cand, w.seg, w.seg_count);
+        uint32_t chunks = 0;
+        rc = op.into_candidates(done, ncols, num_queries, cand, w.seg, w.seg_count, &chunks);
         if (rc) return rc;
         t.stop(s, t.gemm);
         t.start(s);
-        rc = knn_refresh(w.partial, w.cand, w.cand_count, kCandCap, k, w.row_bound, num_queries, w.seg, w.seg_count, chunks,
+        rc = knn_refresh(w.partial, w.cand, w.cand_count, kCandCap, k, w.row_bound, num_queries, chunks ? w.seg : nullptr, w.seg_count, chunks,
                          chunks ? kCandCap / chunks : 0);
         if (rc) return rc;
         t.stop(s, t.topk);

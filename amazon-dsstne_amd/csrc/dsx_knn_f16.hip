@@ -9,6 +9,7 @@
 // 32 components of both operands per step are staged in LDS (double buffered, rows padded to 80 bytes so that the 128-bit
 // reads of 8 lanes cover all banks once).  Products of fp16 values are exact in fp32 and the sums are fp32, as in the
 // reference's GEMM.  Epilogues: plain store (first column block) or candidate lists (everything after it).
+#include <algorithm>
 #include "dsx_device.h"
 #include "dsx_internal.h"
 
@@ -418,45 +419,38 @@ int knn_f16_scores_run(const void* queries16, const void* items16, uint32_t ld, 
     return DSX_OK;
 }
 
-// Chunks per row tile for a search of `batch` queries: enough workgroups to fill every CU four times, at most 64.
-uint32_t knn_f16_sweep_chunks(uint32_t batch)
+// Candidate mode of a column range of n items for `batch` queries.  mode 0: one workgroup per tile (knn_f16_kernel); 1: a
+// sweep (knn_f16_sweep_kernel) when it has workgroups for every CU and at least four tiles per chunk; 2: a sweep whenever every
+// chunk gets a tile (tests at small sizes).  *chunks_used: the chunks of the sweep, 0 when the range went through
+// knn_f16_kernel and only the shared lists were appended to.
+int knn_f16_candidates_run(const void* queries16, const void* items16, uint32_t ld, uint32_t batch, uint32_t n, const CandArgs& cand,
+                           uint64_t* seg, uint32_t* seg_count, uint32_t seg_words, int mode, uint32_t* chunks_used)
 {
-    const uint32_t tiles_m = (batch + 127) / 128;
-    const uint32_t want = 4 * (uint32_t)ctx().num_cus;
-    uint32_t chunks = (want + tiles_m - 1) / tiles_m;
-    if (chunks > kSweepCountStride) chunks = kSweepCountStride;
-    return chunks;
-}
-
-// Whether a range of n columns is worth a sweep: workgroups for every CU, and at least four tiles in every chunk.
-bool knn_f16_sweep_applies(uint32_t batch, uint32_t n)
-{
+    *chunks_used = 0;
+    const uint32_t cus = (uint32_t)ctx().num_cus;
     const uint32_t tiles_m = (batch + 127) / 128, tiles_n = (n + 127) / 128;
-    const uint32_t chunks = knn_f16_sweep_chunks(batch);
-    return tiles_m * chunks >= 2 * (uint32_t)ctx().num_cus && tiles_n >= 4 * chunks;
-}
-
-int knn_f16_sweep_run(const void* queries16, const void* items16, uint32_t ld, uint32_t batch, uint32_t n, const CandArgs& cand, uint64_t* seg,
-                      uint32_t* seg_count, uint32_t seg_cap)
-{
+    const uint32_t chunks = std::min<uint32_t>(kSweepCountStride, (4 * cus + tiles_m - 1) / tiles_m);   // every CU four times over
+    const bool sweep = seg && seg_count && (mode == 2 ? tiles_n >= chunks : (mode == 1 && tiles_m * chunks >= 2 * cus && tiles_n >= 4 * chunks));
+    if (!sweep) return knn_f16_scores_run(queries16, items16, ld, batch, n, nullptr, 0, &cand);
     KnnF16SweepArgs a{};
     a.A = (const _Float16*)queries16;
     a.B = (const _Float16*)items16;
     a.ld = ld;
     a.batch = batch;
     a.n = n;
-    a.tiles_m = (batch + 127) / 128;
-    a.tiles_n = (n + 127) / 128;
-    a.chunks = knn_f16_sweep_chunks(batch);
-    a.tiles_per_chunk = (a.tiles_n + a.chunks - 1) / a.chunks;
+    a.tiles_m = tiles_m;
+    a.tiles_n = tiles_n;
+    a.chunks = chunks;
+    a.tiles_per_chunk = (tiles_n + chunks - 1) / chunks;
     a.seg = seg;
     a.seg_count = seg_count;
-    a.seg_cap = seg_cap;
+    a.seg_cap = seg_words / chunks;
     a.cand = cand;
     const uint32_t total = a.tiles_m * a.chunks;
     const uint32_t grid = ((total + kF16Xcds - 1) / kF16Xcds) * kF16Xcds;
     hipLaunchKernelGGL(knn_f16_sweep_kernel, dim3(grid), dim3(256), 0, ctx().stream, a);
     DSX_LAUNCH_CHECK("knn_f16_sweep_kernel");
+    *chunks_used = chunks;
     return DSX_OK;
 }
 

@@ -728,7 +728,7 @@ def knn_case_f16(pkg, dsx, orc, items_m, queries_m, k):
 @pytest.mark.parametrize("sweep", [0, 2])
 @pytest.mark.parametrize("items,queries,dim,k,blocks", [(1003, 9, 24, 10, 0), (50000, 64, 256, 100, 0), (30011, 70, 64, 100, 1024),
                                                           (9000, 130, 250, 10, 1024), (26000, 33, 32, 200, 1024),
-                                                          (70001, 300, 100, 100, 2048)])
+                                                          (70001, 300, 100, 100, 2048), (60000, 520, 256, 50, 2048)])
 def test_knn_search_f16(pkg, dsx, orc, synth, items, queries, dim, k, blocks, sweep):
     say("knn fp16 items=%d queries=%d dim=%d k=%d first block=%d sweep=%d" % (items, queries, dim, k, blocks, sweep))
     p = synth.knn_config(seed=21, items=items, queries=queries, dim=dim, k=k)
@@ -750,10 +750,11 @@ def test_knn_search_f16(pkg, dsx, orc, synth, items, queries, dim, k, blocks, sw
     assert (np.diff(got_s, axis=1) <= 0).all()
 
 
-def test_knn_search_f16_sweep_spills_clustered_items(pkg, dsx, orc, rng):
+@pytest.mark.parametrize("dim", [64, 128])
+def test_knn_search_f16_sweep_spills_clustered_items(pkg, dsx, orc, rng, dim):
     """300 neighbouring items that all beat a query's bound land in two or three chunks of a sweep, whose lists hold 64 words
     each: the rest goes to the query's shared list, nothing is lost and the search is not redone."""
-    items, queries, dim, k = 40000, 70, 64, 100
+    items, queries, k = 40000, 70, 100
     it = rng.standard_normal((items, dim)).astype(np.float32)
     q = rng.standard_normal((queries, dim)).astype(np.float32)
     u = q[5] / np.linalg.norm(q[5])
@@ -793,11 +794,11 @@ def test_knn_f16_table_layout_and_rounding(pkg, dsx, rng):
     assert (t[items:] == 0).all() and (t[:, dim:] == 0).all()
 
 
-@pytest.mark.parametrize("sweep", [0, 2])
-def test_knn_search_f16_exact_ties_and_full_lists(pkg, dsx, orc, rng, sweep):
+@pytest.mark.parametrize("sweep,dim", [(0, 16), (2, 16), (2, 128)])
+def test_knn_search_f16_exact_ties_and_full_lists(pkg, dsx, orc, rng, sweep, dim):
     """Small integers are exact in fp16 too: bit-identical to the oracle, including the query whose candidates all tie (with
     the sweep: its 64-word lists per chunk fill up and spill into the shared list, which fills up as well)."""
-    items, queries, dim, k = 21000, 40, 16, 100
+    items, queries, k = 21000, 40, 100
     it = rng.integers(-2, 3, size=(items, dim)).astype(np.float32)
     q = rng.integers(-2, 3, size=(queries, dim)).astype(np.float32)
     dsx.dsx_knn_set_block_columns(1024)
