@@ -508,6 +508,33 @@ def test_topk_guided_filtered(pkg, dsx, orc, rng, batch, width, k, maxnnz, with_
     assert_topk_exact(keys, idx, sk, si)
 
 
+@pytest.mark.parametrize("batch,width,k,share", [(64, 27278, 10, 0.13), (64, 27278, 10, 0.004), (16, 27278, 50, 0.4), (3, 300000, 10, 0.13),
+                                                  (9, 27278, 100, 0.13), (5, 70000, 200, 0.05)])
+@pytest.mark.parametrize("filtered", [False, True])
+def test_topk_saturated_rows_scan_and_guided(pkg, dsx, orc, rng, batch, width, k, share, filtered):
+    """Saturated sigmoids: a share of every row is exactly 1.0, the top of the list is ties all the way down and the lowest
+    columns win.  Some of the tied columns are listed in the filter (their zero must not displace anything), one row has
+    fewer than k ones, one has a value above 1.0 late in the row.  Wide rows are split over several workgroups."""
+    say("topk saturated batch=%d width=%d k=%d share=%g filtered=%s" % (batch, width, k, share, filtered))
+    scores = (rng.random((batch, width), dtype=np.float32) * np.float32(0.999)).astype(np.float32)
+    scores[rng.random((batch, width)) < share] = 1.0
+    scores[1, :] = rng.random(width, dtype=np.float32) * np.float32(0.5)
+    scores[1, rng.choice(width, size=max(1, k // 2), replace=False)] = 1.0     # fewer than k ones
+    scores[2, width - 5] = 1.5                                                   # the best score comes last
+    start = end = fidx = None
+    if filtered:
+        start, end, fidx = random_csr(rng, batch, width, 400, empty_rows=(0,))
+    if filtered:
+        keys, idx = run_filtered(pkg, dsx, scores, k, 0, None, start, end, fidx, None)
+        rk, ri = orc.topk_filtered(scores, k, 0, None, start, end, fidx, None)
+    else:
+        keys, idx = run_topk(pkg, dsx, scores, k)
+        rk, ri = orc.topk(scores, k)
+    assert_topk_exact(keys, idx, rk, ri)
+    gk, gi = run_guided(pkg, dsx, scores, k, segment_maxima(scores), 0, None, start, end, fidx, None)
+    assert_topk_exact(gk, gi, rk, ri)
+
+
 def test_topk_guided_indexed_filter_and_position(pkg, dsx, orc, rng):
     rows, batch, width, k, position = 40, 17, 3000, 20, 9
     scores = rng.random((batch, width), dtype=np.float32)
