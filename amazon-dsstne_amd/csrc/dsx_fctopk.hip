@@ -19,7 +19,7 @@ namespace dsx {
 constexpr uint32_t kLayerCandCap = 4096;       // candidate words per row and column range
 static uint32_t g_layer_first_columns = 0;     // 0: default
 static uint32_t g_layer_cap = kLayerCandCap;   // tests lower it to reach the overflow path with small inputs
-static LibScratch g_layer_ws_of[2];            // per lane
+static LibScratch g_layer_ws_of[DSX_MAX_LANES];   // per lane
 static uint32_t* g_layer_flagged = nullptr;    // pinned host memory: the device stores 1 there when it flags a row
 
 __global__ __launch_bounds__(256) void layer_clear_kernel(uint32_t* p, uint32_t n)

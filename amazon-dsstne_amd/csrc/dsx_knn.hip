@@ -18,7 +18,7 @@
 
 namespace dsx {
 
-static LibScratch g_knn_ws_of[2];   // per lane
+static LibScratch g_knn_ws_of[DSX_MAX_LANES];   // per lane
 
 static uint32_t g_knn_block_columns = 0;   // 0: sized by the rule below
 static int g_knn_last_path = 0;            // how the last search ran: DSX_KNN_PATH_*

@@ -74,12 +74,12 @@ using namespace dsx;
 // (four uploads, engine/NNTypes.cpp:583-778) then cost four host copies instead of four round trips.  Consecutive uploads
 // share a slot until it is full (a batch of config 2 is 0.6 MB: the ring holds some fifty batches, so a caller that streams
 // batches is never held up by the ring while the device is several batches behind); a slot is reused only after the copies
-// out of it have finished on both lanes.
+// out of it have finished on every lane.
 constexpr int kUploadSlots = 8;
 constexpr size_t kUploadSlotBytes = (size_t)4 << 20;
 static char* g_upload_host[kUploadSlots] = {};
-static hipEvent_t g_upload_done[kUploadSlots][2] = {};   // [slot][lane]: after the slot's last copy on that lane
-static bool g_upload_busy[kUploadSlots][2] = {};
+static hipEvent_t g_upload_done[kUploadSlots][DSX_MAX_LANES] = {};   // [slot][lane]: after the slot's last copy on that lane
+static bool g_upload_busy[kUploadSlots][DSX_MAX_LANES] = {};
 static int g_upload_slot = 0;       // slot being filled
 static size_t g_upload_fill = 0;    // bytes of it handed out
 
@@ -102,7 +102,7 @@ static void upload_ring_release()
     for (int i = 0; i < kUploadSlots; i++) {
         if (g_upload_host[i]) hipHostFree(g_upload_host[i]);
         g_upload_host[i] = nullptr;
-        for (int l = 0; l < 2; l++) {
+        for (int l = 0; l < DSX_MAX_LANES; l++) {
             if (g_upload_done[i][l]) hipEventDestroy(g_upload_done[i][l]);
             g_upload_done[i][l] = nullptr;
             g_upload_busy[i][l] = false;
@@ -113,61 +113,76 @@ static void upload_ring_release()
 }
 
 
-// Two lanes: independent in-order streams, so that the kernels of two batches can be in flight together (one batch's top-K
-// and input layers fill the gaps of the other's GEMM).  ctx().stream is always the selected lane's stream; everything the
-// library launches goes there.  Operations whose effect both lanes must see in order — uploads, clears, device copies,
-// allocation fills, timers — join the lanes around themselves; downloads and dsx_sync wait for both.
-static hipStream_t g_lane_stream[2] = {nullptr, nullptr};
-static hipEvent_t g_lane_event[2] = {nullptr, nullptr};   // [l]: last join point recorded on lane l
+// Lanes: up to DSX_MAX_LANES independent in-order streams, so that the kernels of several batches can be in flight together
+// (one batch's top-K and input layers fill the gaps of another's GEMM).  ctx().stream is always the selected lane's stream;
+// everything the library launches goes there.  Operations whose effect every lane must see in order — uploads, clears,
+// device copies, allocation fills, timers — join the lanes around themselves; downloads and dsx_sync wait for all of them.
+// A lane's stream is made when the lane is first selected; lane 0 is the context's own stream.
+static hipStream_t g_lane_stream[DSX_MAX_LANES] = {};
+static hipEvent_t g_lane_event[DSX_MAX_LANES] = {};   // [l]: last join point recorded on lane l
 static int g_lane = 0;
 
 namespace dsx {
 int current_lane() { return g_lane; }
 }  // namespace dsx
 
-static hipStream_t other_lane_stream() { return g_lane_stream[g_lane ^ 1]; }
+static bool lanes_in_use() { return g_lane_stream[0] != nullptr; }
 
-// Work can only be queued on a lane while it is selected, so "the other lane has been selected since this lane last waited
-// for it" is all that has to be tracked: a burst of uploads between two batches then costs one cross-stream wait, not one
-// per call (each is an event record, a wait and a barrier packet between two hardware queues).
-static uint32_t g_lane_selected[2] = {1, 0};   // how often each lane has been selected
-static uint32_t g_lane_seen[2] = {0, 0};       // [l]: g_lane_selected[other] when lane l last waited for the other lane
-static bool g_lane_publish[2] = {false, false};   // [l]: lane l holds ordered work the other lane has not been told to wait for
+// Work can only be queued on a lane while it is selected, so "lane o has been selected since lane l last waited for it" is
+// all that has to be tracked: a burst of uploads between two batches then costs one cross-stream wait per lane, not one per
+// call (each is an event record, a wait and a barrier packet between two hardware queues).
+static uint32_t g_lane_selected[DSX_MAX_LANES] = {1, 0};                 // how often each lane has been selected
+static uint32_t g_lane_seen[DSX_MAX_LANES][DSX_MAX_LANES] = {};         // [l][o]: g_lane_selected[o] when lane l last waited for lane o
+static bool g_lane_publish[DSX_MAX_LANES][DSX_MAX_LANES] = {};          // [l][o]: lane l holds ordered work lane o has not been told to wait for
 
-// The selected lane waits for everything queued so far on the other one.
+// Lane `waiter` waits for everything queued so far on lane o.
+static int lane_wait_for(int waiter, int o)
+{
+    DSX_HIP(hipEventRecord(g_lane_event[o], g_lane_stream[o]));
+    DSX_HIP(hipStreamWaitEvent(g_lane_stream[waiter], g_lane_event[o], 0));
+    g_lane_seen[waiter][o] = g_lane_selected[o];
+    g_lane_publish[o][waiter] = false;
+    return DSX_OK;
+}
+
+// The selected lane waits for everything queued so far on the other ones.
 static int lanes_join_before()
 {
-    hipStream_t other = other_lane_stream();
-    if (!other) return DSX_OK;
-    const int o = g_lane ^ 1;
-    if (g_lane_seen[g_lane] != g_lane_selected[o]) {
-        DSX_HIP(hipEventRecord(g_lane_event[o], other));
-        DSX_HIP(hipStreamWaitEvent(ctx().stream, g_lane_event[o], 0));
-        g_lane_seen[g_lane] = g_lane_selected[o];
+    if (!lanes_in_use()) return DSX_OK;
+    for (int o = 0; o < DSX_MAX_LANES; o++) {
+        if (o == g_lane || !g_lane_stream[o]) continue;
+        if (g_lane_seen[g_lane][o] != g_lane_selected[o] || g_lane_publish[o][g_lane])
+            if (int rc = lane_wait_for(g_lane, o)) return rc;
     }
     return DSX_OK;
 }
 
-// The other lane must wait for what was just queued on the selected one: arranged when the other lane is selected next.
+// The other lanes must wait for what was just queued on the selected one: arranged when one of them is selected next.
 static int lanes_join_after()
 {
-    if (other_lane_stream()) g_lane_publish[g_lane] = true;
+    if (!lanes_in_use()) return DSX_OK;
+    for (int o = 0; o < DSX_MAX_LANES; o++)
+        if (o != g_lane) g_lane_publish[g_lane][o] = true;   // (also for lanes that do not exist yet: they start after everything anyway)
     return DSX_OK;
 }
 
 static void lanes_release()
 {
     // lane 0's stream is ctx().stream's original and is destroyed with the context
-    if (g_lane_stream[1]) hipStreamDestroy(g_lane_stream[1]);
+    for (int l = 1; l < DSX_MAX_LANES; l++)
+        if (g_lane_stream[l]) hipStreamDestroy(g_lane_stream[l]);
     for (auto& e : g_lane_event)
         if (e) hipEventDestroy(e);
-    g_lane_stream[0] = g_lane_stream[1] = nullptr;
-    g_lane_event[0] = g_lane_event[1] = nullptr;
+    for (int l = 0; l < DSX_MAX_LANES; l++) {
+        g_lane_stream[l] = nullptr;
+        g_lane_event[l] = nullptr;
+        g_lane_selected[l] = (l == 0) ? 1 : 0;
+        for (int o = 0; o < DSX_MAX_LANES; o++) {
+            g_lane_seen[l][o] = 0;
+            g_lane_publish[l][o] = false;
+        }
+    }
     g_lane = 0;
-    g_lane_selected[0] = 1;
-    g_lane_selected[1] = 0;
-    g_lane_seen[0] = g_lane_seen[1] = 0;
-    g_lane_publish[0] = g_lane_publish[1] = false;
 }
 
 extern "C" {
@@ -211,7 +226,8 @@ int dsx_shutdown(void)
     Context& c = ctx();
     if (!c.initialized) return DSX_OK;
     if (--c.users > 0) return DSX_OK;
-    if (g_lane_stream[1]) hipStreamSynchronize(g_lane_stream[1]);
+    for (int l = 1; l < DSX_MAX_LANES; l++)
+        if (g_lane_stream[l]) hipStreamSynchronize(g_lane_stream[l]);
     if (g_lane_stream[0]) c.stream = g_lane_stream[0];
     hipStreamSynchronize(c.stream);
     lanes_release();
@@ -265,24 +281,25 @@ void* dsx_stream(void) { return (void*)ctx().stream; }
 int dsx_set_lane(int lane)
 {
     DSX_REQUIRE_INIT();
-    DSX_CHECK_ARG(lane == 0 || lane == 1, "dsx_set_lane: lane %d (0 or 1)", lane);
-    if (!g_lane_stream[0]) {
-        if (lane == 0) return DSX_OK;   // nothing to set up until the second lane is asked for
+    DSX_CHECK_ARG(lane >= 0 && lane < DSX_MAX_LANES, "dsx_set_lane: lane %d (0..%d)", lane, DSX_MAX_LANES - 1);
+    if (!lanes_in_use()) {
+        if (lane == 0) return DSX_OK;   // nothing to set up until another lane is asked for
         g_lane_stream[0] = ctx().stream;
-        DSX_HIP(hipStreamCreateWithFlags(&g_lane_stream[1], hipStreamNonBlocking));
-        for (auto& e : g_lane_event) DSX_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
-        // the new lane starts after everything queued so far
-        DSX_HIP(hipEventRecord(g_lane_event[0], g_lane_stream[0]));
-        DSX_HIP(hipStreamWaitEvent(g_lane_stream[1], g_lane_event[0], 0));
+        DSX_HIP(hipEventCreateWithFlags(&g_lane_event[0], hipEventDisableTiming));
+    }
+    if (!g_lane_stream[lane]) {
+        DSX_HIP(hipStreamCreateWithFlags(&g_lane_stream[lane], hipStreamNonBlocking));
+        DSX_HIP(hipEventCreateWithFlags(&g_lane_event[lane], hipEventDisableTiming));
+        // the new lane starts after everything queued so far on the others
+        for (int o = 0; o < DSX_MAX_LANES; o++)
+            if (o != lane && g_lane_stream[o])
+                if (int rc = lane_wait_for(lane, o)) return rc;
     }
     if (lane != g_lane) {
-        const int old = g_lane;
-        if (g_lane_publish[old]) {   // ordered work (uploads, clears, copies) of the lane being left: the new lane runs after it
-            DSX_HIP(hipEventRecord(g_lane_event[old], g_lane_stream[old]));
-            DSX_HIP(hipStreamWaitEvent(g_lane_stream[lane], g_lane_event[old], 0));
-            g_lane_publish[old] = false;
-            g_lane_seen[lane] = g_lane_selected[old];
-        }
+        // ordered work (uploads, clears, copies) of the lanes that published some: the new lane runs after it
+        for (int o = 0; o < DSX_MAX_LANES; o++)
+            if (o != lane && g_lane_stream[o] && g_lane_publish[o][lane])
+                if (int rc = lane_wait_for(lane, o)) return rc;
         g_lane = lane;
         g_lane_selected[lane]++;
         ctx().stream = g_lane_stream[lane];
@@ -387,7 +404,7 @@ static int upload_on_selected_lane(void* dst, const void* src, size_t bytes)
     if (g_upload_fill + bytes > kUploadSlotBytes) {   // on to the next slot, once nothing is being copied out of it any more
         g_upload_slot = (g_upload_slot + 1) % kUploadSlots;
         g_upload_fill = 0;
-        for (int l = 0; l < 2; l++)
+        for (int l = 0; l < DSX_MAX_LANES; l++)
             if (g_upload_busy[g_upload_slot][l]) {
                 DSX_HIP(hipEventSynchronize(g_upload_done[g_upload_slot][l]));
                 g_upload_busy[g_upload_slot][l] = false;
@@ -396,7 +413,7 @@ static int upload_on_selected_lane(void* dst, const void* src, size_t bytes)
     const int slot = g_upload_slot;
     if (!g_upload_host[slot]) {
         DSX_HIP(hipHostMalloc((void**)&g_upload_host[slot], kUploadSlotBytes, hipHostMallocDefault));
-        for (int l = 0; l < 2; l++) DSX_HIP(hipEventCreateWithFlags(&g_upload_done[slot][l], hipEventDisableTiming));
+        for (int l = 0; l < DSX_MAX_LANES; l++) DSX_HIP(hipEventCreateWithFlags(&g_upload_done[slot][l], hipEventDisableTiming));
     }
     char* staged = g_upload_host[slot] + g_upload_fill;
     g_upload_fill += (bytes + 255) / 256 * 256;
@@ -429,12 +446,18 @@ int dsx_memcpy_h2d_unordered(void* dst, const void* src, size_t bytes)
 int dsx_lane_wait_other(void)
 {
     DSX_REQUIRE_INIT();
-    hipStream_t other = other_lane_stream();
-    if (!other) return DSX_OK;
-    const int o = g_lane ^ 1;
-    DSX_HIP(hipEventRecord(g_lane_event[o], other));
-    DSX_HIP(hipStreamWaitEvent(ctx().stream, g_lane_event[o], 0));
-    g_lane_seen[g_lane] = g_lane_selected[o];
+    if (!lanes_in_use()) return DSX_OK;
+    for (int o = 0; o < DSX_MAX_LANES; o++)
+        if (o != g_lane && g_lane_stream[o])
+            if (int rc = lane_wait_for(g_lane, o)) return rc;
+    return DSX_OK;
+}
+
+// Host-side wait for every lane but the selected one.
+static int sync_other_lanes()
+{
+    for (int o = 0; o < DSX_MAX_LANES; o++)
+        if (o != g_lane && g_lane_stream[o]) DSX_HIP(hipStreamSynchronize(g_lane_stream[o]));
     return DSX_OK;
 }
 
@@ -443,7 +466,7 @@ int dsx_memcpy_d2h(void* dst, const void* src, size_t bytes)
     DSX_REQUIRE_INIT();
     if (bytes == 0) return DSX_OK;
     DSX_CHECK_ARG(dst && src, "dsx_memcpy_d2h: null pointer");
-    if (other_lane_stream()) DSX_HIP(hipStreamSynchronize(other_lane_stream()));   // the data may come from either lane
+    if (int rc = sync_other_lanes()) return rc;   // the data may come from any lane
     if (bytes <= kUploadSlotBytes) {
         std::lock_guard<std::mutex> lock(g_alloc_mutex);
         if (int rc = download_small(dst, src, bytes, ctx().stream, 0)) return rc;
@@ -461,7 +484,7 @@ int dsx_memcpy_d2h_pair(void* dst0, const void* src0, size_t bytes0, void* dst1,
 {
     DSX_REQUIRE_INIT();
     DSX_CHECK_ARG((bytes0 == 0 || (dst0 && src0)) && (bytes1 == 0 || (dst1 && src1)), "dsx_memcpy_d2h_pair: null pointer");
-    if (other_lane_stream()) DSX_HIP(hipStreamSynchronize(other_lane_stream()));   // the data may come from either lane
+    if (int rc = sync_other_lanes()) return rc;   // the data may come from any lane
     const size_t off1 = (bytes0 + 255) / 256 * 256;
     if (off1 + bytes1 <= kUploadSlotBytes) {
         std::lock_guard<std::mutex> lock(g_alloc_mutex);
@@ -491,7 +514,7 @@ int dsx_memcpy_d2d(void* dst, const void* src, size_t bytes)
 int dsx_sync(void)
 {
     DSX_REQUIRE_INIT();
-    if (other_lane_stream()) DSX_HIP(hipStreamSynchronize(other_lane_stream()));
+    if (int rc = sync_other_lanes()) return rc;
     DSX_HIP(hipStreamSynchronize(ctx().stream));
     return DSX_OK;
 }
@@ -499,7 +522,7 @@ int dsx_sync(void)
 int dsx_sync_lane(int lane)
 {
     DSX_REQUIRE_INIT();
-    DSX_CHECK_ARG(lane == 0 || lane == 1, "dsx_sync_lane: lane %d (0 or 1)", lane);
+    DSX_CHECK_ARG(lane >= 0 && lane < DSX_MAX_LANES, "dsx_sync_lane: lane %d (0..%d)", lane, DSX_MAX_LANES - 1);
     hipStream_t s = g_lane_stream[lane] ? g_lane_stream[lane] : ctx().stream;
     DSX_HIP(hipStreamSynchronize(s));
     return DSX_OK;
@@ -510,7 +533,7 @@ int dsx_sync_lane(int lane)
 int dsx_memcpy_d2h_lane(int lane, void* dst, const void* src, size_t bytes)
 {
     DSX_REQUIRE_INIT();
-    DSX_CHECK_ARG(lane == 0 || lane == 1, "dsx_memcpy_d2h_lane: lane %d (0 or 1)", lane);
+    DSX_CHECK_ARG(lane >= 0 && lane < DSX_MAX_LANES, "dsx_memcpy_d2h_lane: lane %d (0..%d)", lane, DSX_MAX_LANES - 1);
     if (bytes == 0) return DSX_OK;
     DSX_CHECK_ARG(dst && src, "dsx_memcpy_d2h_lane: null pointer");
     hipStream_t s = g_lane_stream[lane] ? g_lane_stream[lane] : ctx().stream;

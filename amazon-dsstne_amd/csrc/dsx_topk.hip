@@ -938,7 +938,7 @@ __global__ __launch_bounds__(256) void topk_gather_kernel(const V* in_values, V*
     values[pos] = (j < width) ? in_values[(uint64_t)b * width + col] : (V)0;
 }
 
-static LibScratch g_partial_of[2];   // per lane: two lanes may run a split top-K at the same time
+static LibScratch g_partial_of[DSX_MAX_LANES];   // per lane: lanes may run a split top-K at the same time
 
 static int ensure_partial(size_t bytes, uint64_t** out)
 {

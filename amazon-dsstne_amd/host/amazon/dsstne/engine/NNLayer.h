@@ -64,28 +64,44 @@ private:
     // (_segWidth == 0: none): NNNetwork::CalculateTopK then reads only the segments that can hold a result.
     unique_ptr<GpuBuffer<NNFloat>> _pbSegMax;
     uint32_t _segWidth = 0;
-    // With two lanes (NNNetwork::SetLanes) every layer has a second set of the three members above: the batch before the
-    // current one may still be running on the other lane's stream.  SwapLane exchanges the sets, so that the names above
-    // always denote the current batch's buffers.
-    unique_ptr<GpuBuffer<NNFloat>> _pbUnitOther;
-    unique_ptr<GpuBuffer<NNFloat>> _pbSegMaxOther;
-    uint32_t _segWidthOther = 0;
+    // With several lanes (NNNetwork::SetLanes) every layer has one set of the three members above (and of the two deferral
+    // members below) per lane: the batches before the current one may still be running on the other lanes' streams.  The
+    // names above always denote the current batch's buffers; SwitchLane parks them under the lane they belong to and takes
+    // out the set of the lane the next batch runs on.
+    struct LaneSet {
+        unique_ptr<GpuBuffer<NNFloat>> unit;
+        unique_ptr<GpuBuffer<NNFloat>> segMax;
+        uint32_t segWidth = 0;
+        bool deferred = false;
+        uint32_t deferredBatch = 0;
+    };
+    LaneSet _parked[DSX_MAX_LANES];
+    uint32_t _currentLane = 0;
     uint32_t _lanes = 1;
     // A wide output layer that feeds nothing but a top-K is not computed by the forward pass: NNNetwork::CalculateTopK /
     // CalculateFilteredTopK then run the layer and the top-K in one call that never stores the layer's result (dsx_fc_topk), and
     // whoever asks for the units themselves (NNNetwork::GetUnitBuffer, GetUnits) has them computed at that moment (Materialise).
     // _deferred: the units of the current batch have not been computed yet; _deferredBatch: its rows.
     bool _bDeferOutput = true;   // NNNetwork::SetDeferredOutput
-    bool _deferred = false, _deferredOther = false;
-    uint32_t _deferredBatch = 0, _deferredBatchOther = 0;
+    bool _deferred = false;
+    uint32_t _deferredBatch = 0;
     void Materialise();
-    void SwapLane()
+    void SwitchLane(uint32_t lane)
     {
-        _pbUnit.swap(_pbUnitOther);
-        _pbSegMax.swap(_pbSegMaxOther);
-        std::swap(_segWidth, _segWidthOther);
-        std::swap(_deferred, _deferredOther);
-        std::swap(_deferredBatch, _deferredBatchOther);
+        if (lane == _currentLane) return;
+        LaneSet& mine = _parked[_currentLane];
+        mine.unit.swap(_pbUnit);
+        mine.segMax.swap(_pbSegMax);
+        mine.segWidth = _segWidth;
+        mine.deferred = _deferred;
+        mine.deferredBatch = _deferredBatch;
+        LaneSet& next = _parked[lane];
+        _pbUnit.swap(next.unit);
+        _pbSegMax.swap(next.segMax);
+        _segWidth = next.segWidth;
+        _deferred = next.deferred;
+        _deferredBatch = next.deferredBatch;
+        _currentLane = lane;
     }
     int32_t _priority;
 

@@ -45,7 +45,7 @@ private:
     map<string, NNLayer*> _mLayer;
     bool _bDirty;
     bool _verbose;
-    uint32_t _lanes;                            // 1: one set of unit buffers, one stream; 2: consecutive batches alternate
+    uint32_t _lanes;                            // 1: one set of unit buffers, one stream; 2 (default) to DSX_MAX_LANES: consecutive batches take turns
     uint32_t _lane;                             // the lane of the current batch
 
     NNNetwork(NNNetworkDescriptor& nd, uint32_t batch = DefaultBatch);

@@ -76,20 +76,26 @@ struct NNDataSetBase {
     uint32_t _batch;
 
     // No counterpart in the reference (one set of arrays, blocking uploads).  Sparse data that arrives batch by batch
-    // (LoadSparseData) goes to a second set of device arrays, the one no kernel in flight reads, on the lane the next
-    // PredictBatch will use: the copy overlaps with the batch before it.  _pbSparseStart / End / Index / Data above always
-    // name the set that holds the latest load; kernels launched earlier keep reading the set they were given.
-    unique_ptr<GpuBuffer<uint64_t>> _pbSparseStartOther;
-    unique_ptr<GpuBuffer<uint64_t>> _pbSparseEndOther;
-    unique_ptr<GpuBuffer<uint32_t>> _pbSparseIndexOther;
+    // (LoadSparseData) goes to the set of device arrays that belongs to the lane the next PredictBatch will use, which no
+    // kernel of another lane reads: the copy overlaps with the batches before it.  _pbSparseStart / End / Index / Data above
+    // always name the set that holds the latest load (it belongs to lane _sparseLane); kernels launched earlier keep reading
+    // the set they were given.  The other lanes' sets are parked here.
     struct SparseSetState {
-        int _uploadLane = -1;        // lane whose stream carries the set's last unordered upload (-1: ordered on both lanes)
-        uint32_t _readLanes = 0;     // lanes that have launched readers of the set since that upload
-        uint32_t _orderedLanes = 3;  // lanes that are known to run after that upload
-        void* _uploaded = NULL;      // marker behind that upload: the next load into this set waits for it on the host, which
-                                     // keeps a caller that streams batches two batches ahead of the device and no more
+        int _uploadLane = -1;                 // lane whose stream carries the set's last unordered upload (-1: ordered on every lane)
+        uint32_t _readLanes = 0;              // lanes that have launched readers of the set since that upload
+        uint32_t _orderedLanes = 0xffffffffu; // lanes that are known to run after that upload
+        void* _uploaded = NULL;               // marker behind that upload: the next load into this set waits for it on the host, which
+                                              // keeps a caller that streams batches a few batches ahead of the device and no more
     };
-    SparseSetState _sparseSet, _sparseSetOther;
+    struct ParkedSparseSet {
+        unique_ptr<GpuBuffer<uint64_t>> _pbSparseStart;
+        unique_ptr<GpuBuffer<uint64_t>> _pbSparseEnd;
+        unique_ptr<GpuBuffer<uint32_t>> _pbSparseIndex;
+        SparseSetState _state;
+    };
+    ParkedSparseSet _parkedSparse[DSX_MAX_LANES];
+    SparseSetState _sparseSet;
+    int _sparseLane = 0;
     // Call before launching a kernel that reads the _pbSparse* arrays on the selected lane.
     void NoteSparseRead();
     // The lane the next PredictBatch will run on (kept by NNNetwork); a wrong value costs a wait between the lanes, no more.
@@ -146,7 +152,7 @@ public:
     unique_ptr<GpuBuffer<T>> _pbData;
     vector<T> _vSparseData;
     unique_ptr<GpuBuffer<T>> _pbSparseData;
-    unique_ptr<GpuBuffer<T>> _pbSparseDataOther;   // see _pbSparseStartOther
+    unique_ptr<GpuBuffer<T>> _parkedSparseData[DSX_MAX_LANES];   // see _parkedSparse
 
     // dense
     NNDataSet(uint32_t examples, const NNDataSetDimensions& dim, const string& name = "");

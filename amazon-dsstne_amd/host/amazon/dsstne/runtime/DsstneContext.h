@@ -13,8 +13,8 @@ private:
     const uint32_t batchSize;
     const uint32_t maxK;
     // one set per lane of the network: the results of the batch before the current one stay readable while the current runs
-    std::map<string, GpuBuffer<NNFloat>*> dOutputScores[2];
-    std::map<string, GpuBuffer<uint32_t>*> dOutputIndexes[2];
+    std::map<string, GpuBuffer<NNFloat>*> dOutputScores[DSX_MAX_LANES];
+    std::map<string, GpuBuffer<uint32_t>*> dOutputIndexes[DSX_MAX_LANES];
     std::vector<NNDataSetBase*> ownedDataSets;
 
 public:
@@ -26,9 +26,9 @@ public:
     void initInputLayerDataSets(const std::vector<NNDataSetDescriptor> datasetDescriptors);
     GpuBuffer<NNFloat>* getOutputScoresBuffer(const std::string& layerName);     // throws std::out_of_range for an unknown layer
     GpuBuffer<uint32_t>* getOutputIndexesBuffer(const std::string& layerName);
-    // the same for a given lane (0 or 1): the batch before the current one left its results in the other lane's buffers
-    GpuBuffer<NNFloat>* getOutputScoresBuffer(const std::string& layerName, int lane) { return dOutputScores[lane & 1].at(layerName); }
-    GpuBuffer<uint32_t>* getOutputIndexesBuffer(const std::string& layerName, int lane) { return dOutputIndexes[lane & 1].at(layerName); }
+    // the same for a given lane: the batch before the current one left its results in the buffers of the lane before the current one
+    GpuBuffer<NNFloat>* getOutputScoresBuffer(const std::string& layerName, int lane) { return dOutputScores[lane % DSX_MAX_LANES].at(layerName); }
+    GpuBuffer<uint32_t>* getOutputIndexesBuffer(const std::string& layerName, int lane) { return dOutputIndexes[lane % DSX_MAX_LANES].at(layerName); }
 
     static DsstneContext* fromPtr(long ptr)
     {

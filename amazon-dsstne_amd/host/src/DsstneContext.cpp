@@ -29,7 +29,7 @@ DsstneContext::DsstneContext(const string& networkFilename, uint32_t batchSize, 
             size_t outputBufferLength = (size_t)maxK * batchSize;
             printf("DsstneContext::DsstneContext: Allocating output score and index buffers, each of size %zu for output layer %s\n",
                    outputBufferLength, layerName.c_str());
-            for (int lane = 0; lane < 2; lane++) {
+            for (int lane = 0; lane < DSX_MAX_LANES; lane++) {
                 dOutputScores[lane][layerName] = new GpuBuffer<NNFloat>(outputBufferLength, false, false);
                 dOutputIndexes[lane][layerName] = new GpuBuffer<uint32_t>(outputBufferLength, false, false);
             }
@@ -51,7 +51,7 @@ GpuBuffer<uint32_t>* DsstneContext::getOutputIndexesBuffer(const std::string& la
 DsstneContext::~DsstneContext()
 {
     const string networkName = getNetwork() ? getNetwork()->GetName() : string("<none>");
-    for (int lane = 0; lane < 2; lane++) {
+    for (int lane = 0; lane < DSX_MAX_LANES; lane++) {
         for (const auto& kv : dOutputScores[lane]) delete kv.second;
         for (const auto& kv : dOutputIndexes[lane]) delete kv.second;
         dOutputScores[lane].clear();

@@ -69,7 +69,7 @@ NNDataSetBase::~NNDataSetBase()
 {
     if (dsx_is_initialized()) {
         dsx_marker_destroy(_sparseSet._uploaded);
-        dsx_marker_destroy(_sparseSetOther._uploaded);
+        for (auto& set : _parkedSparse) dsx_marker_destroy(set._state._uploaded);
     }
 }
 
@@ -185,7 +185,7 @@ template <typename T> void NNDataSet<T>::checkSparseLoad(const uint64_t start0, 
 
 template <typename T> void NNDataSet<T>::uploadSparse()
 {
-    { void* marker = _sparseSet._uploaded; _sparseSet = SparseSetState(); _sparseSet._uploaded = marker; }   // the uploads below are ordered on both lanes
+    { void* marker = _sparseSet._uploaded; _sparseSet = SparseSetState(); _sparseSet._uploaded = marker; }   // the uploads below are ordered on every lane
     // The buffers were sized at construction (or by Shard); batches loaded later reuse them without reallocation.
     _pbSparseStart->Upload(_vSparseStart.data());
     _pbSparseEnd->Upload(_vSparseEnd.data());
@@ -221,21 +221,34 @@ void NNDataSet<T>::LoadSparseData(const uint64_t* srcSparseStart, const uint64_t
     const bool direct = _pbSparseStart && _pbSparseEnd && _pbSparseIndex && _pbSparseStart->_length >= _uniqueExamples &&
                         _pbSparseIndex->_length >= dataLength && (!_pbSparseData || _pbSparseData->_length >= dataLength);
     if (direct) {
-        if (!_pbSparseStartOther) {
-            _pbSparseStartOther.reset(new GpuBuffer<uint64_t>(_pbSparseStart->_length, false, _bStreaming));
-            _pbSparseEndOther.reset(new GpuBuffer<uint64_t>(_pbSparseEnd->_length, false, _bStreaming));
-            _pbSparseIndexOther.reset(new GpuBuffer<uint32_t>(_pbSparseIndex->_length, false, _bStreaming));
-            if (_pbSparseData) _pbSparseDataOther.reset(new GpuBuffer<T>(_pbSparseData->_length, false, _bStreaming));
-        }
-        _pbSparseStart.swap(_pbSparseStartOther);
-        _pbSparseEnd.swap(_pbSparseEndOther);
-        _pbSparseIndex.swap(_pbSparseIndexOther);
-        _pbSparseData.swap(_pbSparseDataOther);
-        std::swap(_sparseSet, _sparseSetOther);
         const int selected = dsx_get_lane();
-        const int target = (s_nextLane == 1) ? 1 : 0;
+        const int target = (s_nextLane >= 0 && s_nextLane < DSX_MAX_LANES) ? s_nextLane : 0;
+        if (target != _sparseLane) {   // park the arrays of the lane that loaded last, take out the target lane's
+            ParkedSparseSet& mine = _parkedSparse[_sparseLane];
+            mine._pbSparseStart.swap(_pbSparseStart);
+            mine._pbSparseEnd.swap(_pbSparseEnd);
+            mine._pbSparseIndex.swap(_pbSparseIndex);
+            mine._state = _sparseSet;
+            _parkedSparseData[_sparseLane].swap(_pbSparseData);
+            ParkedSparseSet& next = _parkedSparse[target];
+            if (!next._pbSparseStart || next._pbSparseStart->_length < mine._pbSparseStart->_length ||
+                next._pbSparseIndex->_length < mine._pbSparseIndex->_length) {   // first use, or the arrays have grown since (Shard)
+                next._pbSparseStart.reset(new GpuBuffer<uint64_t>(mine._pbSparseStart->_length, false, _bStreaming));
+                next._pbSparseEnd.reset(new GpuBuffer<uint64_t>(mine._pbSparseEnd->_length, false, _bStreaming));
+                next._pbSparseIndex.reset(new GpuBuffer<uint32_t>(mine._pbSparseIndex->_length, false, _bStreaming));
+                if (_parkedSparseData[_sparseLane]) _parkedSparseData[target].reset(new GpuBuffer<T>(_parkedSparseData[_sparseLane]->_length, false, _bStreaming));
+                next._state = SparseSetState();
+                next._state._orderedLanes = 0;   // nothing has been loaded into it yet
+            }
+            _pbSparseStart.swap(next._pbSparseStart);
+            _pbSparseEnd.swap(next._pbSparseEnd);
+            _pbSparseIndex.swap(next._pbSparseIndex);
+            _pbSparseData.swap(_parkedSparseData[target]);
+            _sparseSet = next._state;
+            _sparseLane = target;
+        }
         if (target != selected) dsxFatal(dsx_set_lane(target), "NNDataSet::LoadSparseData");
-        if (_sparseSet._readLanes & ~(1u << target)) dsxFatal(dsx_lane_wait_other(), "NNDataSet::LoadSparseData");   // readers on the other lane
+        if (_sparseSet._readLanes & ~(1u << target)) dsxFatal(dsx_lane_wait_other(), "NNDataSet::LoadSparseData");   // readers on other lanes
         // The load before the last went into this set: once its copies are through, the device is at most two batches behind.
         // (A host that queues dozens of batches ahead makes the runtime stall in bursts of 150-200 us: measured 105-137 us per
         // batch of 1024 instead of 102.)
@@ -424,8 +437,8 @@ int NNDataSetBase::s_nextLane = 0;
 
 void NNDataSetBase::NoteSparseRead()
 {
-    const uint32_t lane = 1u << (dsx_get_lane() & 1);
-    if (_sparseSet._uploadLane >= 0 && !(_sparseSet._orderedLanes & lane)) {   // loaded on the other lane: run after that copy
+    const uint32_t lane = 1u << dsx_get_lane();
+    if (_sparseSet._uploadLane >= 0 && !(_sparseSet._orderedLanes & lane)) {   // loaded on another lane: run after that copy
         dsxFatal(dsx_lane_wait_other(), "NNDataSetBase::NoteSparseRead");
         _sparseSet._orderedLanes |= lane;
     }

@@ -62,9 +62,8 @@ void NNLayer::Deallocate()
     _pbUnit.reset();
     _pbSegMax.reset();
     _segWidth = 0;
-    _pbUnitOther.reset();
-    _pbSegMaxOther.reset();
-    _segWidthOther = 0;
+    _deferred = false;
+    for (auto& set : _parked) set = LaneSet();
 }
 
 void NNLayer::SetBatch(uint32_t batch)
@@ -83,9 +82,12 @@ void NNLayer::Allocate(bool validate)
     // hidden and output layers, dense inputs and sparse inputs that cannot use the sparse-Z path own an activation buffer
     if (!_bSparse || !_bFastSparse || (_kind != Input) || (_bSparse && (_kind == Input) && validate)) {
         _pbUnit.reset(new GpuBuffer<NNFloat>(size));
-        if (_lanes > 1) _pbUnitOther.reset(new GpuBuffer<NNFloat>(size));
-        printf("NNLayer::Allocate: Allocating %" PRIu64 " bytes (%u, %u) of unit data for layer %s%s\n", size * sizeof(NNFloat), _maxLocalStride,
-               _localBatch, _name.c_str(), _lanes > 1 ? ", twice (two lanes)" : "");
+        for (uint32_t lane = 0; lane < _lanes; lane++)
+            if (lane != _currentLane) _parked[lane].unit.reset(new GpuBuffer<NNFloat>(size));
+        printf("NNLayer::Allocate: Allocating %" PRIu64 " bytes (%u, %u) of unit data for layer %s", size * sizeof(NNFloat), _maxLocalStride, _localBatch,
+               _name.c_str());
+        if (_lanes > 1) printf(", %u times (one per lane)", _lanes);
+        printf("\n");
     }
     _bDirty = false;
 }

@@ -274,12 +274,12 @@ void NNNetwork::PredictBatch(uint32_t layers)
         }
     }
     if (_lanes > 1) {
-        // this batch takes the lane the batch before the last one used
-        _lane ^= 1;
-        for (auto l : _vLayer) l->SwapLane();
+        // this batch takes the lane that has been idle longest
+        _lane = (_lane + 1) % _lanes;
+        for (auto l : _vLayer) l->SwitchLane(_lane);
         dsxFatal(dsx_set_lane((int)_lane), "NNNetwork::PredictBatch: lane");
     }
-    NNDataSetBase::s_nextLane = (_lanes > 1) ? (int)(_lane ^ 1) : (int)_lane;   // where a LoadSparseData for the next batch should go
+    NNDataSetBase::s_nextLane = (int)((_lane + 1) % _lanes);   // where a LoadSparseData for the next batch should go
     uint32_t batch = _batch;
     if (_position + batch > _examples) batch = _examples - _position;
     ClearUpdates();
@@ -289,8 +289,8 @@ void NNNetwork::PredictBatch(uint32_t layers)
 
 bool NNNetwork::SetLanes(uint32_t lanes)
 {
-    if (lanes < 1 || lanes > 2) {
-        printf("NNNetwork::SetLanes: %u lanes requested (1 or 2).\n", lanes);
+    if (lanes < 1 || lanes > DSX_MAX_LANES) {
+        printf("NNNetwork::SetLanes: %u lanes requested (1..%d).\n", lanes, DSX_MAX_LANES);
         return false;
     }
     if (lanes == _lanes) return true;
@@ -301,6 +301,7 @@ bool NNNetwork::SetLanes(uint32_t lanes)
     NNDataSetBase::s_nextLane = (lanes > 1) ? 1 : 0;
     for (auto l : _vLayer) {
         l->_lanes = lanes;
+        l->_currentLane = 0;
         l->_bDirty = true;   // unit buffers are allocated anew
     }
     _bDirty = true;

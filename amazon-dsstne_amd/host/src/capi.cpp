@@ -27,8 +27,8 @@ struct dsstne_context {
     int maxK = 0;
     map<string, NNDataSetBase*> datasets;
     vector<NNDataSetBase*> pending;
-    map<string, GpuBuffer<NNFloat>*> scores[2];      // per lane of the network
-    map<string, GpuBuffer<uint32_t>*> indexes[2];
+    map<string, GpuBuffer<NNFloat>*> scores[DSX_MAX_LANES];      // per lane of the network
+    map<string, GpuBuffer<uint32_t>*> indexes[DSX_MAX_LANES];
 
     NNNetwork* net() const { return dc ? dc->getNetwork() : network; }
     GpuBuffer<NNFloat>* scoreBuf(const string& layer) { return dc ? dc->getOutputScoresBuffer(layer) : scores[network->GetLane()].at(layer); }
@@ -56,7 +56,7 @@ static void makeResultBuffers(dsstne_context* c)
     if (c->maxK <= 0) return;
     vector<const NNLayer*> outs;
     for (auto it = c->network->GetLayers(NNLayer::Kind::Output, outs); it != outs.end(); ++it) {
-        for (int lane = 0; lane < 2; lane++) {
+        for (int lane = 0; lane < DSX_MAX_LANES; lane++) {
             c->scores[lane][(*it)->GetName()] = new GpuBuffer<NNFloat>((size_t)c->maxK * c->batch);
             c->indexes[lane][(*it)->GetName()] = new GpuBuffer<uint32_t>((size_t)c->maxK * c->batch);
         }
@@ -198,7 +198,7 @@ int dsstne_set_weights(dsstne_context* c, const char* input_layer, const char* o
 void dsstne_shutdown(dsstne_context* c)
 {
     if (!c) return;
-    for (int lane = 0; lane < 2; lane++) {
+    for (int lane = 0; lane < DSX_MAX_LANES; lane++) {
         for (auto& kv : c->scores[lane]) delete kv.second;
         for (auto& kv : c->indexes[lane]) delete kv.second;
     }
@@ -365,7 +365,7 @@ int dsstne_get_topk_previous(dsstne_context* c, const char* layer, uint32_t rows
     CAPI_TRY
     NNNetwork* n = c->net();
     if (n->GetLanes() < 2) return fail("dsstne_get_topk_previous: the network runs on one lane");
-    const int lane = (int)(n->GetLane() ^ 1u);
+    const int lane = (int)((n->GetLane() + n->GetLanes() - 1) % n->GetLanes());
     GpuBuffer<NNFloat>* s = c->dc ? c->dc->getOutputScoresBuffer(layer, lane) : c->scores[lane].at(layer);
     GpuBuffer<uint32_t>* i = c->dc ? c->dc->getOutputIndexesBuffer(layer, lane) : c->indexes[lane].at(layer);
     dsxFatal(dsx_memcpy_d2h_lane(lane, scores, s->_pDevData, (size_t)rows * k * sizeof(float)), "dsstne_get_topk_previous");
@@ -377,7 +377,7 @@ int dsstne_get_topk_previous(dsstne_context* c, const char* layer, uint32_t rows
 int dsstne_set_lanes(dsstne_context* c, uint32_t lanes)
 {
     CAPI_TRY
-    return c->net()->SetLanes(lanes) ? 0 : fail("dsstne_set_lanes: %u lanes (1 or 2)", lanes);
+    return c->net()->SetLanes(lanes) ? 0 : fail("dsstne_set_lanes: %u lanes (1..%d)", lanes, DSX_MAX_LANES);
     CAPI_CATCH(-1)
 }
 

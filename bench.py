@@ -119,6 +119,8 @@ def network_bench(args, pkg, lib):
     # results stay in HBM; consecutive steps take consecutive batches of the resident dataset.
     net = Network(p)
     net.bind_input()
+    if args.lanes != 2:
+        net.set_lanes(args.lanes)   # NNNetwork's default is two
 
     def step(i=0):
         net.predict_batch((i % batches) * B)
@@ -143,7 +145,7 @@ def network_bench(args, pkg, lib):
     net.set_lanes(1)
     settle(pkg, lib, step)
     ms_one_lane = float(np.median(timed_windows(step, net.sync, args.steps, 3)))
-    net.set_lanes(2)
+    net.set_lanes(args.lanes)
     # ... and with the output layer stored by PredictBatch as the reference does, instead of computed together with the top-K
     # (NNNetwork::SetDeferredOutput; only layers of 131,072 units or more are deferred, so this differs for config 4 alone)
     net.set_deferred_output(False)
@@ -333,14 +335,14 @@ def network_bench(args, pkg, lib):
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": p.name, "batch": B, "input_width": p.widths[0], "layers": p.widths[1:], "top_k": K, "filtered": True,
-                   "resident_batches": batches, "batch_nnz": nnzB, "mean_batch_nnz": round(nnz_mean, 1)},
+                   "resident_batches": batches, "batch_nnz": nnzB, "mean_batch_nnz": round(nnz_mean, 1), "lanes": args.lanes},
         "windows": {"count": WINDOWS, "steps_each": args.steps, "ms_per_step": [round(w, 5) for w in windows],
                     "min": round(min(windows), 5), "median": round(ms_step, 5), "max": round(max(windows), 5),
                     "note": "value is the median window; the timed steps cycle over the resident batches"},
         "roofline": roofline,
         "pipeline": {"gemm_flops_per_step": flops_step, "achieved": round(flops_step / ms_step / 1e9, 3), "peak": FP32_MFMA_PEAK_TF,
                      "unit": "TFLOP/s", "frac": round(flops_step / ms_step / 1e9 / FP32_MFMA_PEAK_TF, 4),
-                     "note": "all dense-layer flops of a step over the timed step itself (two lanes, every kernel of the step included): the fraction of the fp32 MFMA peak the whole path sustains"},
+                     "note": "all dense-layer flops of a step over the timed step itself (every kernel of the step included, batches on %d lanes)" % args.lanes + ": the fraction of the fp32 MFMA peak the whole path sustains"},
         "kernels": {n: {k: (round(v, 5) if isinstance(v, float) else v) for k, v in kv.items()} for n, kv in kernels.items()},
         "cpu_baseline": cpu,
         "clock_settle_ms": SETTLE_SECONDS * 1e3,
@@ -429,6 +431,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=2, help="1..4 = networks of the benchmark definition, 5 = KNN")
+    ap.add_argument("--lanes", type=int, default=2, help="NNNetwork::SetLanes for the timed step: batches in flight (1..4, the library's default is 2)")
     ap.add_argument("--knn-items", type=int, default=2000000)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget; 0 skips it")
     ap.add_argument("--calibrate-copy", type=int, default=0, help="also run a plain d2d copy of this many MiB (counter calibration)")

@@ -84,7 +84,8 @@ int dsstne_get_topk(dsstne_context* ctx, const char* layer, uint32_t rows, uint3
  * between two sets of unit and result buffers on two device streams, so a batch's kernels overlap with those of the batch
  * before it (NNNetwork::SetLanes).  dsstne_get_topk reads the batch predicted last; dsstne_get_topk_previous the one before
  * it, waiting for that batch only — a loop that issues batch i+1 and then collects batch i keeps the device busy.
- * dsstne_set_lanes(ctx, 1) goes back to one set of buffers and one stream. */
+ * dsstne_set_lanes(ctx, 1) goes back to one set of buffers and one stream; up to four lanes can be asked for (consecutive
+ * batches then take turns on as many sets of buffers). */
 int dsstne_get_topk_previous(dsstne_context* ctx, const char* layer, uint32_t rows, uint32_t k, float* scores, uint32_t* indexes);
 int dsstne_set_lanes(dsstne_context* ctx, uint32_t lanes);
 /* No counterpart in the reference (NNNetwork::SetDeferredOutput).  By default a wide output layer that feeds nothing else is
@@ -99,7 +100,7 @@ int dsstne_get_units(dsstne_context* ctx, const char* layer, float* units, size_
 /* NNNetwork::GetUnitBuffer (engine/NNNetwork.cpp:2006-2020): device address of the layer's [batch][stride] activations of the
  * batch predicted last, as the reference's JNI predict takes it (Dsstne.cpp:366).  The call returns once that batch's
  * forward pass has finished on the device, so the caller may read the memory with any copy or kernel of its own; the
- * address changes from batch to batch with two lanes (fetch it per batch, as the reference's callers do).  NULL on failure. */
+ * address changes from batch to batch with more than one lane (fetch it per batch, as the reference's callers do).  NULL on failure. */
 void* dsstne_get_unit_buffer(dsstne_context* ctx, const char* layer);
 /* NNLayer::SetUnits (engine/NNLayer.cpp:318-368 group): overwrites the layer's unit buffer (batch x stride values) from the host. */
 int dsstne_set_units(dsstne_context* ctx, const char* layer, const float* units, size_t count);

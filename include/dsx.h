@@ -119,20 +119,22 @@ int dsx_memset(void* device_ptr, int value, size_t bytes);
 int dsx_memcpy_h2d(void* device_dst, const void* host_src, size_t bytes);
 int dsx_memcpy_d2h(void* host_dst, const void* device_src, size_t bytes);   /* GpuBuffer::Download */
 int dsx_memcpy_d2d(void* device_dst, const void* device_src, size_t bytes); /* GpuBuffer::Copy     */
-int dsx_sync(void);                                                          /* waits for both lanes */
-/* No counterpart in the reference (which runs everything on the default stream with blocking copies): the library has two
- * lanes, each an in-order stream; whatever is launched goes to the selected one (lane 0 until told otherwise).  Two batches
- * issued on different lanes run concurrently; uploads, clears, device-to-device copies and timers order both lanes around
- * themselves, dsx_memcpy_d2h and dsx_sync wait for both, dsx_memcpy_d2h_lane for one lane only. */
+int dsx_sync(void);                                                          /* waits for every lane */
+/* No counterpart in the reference (which runs everything on the default stream with blocking copies): the library has up to
+ * DSX_MAX_LANES lanes, each an in-order stream; whatever is launched goes to the selected one (lane 0 until told otherwise;
+ * a lane's stream is made when the lane is first selected).  Batches issued on different lanes run concurrently; uploads,
+ * clears, device-to-device copies and timers order all lanes around themselves, dsx_memcpy_d2h and dsx_sync wait for all of
+ * them, dsx_memcpy_d2h_lane for one lane only. */
+#define DSX_MAX_LANES 4
 int dsx_set_lane(int lane);
 int dsx_get_lane(void);
-int dsx_sync_lane(int lane);   /* waits for everything queued on one lane (before the second lane exists: on the only stream) */
+int dsx_sync_lane(int lane);   /* waits for everything queued on one lane (a lane never selected: on the selected one) */
 int dsx_memcpy_d2h_lane(int lane, void* host_dst, const void* device_src, size_t bytes);
 /* For data that arrives batch by batch (no counterpart in the reference, whose uploads block).  dsx_memcpy_h2d_unordered is
- * dsx_memcpy_h2d on the selected lane only: the other lane is neither waited for nor told to wait, so the copy overlaps with
- * whatever the other lane runs.  The caller guarantees that nothing queued on the other lane touches device_dst, and calls
- * dsx_lane_wait_other (the selected lane waits for everything queued so far on the other one) before work on one lane
- * depends on what the other lane wrote. */
+ * dsx_memcpy_h2d on the selected lane only: the other lanes are neither waited for nor told to wait, so the copy overlaps with
+ * whatever they run.  The caller guarantees that nothing queued on another lane touches device_dst, and calls
+ * dsx_lane_wait_other (the selected lane waits for everything queued so far on the other ones) before work on one lane
+ * depends on what another lane wrote. */
 int dsx_memcpy_h2d_unordered(void* device_dst, const void* host_src, size_t bytes);
 int dsx_lane_wait_other(void);
 /* A marker is a point in the selected lane's queue (no counterpart in the reference): dsx_marker_record places it after

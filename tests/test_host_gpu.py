@@ -325,12 +325,12 @@ def reference_batches(orc, p, positions):
     return out
 
 
-@pytest.mark.parametrize("config,batches,lanes", [(1, 9, 2), (2, 4, 2), (1, 5, 1), (1, 40, 2)])
+@pytest.mark.parametrize("config,batches,lanes", [(1, 9, 2), (2, 4, 2), (1, 5, 1), (1, 40, 2), (1, 11, 3), (2, 6, 4), (1, 40, 4)])
 def test_streamed_batches_on_two_lanes(pkg, dsx, orc, synth, config, batches, lanes):
     """Batches handed over as host arrays one after the other (NNDataSet::LoadSparseData, as the reference's JNI predict feeds
     it): the dataset holds one batch, every load replaces it, and the results of batch i are collected while batch i + 1 is
-    already queued.  The loads go to alternating sets of device arrays on alternating lanes; every batch must still see its
-    own data, as input and as filter."""
+    already queued.  The loads go to the set of device arrays of the lane the batch will run on, lane after lane in turn; every
+    batch must still see its own data, as input and as filter."""
     import copy
     from amazon_dsstne_amd import host_api
     big = synth.config(config, batches=batches)
@@ -352,18 +352,18 @@ def test_streamed_batches_on_two_lanes(pkg, dsx, orc, synth, config, batches, la
     net = host_api.Network(one, max_k=big.k)
     try:
         net.bind_input()
-        if lanes == 1:
-            net.set_lanes(1)
+        if lanes != 2:
+            net.set_lanes(lanes)
         got = []
         for n, pos in enumerate(positions):
             net.load_sparse(*batch_arrays(pos))
             net.predict_batch(0)
             net.topk(big.k, filter_dataset="input")
-            if lanes == 2 and n > 0:
+            if lanes >= 2 and n > 0:
                 got.append(net.get_topk_previous(big.batch))            # the batch before, while this one runs
             elif lanes == 1:
                 got.append(net.get_topk(big.batch))
-        if lanes == 2:
+        if lanes >= 2:
             got.append(net.get_topk(big.batch))
         for n, ((rows, keys, idx, scores), (gk, gi)) in enumerate(zip(want, got)):
             assert_topk_parity(gk, gi, keys, idx, scores, "%s streamed batch %d on %d lane(s)" % (big.name, n, lanes))
@@ -385,10 +385,10 @@ def test_streamed_batches_on_two_lanes(pkg, dsx, orc, synth, config, batches, la
         net.close()
 
 
-@pytest.mark.parametrize("config,batches", [(1, 7), (2, 3)])
-def test_two_lanes_keep_batches_apart(pkg, dsx, orc, synth, config, batches):
-    """Consecutive PredictBatch calls alternate between two sets of buffers on two streams (NNNetwork::SetLanes).  A loop that
-    issues batch i+1 before it collects batch i must get every batch's own results; the last batch is short."""
+@pytest.mark.parametrize("config,batches,lanes", [(1, 7, 2), (2, 3, 2), (1, 9, 3), (2, 5, 4), (1, 7, 4)])
+def test_two_lanes_keep_batches_apart(pkg, dsx, orc, synth, config, batches, lanes):
+    """Consecutive PredictBatch calls take turns on the sets of buffers and streams of two to four lanes (NNNetwork::SetLanes).
+    A loop that issues batch i+1 before it collects batch i must get every batch's own results; the last batch is short."""
     from amazon_dsstne_amd import host_api
     p = synth.config(config, batches=batches)
     short = p.batch // 3
@@ -400,6 +400,8 @@ def test_two_lanes_keep_batches_apart(pkg, dsx, orc, synth, config, batches):
     net = host_api.Network(p, max_k=p.k)
     try:
         net.bind_input()
+        if lanes != 2:
+            net.set_lanes(lanes)
         got = []
         for n, pos in enumerate(positions):
             net.predict_batch(pos)
@@ -422,7 +424,7 @@ def test_two_lanes_keep_batches_apart(pkg, dsx, orc, synth, config, batches):
         net.predict_batch(positions[1])
         unit = net.units(rows=p.batch)
         _, ref_unit, _, _ = orc.forward(p, positions[1], p.batch, filtered=False, want_unit=True, want_topk=False)
-        assert_units_close(unit, ref_unit, p, positions[1], p.name + " units on two lanes")
+        assert_units_close(unit, ref_unit, p, positions[1], p.name + " units on several lanes")
         net.load_sparse(p.start, p.end, p.sparse_data, p.sparse_index)
         net.predict_batch(positions[0])
         net.topk(p.k, filter_dataset="input")
@@ -437,11 +439,14 @@ def test_two_lanes_keep_batches_apart(pkg, dsx, orc, synth, config, batches):
             net.topk(p.k, filter_dataset="input")
             gk, gi = net.get_topk(want[n][0])
             assert_topk_parity(gk, gi, want[n][1], want[n][2], want[n][3], "%s batch %d on one lane" % (p.name, n))
-        net.set_lanes(2)
-        net.predict_batch(positions[0])
-        net.topk(p.k, filter_dataset="input")
-        gk, gi = net.get_topk(want[0][0])
-        assert_topk_parity(gk, gi, want[0][1], want[0][2], want[0][3], p.name + " back on two lanes")
+        net.set_lanes(lanes)
+        for n, pos in enumerate(positions[:3]):
+            net.predict_batch(pos)
+            net.topk(p.k, filter_dataset="input")
+        gk, gi = net.get_topk(want[2][0])
+        assert_topk_parity(gk, gi, want[2][1], want[2][2], want[2][3], p.name + " back on %d lanes" % lanes)
+        gk, gi = net.get_topk_previous(want[1][0])
+        assert_topk_parity(gk, gi, want[1][1], want[1][2], want[1][3], p.name + " back on %d lanes, batch before" % lanes)
     finally:
         net.close()
 
@@ -449,8 +454,8 @@ def test_two_lanes_keep_batches_apart(pkg, dsx, orc, synth, config, batches):
 def test_unit_buffer_read_with_a_bare_hipmemcpy(pkg, dsx, orc, synth):
     """The reference's callers follow PredictBatch with GetUnitBuffer and a plain cudaMemcpy on the default stream
     (utils/NNRecsGenerator.cpp:83, java/src/main/native/com_amazon_dsstne_Dsstne.cpp:366).  The same pattern with hipMemcpy from the
-    HIP runtime itself, not through this library: every batch read this way must be that batch's finished activations, on two
-    lanes (the pointer alternates between two buffers) and on one."""
+    HIP runtime itself, not through this library: every batch read this way must be that batch's finished activations, on several
+    lanes (the pointer goes round as many buffers) and on one."""
     import ctypes as C
     from amazon_dsstne_amd import host_api
     hip = C.CDLL("libamdhip64.so")
@@ -462,7 +467,7 @@ def test_unit_buffer_read_with_a_bare_hipmemcpy(pkg, dsx, orc, synth):
     net = host_api.Network(p, max_k=p.k)
     try:
         net.bind_input()
-        for lanes in (2, 1):
+        for lanes in (2, 1, 4, 3):
             net.set_lanes(lanes)
             seen = set()
             for rep in range(2):
