@@ -737,7 +737,13 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
     constexpr int kFU = 4;
     uint32_t fcol[kFU];
     float fm[kFU], fv[kFU];
+    // A row with few listed columns and the default multiplier does not read their scores at all (one round trip less on the
+    // way to the bound): a segment that holds a listed column is simply left out of the bound, and a listed column's zero is
+    // only looked at when zeros can still enter a list.  A long list would leave too few segments for a good bound: such rows,
+    // and rows with multipliers, read the listed scores first and leave out only the segments whose maximum is one of them.
+    bool light = false;   // the same for the whole workgroup
     if constexpr (FILTERED) {
+        light = !a.fmul && (fe - fs) * 2 <= a.nseg;
         const uint32_t words = (a.width + 31) / 32;
         for (uint32_t i = threadIdx.x; i < words; i += kTopkThreads) sBitmap[i] = 0;
         for (uint32_t i = threadIdx.x; i < a.nseg; i += kTopkThreads) sFiltMax[i] = 0;
@@ -756,17 +762,28 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
                 if (a.fmul) fm[u] = a.fmul[t];
             }
         }
+        if (light) {   // (at most nseg / 2 <= 1024 listed columns: they are all in fcol)
 #pragma unroll
-        for (int u = 0; u < kFU; u++) {
-            fv[u] = 0.0f;
-            if (fcol[u] < a.width) fv[u] = row[fcol[u]];
-        }
+            for (int u = 0; u < kFU; u++) {
+                fv[u] = 0.0f;
+                if (fcol[u] < a.width) {
+                    atomicOr(&sBitmap[fcol[u] >> 5], 1u << (fcol[u] & 31));
+                    sFiltMax[fcol[u] / kGuidedSegWidth] = 0xffffffffu;   // equal to no key of a maximum that takes part (NaN patterns aside, which are 0 here)
+                }
+            }
+        } else {
 #pragma unroll
-        for (int u = 0; u < kFU; u++)
-            if (fcol[u] < a.width) mark(fcol[u], fv[u]);
-        for (uint64_t t = fs + (uint64_t)kFU * kTopkThreads + threadIdx.x; t < fe; t += kTopkThreads) {
-            const uint32_t c = a.fidx[t];
-            if (c < a.width) mark(c, row[c]);
+            for (int u = 0; u < kFU; u++) {
+                fv[u] = 0.0f;
+                if (fcol[u] < a.width) fv[u] = row[fcol[u]];
+            }
+#pragma unroll
+            for (int u = 0; u < kFU; u++)
+                if (fcol[u] < a.width) mark(fcol[u], fv[u]);
+            for (uint64_t t = fs + (uint64_t)kFU * kTopkThreads + threadIdx.x; t < fe; t += kTopkThreads) {
+                const uint32_t c = a.fidx[t];
+                if (c < a.width) mark(c, row[c]);
+            }
         }
     }
     __syncthreads();
@@ -789,7 +806,7 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
             tk[e] = mk[e];
             if constexpr (FILTERED) {
                 const uint32_t idx = e * kTopkThreads + threadIdx.x;
-                if (idx < a.nseg && sFiltMax[idx] == mk[e]) tk[e] = 0;
+                if (idx < a.nseg && (light ? sFiltMax[idx] != 0 : sFiltMax[idx] == mk[e])) tk[e] = 0;
             }
         }
         const uint32_t tw = wave_kth_key<E>(tk, a.k);
@@ -865,19 +882,24 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
         list.drain();
     }
 
-    // Every listed column is injected once with score * multiplier; the lane that clears a column's bit owns it.
+    // Every listed column is injected once with score * multiplier; the lane that clears a column's bit owns it.  A listed
+    // column multiplied by 0 scores 0 (or nothing at all, if its score is not finite): it cannot enter the list of a
+    // wavefront that already holds k scores above 0, and the final k-th score is at least that wavefront's.
     if constexpr (FILTERED) {
         __syncthreads();
-        for (uint64_t base = fs; base < fe; base += (uint64_t)kFU * kTopkThreads) {
-            if (base != fs) {
+        const bool zeros_matter = a.fmul != nullptr || !(list.thr_key > 0.0f);   // wave-uniform
+        for (uint64_t base = fs; base < fe && zeros_matter; base += (uint64_t)kFU * kTopkThreads) {
+            if (base != fs || light) {
+                if (base != fs) {
 #pragma unroll
-                for (int u = 0; u < kFU; u++) {
-                    const uint64_t t = base + (uint64_t)u * kTopkThreads + threadIdx.x;
-                    fcol[u] = 0xffffffffu;
-                    fm[u] = 0.0f;
-                    if (t < fe) {
-                        fcol[u] = a.fidx[t];
-                        if (a.fmul) fm[u] = a.fmul[t];
+                    for (int u = 0; u < kFU; u++) {
+                        const uint64_t t = base + (uint64_t)u * kTopkThreads + threadIdx.x;
+                        fcol[u] = 0xffffffffu;
+                        fm[u] = 0.0f;
+                        if (t < fe) {
+                            fcol[u] = a.fidx[t];
+                            if (a.fmul) fm[u] = a.fmul[t];
+                        }
                     }
                 }
 #pragma unroll
