@@ -429,7 +429,7 @@ int dsx_memcpy_h2d(void* dst, const void* src, size_t bytes)
     DSX_REQUIRE_INIT();
     if (bytes == 0) return DSX_OK;
     DSX_CHECK_ARG(dst && src, "dsx_memcpy_h2d: null pointer");
-    // the destination may still be read by kernels of the other lane, and is read by whatever either lane runs next
+    // the destination may still be read by kernels of another lane, and is read by whatever any lane runs next
     if (int rc = lanes_join_before()) return rc;
     if (int rc = upload_on_selected_lane(dst, src, bytes)) return rc;
     return lanes_join_after();

@@ -76,7 +76,8 @@ public:
     // No counterpart in the reference.  With two lanes (the default) consecutive PredictBatch calls alternate between two sets
     // of unit buffers and two device streams: a batch's kernels (and the top-K calls that follow its PredictBatch) overlap
     // with those of the batch before it.  Everything read back through this API waits as needed; a device pointer obtained
-    // from GetUnitBuffer belongs to the batch predicted last.  One lane restores single buffers.
+    // from GetUnitBuffer belongs to the batch predicted last.  One lane restores single buffers; three or four (at most
+    // DSX_MAX_LANES) let consecutive batches take turns on as many sets.
     bool SetLanes(uint32_t lanes);
     // No counterpart in the reference.  By default a wide output layer that feeds nothing else is not computed by PredictBatch
     // but together with the CalculateTopK / CalculateFilteredTopK that follows, without storing its result; GetUnitBuffer and

@@ -40,7 +40,7 @@ NNNetwork::NNNetwork(NNNetworkDescriptor& d, uint32_t batch)
       _errorFunction(d._errorFunction), _mode(Prediction), _bShuffleIndices(d._bShuffleIndices), _pDescriptor(NULL), _bDirty(true),
       _verbose(false), _lanes(2), _lane(0)
 {
-    NNDataSetBase::s_nextLane = 1;   // the first PredictBatch of a network with two lanes runs on the second one
+    NNDataSetBase::s_nextLane = 1;   // the first PredictBatch of a network with several lanes runs on the second one
     // keep the scalar settings (not the weight payloads) for SaveNetCDF round trips
     _pDescriptor = new NNNetworkDescriptor(d);
     _pDescriptor->_vLayerDescriptor.clear();
@@ -515,7 +515,7 @@ NNFloat* NNNetwork::GetUnitBuffer(const string& layer)
     // The reference's callers follow this call with a plain cudaMemcpy or a kernel of their own
     // (utils/NNRecsGenerator.cpp:83, java/src/main/native/com_amazon_dsstne_Dsstne.cpp:366), which the default stream ordered
     // after the forward pass.  The lanes' streams are not ordered against the null stream, so the batch that filled this
-    // buffer is waited for here; a batch in flight on the other lane keeps running.
+    // buffer is waited for here; a batch in flight on another lane keeps running.
     dsxFatal(dsx_sync_lane((int)_lane), "NNNetwork::GetUnitBuffer");
     return itr->second->GetUnitBuffer();
 }

@@ -145,7 +145,7 @@ class Network:
         return scores, idx
 
     def get_topk_previous(self, rows, k=None, layer="Output"):
-        """Results of the batch before the current one (two lanes): waits for that batch only."""
+        """Results of the batch before the current one (two or more lanes): waits for that batch only."""
         k = k or self.p.k
         scores = np.empty((rows, k), dtype=np.float32)
         idx = np.empty((rows, k), dtype=np.uint32)

@@ -251,7 +251,7 @@ int dsx_topk_filtered(const float* in, float* keys, uint32_t* values, uint32_t b
  * alone does not fill the device (at most width / 8192), and at least ceil(width / 262,080) with a filter.  When
  * batch x s x k exceeds 2,097,152 words (only possible with a filter over more than 262,080 columns) the
  * call fails with DSX_EINVAL.  Results are those of dsx_topk_filtered / dsx_topk, bit for bit.  All calls on a GPU share the
- * one array: calls that overlap on one GPU (the two lanes, several threads) race. */
+ * one array: calls that overlap on one GPU (several lanes, several threads) race. */
 int dsx_topk_filtered_static(const float* in, float* keys, uint32_t* values, uint32_t batch, uint32_t width, uint32_t k,
                              uint32_t position, const uint32_t* index, const uint64_t* filter_start, const uint64_t* filter_end,
                              const uint32_t* filter_index, const float* filter_mul);
