@@ -88,6 +88,7 @@ struct SparseZArgs {
     uint32_t act;
     float slope, alpha, lambda;
     uint32_t lpr_log2;   // log2 of lanes per weight row
+    int tile_major;      // blockIdx.x is the column tile and blockIdx.y the row (see launch_sparse_z); otherwise the other way round
 };
 
 // T: storage type of the non-zero values; UNITVAL: every value is exactly 1 (Boolean, unweighted): no multiply;
@@ -100,7 +101,8 @@ __global__ __launch_bounds__(kSparseThreads) void sparse_z_kernel(SparseZArgs a)
     __shared__ float sVal[UNITVAL ? 1 : kSparseChunk];
     __shared__ float sRed[kSparseThreads * VEC];
 
-    const uint32_t b = blockIdx.x;
+    const uint32_t b = a.tile_major ? blockIdx.y : blockIdx.x;
+    const uint32_t tile = a.tile_major ? blockIdx.x : blockIdx.y;
     uint32_t r = a.position + b;
     if (a.index) r = a.index[r];
     const uint64_t start = a.start[r];
@@ -111,7 +113,7 @@ __global__ __launch_bounds__(kSparseThreads) void sparse_z_kernel(SparseZArgs a)
     const uint32_t G = kSparseThreads >> a.lpr_log2;
     const uint32_t g = threadIdx.x >> a.lpr_log2;
     const uint32_t lane = threadIdx.x & (lpr - 1);
-    const uint32_t col = (blockIdx.y * lpr + lane) * VEC;
+    const uint32_t col = (tile * lpr + lane) * VEC;
     const bool active = col < a.stride;
     float* urow = a.unit + (uint64_t)b * a.stride;
 
@@ -203,11 +205,17 @@ static int launch_sparse_z(const SparseZArgs& a0, uint32_t batch)
     };
     int vec = aligned(16) ? 4 : (aligned(8) ? 2 : 1);
     uint32_t lanes_needed = (a.stride + vec - 1) / vec;
-    uint32_t lpr_log2 = 4;   // at least 16 lanes per weight row
-    while ((1u << lpr_log2) < lanes_needed && lpr_log2 < 8) lpr_log2++;
+    // Lanes per weight row: at least 16, at most 64.  A wide layer is cut into column tiles of 64 lanes (256 columns with
+    // 128-bit gathers), each with a workgroup of its own per row whose four lane groups share the row's non-zeros; the tile
+    // is the fastest grid dimension, so consecutive workgroups — which go to consecutive XCDs — are different tiles of one row,
+    // and an XCD's L2 sees one or two column tiles of the weight matrix instead of all of it (27,278 x 1,024 at batch 4,096:
+    // 270 -> 163 us; 38 % of the gathers hit in L2 before).
+    uint32_t lpr_log2 = 4;
+    while ((1u << lpr_log2) < lanes_needed && lpr_log2 < 6) lpr_log2++;
     a.lpr_log2 = lpr_log2;
     uint32_t tiles = (lanes_needed + (1u << lpr_log2) - 1) >> lpr_log2;
-    dim3 grid(batch, tiles);
+    a.tile_major = batch <= 65535;   // (the second grid dimension ends there)
+    dim3 grid = a.tile_major ? dim3(tiles, batch) : dim3(batch, tiles);
     hipStream_t s = ctx().stream;
     switch (vec) {
     case 4: hipLaunchKernelGGL((sparse_z_kernel<T, BOOLEAN, UNITVAL, 4, FUSED>), grid, dim3(kSparseThreads), 0, s, a); break;
