@@ -205,13 +205,14 @@ static int launch_sparse_z(const SparseZArgs& a0, uint32_t batch)
     };
     int vec = aligned(16) ? 4 : (aligned(8) ? 2 : 1);
     uint32_t lanes_needed = (a.stride + vec - 1) / vec;
-    // Lanes per weight row: at least 16, at most 64.  A wide layer is cut into column tiles of 64 lanes (256 columns with
-    // 128-bit gathers), each with a workgroup of its own per row whose four lane groups share the row's non-zeros; the tile
-    // is the fastest grid dimension, so consecutive workgroups — which go to consecutive XCDs — are different tiles of one row,
-    // and an XCD's L2 sees one or two column tiles of the weight matrix instead of all of it (27,278 x 1,024 at batch 4,096:
-    // 270 -> 163 us; 38 % of the gathers hit in L2 before).
+    // Lanes per weight row: at least 16, at most 64, and half a row where that allows it.  The layer is cut into column tiles
+    // that wide (up to 256 columns with 128-bit gathers), each with a workgroup of its own per row whose lane groups share
+    // the row's non-zeros; the tile is the fastest grid dimension, so consecutive workgroups — which go to consecutive XCDs —
+    // are different tiles of one row, and an XCD's L2 sees some column tiles of the weight matrix instead of all of it
+    // (27,278 x 1,024 at batch 4,096: 38 % of the gathers hit in L2 with one tile, 270 -> 163 us with four;
+    // 27,278 x 128 at batch 1,024: 14.6 -> 12.1 us with two).
     uint32_t lpr_log2 = 4;
-    while ((1u << lpr_log2) < lanes_needed && lpr_log2 < 6) lpr_log2++;
+    while ((2u << lpr_log2) < lanes_needed && lpr_log2 < 6) lpr_log2++;
     a.lpr_log2 = lpr_log2;
     uint32_t tiles = (lanes_needed + (1u << lpr_log2) - 1) >> lpr_log2;
     a.tile_major = batch <= 65535;   // (the second grid dimension ends there)
