@@ -10,7 +10,7 @@
 //   * a score enters only if it beats the list's current k-th word; the common case costs three vector instructions per
 //     16-byte group; survivors are compacted with a 64-bit ballot into a per-wave LDS staging area and, once L of them are
 //     waiting, bitonic-sorted (cross-lane exchanges) and merged into the register list, which tightens the threshold;
-//   * for k <= 32 the threshold is primed before the scan from the k-th best of the lanes' first-span maxima (a binary
+//   * for k <= 128 the threshold is primed before the scan from the k-th best of the lanes' first-span maxima (a binary
 //     search over key bits), so a 27k-column row stages about forty words, no wave ever sorts, and the final order comes
 //     from counting, for each staged word, how many staged words are larger;
 //   * the kernel is bound by instruction issue as much as by HBM (four waves per SIMD run the same phases in step), so the
@@ -544,36 +544,49 @@ __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kern
         }
     };
 
-    // Priming (k <= 32): before anything is admitted, every lane takes the best score of its first CH groups.  The k-th
-    // best of a wave's 64 lane maxima is a score that at least k unfiltered items reach, so nothing below it can be in the
+    // Priming (k <= 128): before anything is admitted, every lane takes the best score of either half of its first CH groups.
+    // The k-th best of a wave's 128 maxima is a score that at least k unfiltered items reach, so nothing below it can be in the
     // result; the k-th best of the 4k scores the four waves publish is a bound for the whole workgroup.  It is found by
     // binary search on the key bits (no sorting), and the scan then admits a few dozen items per row instead of a few
     // hundred.  Groups that hold a listed column are left out, and a lane with nothing else contributes -inf, which only
     // weakens the bound.
-    if (R == 1 && a.k <= 32 && g0 < g1) {
-        __shared__ uint32_t sPrime[kTopkWaves][32];
-        float m = -__builtin_inff();
+    if (R <= 2 && g0 < g1) {   // (k <= 128: two maxima per lane give a wavefront at least k values)
+        constexpr int PV = 2;   // maxima per lane, over CH / PV groups each
+        __shared__ uint32_t sPrime[kTopkWaves][PV * kWave];
         uint32_t taint = 0;
         if constexpr (FILTERED) taint = (sTaint[threadIdx.x >> 2] >> ((threadIdx.x & 3) * 8)) & 0xffu;
+        uint32_t key[PV];
 #pragma unroll
-        for (int u = 0; u < CH; u++) {
-            const float gm = fmaxf(fmaxf(cur[u].x, cur[u].y), fmaxf(cur[u].z, cur[u].w));   // fmaxf drops NaN
-            m = fmaxf(m, ((taint >> u) & 1u) ? -__builtin_inff() : gm);
+        for (int v = 0; v < PV; v++) {
+            float m = -__builtin_inff();
+#pragma unroll
+            for (int u = v * (CH / PV); u < (v + 1) * (CH / PV); u++) {
+                const float gm = fmaxf(fmaxf(cur[u].x, cur[u].y), fmaxf(cur[u].z, cur[u].w));   // fmaxf drops NaN
+                m = fmaxf(m, ((taint >> u) & 1u) ? -__builtin_inff() : gm);
+            }
+            key[v] = score_key(m);
         }
-        const uint32_t key[1] = {score_key(m)};
-        const uint32_t tw = wave_kth_key<1>(key, a.k);
-        const bool pub = key[0] >= tw;   // at least k lanes
-        const uint64_t pm = __ballot(pub);
-        const uint32_t pos = __builtin_amdgcn_mbcnt_hi((uint32_t)(pm >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)pm, 0u));
-        if (pub && pos < a.k) sPrime[wave][pos] = key[0];
-        __syncthreads();
-        uint32_t all[2];
+        const uint32_t tw = wave_kth_key<PV>(key, a.k);
+        uint32_t published = 0;   // wave-uniform
 #pragma unroll
-        for (int n = 0; n < 2; n++) {
+        for (int v = 0; v < PV; v++) {
+            const bool pub = key[v] >= tw;   // at least k values of the wavefront
+            const uint64_t pm = __ballot(pub);
+            const uint32_t pos = published + __builtin_amdgcn_mbcnt_hi((uint32_t)(pm >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)pm, 0u));
+            if (pub && pos < a.k) sPrime[wave][pos] = key[v];
+            published += (uint32_t)__popcll(pm);
+        }
+        __syncthreads();
+        uint32_t all[4 * PV];
+#pragma unroll
+        for (int n = 0; n < 4 * PV; n++) {
             const uint32_t i = n * kWave + lane;
             all[n] = (i < kTopkWaves * a.k) ? sPrime[i / a.k][i % a.k] : 0u;
         }
-        const uint32_t t = wave_kth_key<2>(all, a.k);
+        uint32_t t;
+        if (a.k <= 32) t = wave_kth_key<2>(reinterpret_cast<const uint32_t(&)[2]>(all), a.k);
+        else if (a.k <= 64) t = wave_kth_key<4>(reinterpret_cast<const uint32_t(&)[4]>(all), a.k);
+        else t = wave_kth_key<4 * PV>(all, a.k);
         if (t > score_key(-__builtin_inff())) list.prime(t);
     }
 
