@@ -38,13 +38,37 @@ string getOptionalArgValue(int argc, char** argv, string flag, string defaultVal
 
 bool isArgSet(int argc, char** argv, string flag) { return cmdOptionExists(argv, argv + argc, flag); }
 
+vector<string>& split(const string& s, char delim, vector<string>& elems)
+{
+    stringstream ss(s);
+    string item;
+    while (getline(ss, item, delim)) elems.push_back(item);
+    return elems;
+}
+
 vector<string> split(const string& s, char delim)
 {
     vector<string> out;
-    stringstream ss(s);
-    string item;
-    while (getline(ss, item, delim)) out.push_back(item);
+    split(s, delim, out);
     return out;
+}
+
+bool isNetCDFfile(const string& filename)
+{
+    const size_t dot = filename.find_last_of('.');
+    return dot != string::npos && filename.compare(dot, string::npos, NETCDF_FILE_EXTENTION) == 0;
+}
+
+bool isDirectory(const string& dirname)
+{
+    struct stat st;
+    return stat(dirname.c_str(), &st) == 0 && S_ISDIR(st.st_mode);
+}
+
+bool isFile(const string& filename)
+{
+    struct stat st;
+    return stat(filename.c_str(), &st) == 0 && S_ISREG(st.st_mode);
 }
 
 bool fileExists(const string& fileName)

@@ -18,10 +18,6 @@
 
 using namespace std;
 
-static const string INPUT_DATASET_SUFFIX = "_input";
-static const string NETCDF_FILE_EXTENSION = ".nc";
-static const unsigned long FIXED_SEED = 12134ull;
-
 static void printUsagePredict()
 {
     cout << "Predict: Generates predictions from a trained neural network given a signals/input dataset." << endl;
@@ -84,7 +80,7 @@ int main(int argc, char** argv)
     // samples text -> sparse dataset file next to the working directory, named so that training files are not overwritten
     unordered_map<string, unsigned int> mSignals;
     const string dataSetFilesPrefix = dataSetName + "_predict";
-    const string inputNetCDFFileName = dataSetFilesPrefix + NETCDF_FILE_EXTENSION;
+    const string inputNetCDFFileName = dataSetFilesPrefix + NETCDF_FILE_EXTENTION;
     {
         vector<unsigned int> vSparseStart, vSparseEnd, vSparseIndex;
         vector<float> vSparseData;

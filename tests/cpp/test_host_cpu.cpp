@@ -162,6 +162,34 @@ static void testTopKsort()
     CHECK(tvf[0] == 7 && tvf[1] == 5 && tvf[2] == 2);
 }
 
+// The reference's own case (tst/unittests/TestUtils.cpp:10-17) and the helpers beside it.
+static void testUtils(const string& dir)
+{
+    CHECK(isNetCDFfile("network.nc"));
+    CHECK(!isNetCDFfile("network.nic"));
+    CHECK(!isNetCDFfile("network"));
+    CHECK(isNetCDFfile("a.b/net.v2.nc") && !isNetCDFfile("net.nc.bak"));
+    vector<string> parts = {"head"};
+    vector<string>& same = split("a,b,,c", ',', parts);
+    CHECK(&same == &parts && parts.size() == 5 && parts[0] == "head" && parts[3] == "" && parts[4] == "c");
+    CHECK(split("x:y", ':').size() == 2 && split("", ':').empty());
+    const string file = dir + "/utils_probe.txt";
+    FILE* f = fopen(file.c_str(), "w");
+    fputs("x\n", f);
+    fclose(f);
+    CHECK(isDirectory(dir) && !isFile(dir));
+    CHECK(isFile(file) && !isDirectory(file));
+    CHECK(!isFile(dir + "/no_such_entry") && !isDirectory(dir + "/no_such_entry"));
+    for (int i = 0; i < 200; i++) {
+        const int r = rand(3, 5);
+        const float x = rand(-1.0f, 2.0f);
+        CHECK(r >= 3 && r <= 5);
+        CHECK(x >= -1.0f && x <= 2.0f);
+    }
+    CHECK(rand(7, 7) == 7);
+    CHECK(INPUT_DATASET_SUFFIX == "_input" && OUTPUT_DATASET_SUFFIX == "_output" && FIXED_SEED == 12134ul);
+}
+
 static void testKnnHost(const string& dir)
 {
     {
@@ -535,6 +563,7 @@ int main(int argc, char** argv)
     testNetworkFileRoundTrip(dir);
     testFilters(dir);
     testTopKsort();
+    testUtils(dir);
     testKnnHost(dir);
     testLoadIndex();
     testParseSamplesAndDatasetFile(dir);
