@@ -19,6 +19,7 @@
 //     listed columns are dropped from the scan and injected once, after the scan, with score * multiplier;
 //   * rows split over several segments write packed partial lists that a second small kernel merges.
 #include <algorithm>
+#include <type_traits>
 #include "dsx_device.h"
 #include "dsx_internal.h"
 
@@ -324,22 +325,24 @@ __device__ __forceinline__ void finish_row(WaveTopK<R>& list, uint64_t (*sStage)
     // already sit in LDS); a wave with a register list flushes what is left and publishes its first k words.
     __shared__ uint32_t sPublished[kTopkWaves];
     __shared__ uint32_t sFlushed[kTopkWaves];
-    if (wave != 0) {
-        if (list.flushed) {
-            list.finish();
+    __shared__ uint32_t sPlace[2 * kWave];
+    if (wave != 0 && list.flushed) {
+        list.finish();
 #pragma unroll
-            for (int r = 0; r < R; r++) {
-                const uint32_t p = r * kWave + lane;
-                if (p < a.k) sStage[wave][p] = list.q[r];
-            }
-        }
-        if (lane == 0) {
-            sPublished[wave] = list.flushed ? a.k : list.count;
-            sFlushed[wave] = list.flushed ? 1u : 0u;
+        for (int r = 0; r < R; r++) {
+            const uint32_t p = r * kWave + lane;
+            if (p < a.k) sStage[wave][p] = list.q[r];
         }
     }
+    if (lane == 0) {
+        sPublished[wave] = (wave != 0 && list.flushed) ? a.k : list.count;
+        sFlushed[wave] = list.flushed ? 1u : 0u;
+    }
+    if (wave == 1) {
+        sPlace[lane] = 0;
+        sPlace[kWave + lane] = 0;
+    }
     __syncthreads();
-    if (wave != 0) return;
 
     uint64_t* partial = a.partial ? a.partial + ((uint64_t)b * a.partial_slots + a.partial_slot0 + seg) * a.k : nullptr;
     float* keys = a.keys + (uint64_t)b * a.k;
@@ -360,34 +363,39 @@ __device__ __forceinline__ void finish_row(WaveTopK<R>& list, uint64_t (*sStage)
         }
     };
 
-    const uint32_t n0 = list.count, n1 = sPublished[1], n2 = sPublished[2], n3 = sPublished[3];
+    const uint32_t n0 = sPublished[0], n1 = sPublished[1], n2 = sPublished[2], n3 = sPublished[3];
     const uint32_t total = n0 + n1 + n2 + n3;
-    const bool any_flushed = list.flushed || (sFlushed[1] | sFlushed[2] | sFlushed[3]) != 0;
+    const bool any_flushed = (sFlushed[0] | sFlushed[1] | sFlushed[2] | sFlushed[3]) != 0;   // the same for every wave
     if (!any_flushed && total <= 2 * kWave) {
-        // Common case for small k: at most 128 staged words in all.  Lane i takes the i-th (and the 64 + i-th) of them and
-        // counts how many are larger; that count is its place in the result, so no sorting network runs at all.
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
+        // Common case for small k: at most 128 staged words in all.  Lane i takes the i-th (and the 64 + i-th) of them; the
+        // number of staged words that are larger is its place in the result, so no sorting network runs at all.  The
+        // counting is shared: every wave compares all words with its own staged ones and adds its count in LDS.
         auto fetch = [&](uint32_t i) -> uint64_t {
             if (i >= total) return 0ull;   // never larger than anything
             const uint32_t w = (i >= n0) + (i >= n0 + n1) + (i >= n0 + n1 + n2);
             const uint32_t first = (w == 0) ? 0 : (w == 1) ? n0 : (w == 2) ? n0 + n1 : n0 + n1 + n2;
             return sStage[w][i - first];
         };
-        const bool two = total > kWave;   // wave-uniform
+        const bool two = total > kWave;   // workgroup-uniform
         const uint64_t word0 = fetch(lane), word1 = two ? fetch(kWave + lane) : 0ull;
-        // all words side by side in LDS (wave 0's own staging area is free once its words sit in registers)
-        __builtin_amdgcn_wave_barrier();
-        sStage[0][lane] = word0;
-        sStage[0][kWave + lane] = word1;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        uint32_t place0 = 0, place1 = 0;
-        for (uint32_t i = 0; i < total; i += 4) {   // broadcast reads, four in flight; the row has room beyond 128 + 3
-            const uint64_t o0 = sStage[0][i], o1 = sStage[0][i + 1], o2 = sStage[0][i + 2], o3 = sStage[0][i + 3];
-            place0 += (o0 > word0 ? 1u : 0u) + (o1 > word0 ? 1u : 0u) + (o2 > word0 ? 1u : 0u) + (o3 > word0 ? 1u : 0u);
-            if (two) place1 += (o0 > word1 ? 1u : 0u) + (o1 > word1 ? 1u : 0u) + (o2 > word1 ? 1u : 0u) + (o3 > word1 ? 1u : 0u);
+        const uint32_t mine = sPublished[wave];
+        uint32_t part0 = 0, part1 = 0;
+        for (uint32_t i = 0; i < mine; i += 4) {   // broadcast reads, four in flight (a staging row has room beyond any count)
+            uint64_t o[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) o[u] = sStage[wave][i + u];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                if (i + u >= mine) o[u] = 0ull;   // stale words beyond the count
+                part0 += (o[u] > word0) ? 1u : 0u;
+                if (two) part1 += (o[u] > word1) ? 1u : 0u;
+            }
         }
+        if (part0 != 0) atomicAdd(&sPlace[lane], part0);
+        if (part1 != 0) atomicAdd(&sPlace[kWave + lane], part1);
+        __syncthreads();
+        if (wave != 0) return;
+        const uint32_t place0 = sPlace[lane], place1 = sPlace[kWave + lane];
         if (word0 != 0 && place0 < a.k) write_slot(place0, word0);
         if (word1 != 0 && place1 < a.k) write_slot(place1, word1);
         for (uint32_t p = total + lane; p < a.k; p += kWave) write_slot(p, 0ull);
@@ -397,6 +405,7 @@ __device__ __forceinline__ void finish_row(WaveTopK<R>& list, uint64_t (*sStage)
         }
         return;
     }
+    if (wave != 0) return;
 
     for (uint32_t w = 1; w < kTopkWaves; w++) {
         const uint32_t n = sPublished[w];
@@ -494,7 +503,7 @@ __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kern
     // second span: waiting for them then costs no more than waiting for the first span, which priming needs anyway, and the
     // listed scores (requested last) are not waited for until the scan is over.
     constexpr int kFU = 4;
-    __shared__ uint32_t sTaint[kTopkThreads / 4];   // one byte per lane: bit u = group u of the first span holds a listed column
+    __shared__ uint32_t sTaint[kTopkThreads / 2];   // 16 bits per lane: bit u = group u of the first two spans holds a listed column
     uint32_t fcol[kFU];
     float fm[kFU], fv[kFU];
     if constexpr (FILTERED) {
@@ -513,14 +522,14 @@ __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kern
     if constexpr (FILTERED) {
         const uint32_t words = (hi - lo + 31) / 32;
         for (uint32_t i = threadIdx.x; i < words; i += kTopkThreads) sBitmap[i] = 0;
-        if (threadIdx.x < kTopkThreads / 4) sTaint[threadIdx.x] = 0;
+        if (threadIdx.x < kTopkThreads / 2) sTaint[threadIdx.x] = 0;
         __syncthreads();
         auto mark = [&](uint32_t c) {
             if (c >= lo && c < hi) {
                 atomicOr(&sBitmap[(c - lo) >> 5], 1u << ((c - lo) & 31));
                 if (c >= head && c < tail0) {
                     const uint32_t gi = (c - head) / 4 - g0;
-                    if (gi < CH * step) atomicOr(&sTaint[(gi % step) >> 2], 1u << (((gi % step) & 3) * 8 + gi / step));
+                    if (gi < 2 * CH * step) atomicOr(&sTaint[(gi % step) >> 1], 1u << (((gi % step) & 1) * 16 + gi / step));
                 }
             }
         };
@@ -544,25 +553,29 @@ __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kern
         }
     };
 
-    // Priming (k <= 128): before anything is admitted, every lane takes the best score of either half of its first CH groups.
+    // Priming (k <= 128): before anything is admitted, every lane takes the best score of its groups in each of the first two spans.
     // The k-th best of a wave's 128 maxima is a score that at least k unfiltered items reach, so nothing below it can be in the
     // result; the k-th best of the 4k scores the four waves publish is a bound for the whole workgroup.  It is found by
     // binary search on the key bits (no sorting), and the scan then admits a few dozen items per row instead of a few
     // hundred.  Groups that hold a listed column are left out, and a lane with nothing else contributes -inf, which only
     // weakens the bound.
-    if (R <= 2 && g0 < g1) {   // (k <= 128: two maxima per lane give a wavefront at least k values)
-        constexpr int PV = 2;   // maxima per lane, over CH / PV groups each
-        __shared__ uint32_t sPrime[kTopkWaves][PV * kWave];
+    // The two maxima of a lane are those of its groups in the first and in the second span: together the first 2 * CH * 4 KiB of
+    // the segment, 60 % of a 27,278-column row.  (A bound from the first span alone admits twice as many items on average
+    // and, in the unlucky row of a large batch, ten times as many: the slowest row sets the kernel's time.)
+    __shared__ uint32_t sPrime[kTopkWaves][2 * kWave];
+    auto prime_from_first_spans = [&]() {
+        constexpr int PV = 2;
         uint32_t taint = 0;
-        if constexpr (FILTERED) taint = (sTaint[threadIdx.x >> 2] >> ((threadIdx.x & 3) * 8)) & 0xffu;
+        if constexpr (FILTERED) taint = (sTaint[threadIdx.x >> 1] >> ((threadIdx.x & 1) * 16)) & 0xffffu;
         uint32_t key[PV];
 #pragma unroll
         for (int v = 0; v < PV; v++) {
             float m = -__builtin_inff();
 #pragma unroll
-            for (int u = v * (CH / PV); u < (v + 1) * (CH / PV); u++) {
-                const float gm = fmaxf(fmaxf(cur[u].x, cur[u].y), fmaxf(cur[u].z, cur[u].w));   // fmaxf drops NaN
-                m = fmaxf(m, ((taint >> u) & 1u) ? -__builtin_inff() : gm);
+            for (int u = 0; u < CH; u++) {
+                const float4& g = (v == 0) ? cur[u] : nxt[u];
+                const float gm = fmaxf(fmaxf(g.x, g.y), fmaxf(g.z, g.w));   // fmaxf drops NaN
+                m = fmaxf(m, ((taint >> (v * CH + u)) & 1u) ? -__builtin_inff() : gm);
             }
             key[v] = score_key(m);
         }
@@ -577,18 +590,20 @@ __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kern
             published += (uint32_t)__popcll(pm);
         }
         __syncthreads();
-        uint32_t all[4 * PV];
+        uint32_t all[4 * PV];   // the 4k published keys, side by side
 #pragma unroll
         for (int n = 0; n < 4 * PV; n++) {
             const uint32_t i = n * kWave + lane;
             all[n] = (i < kTopkWaves * a.k) ? sPrime[i / a.k][i % a.k] : 0u;
         }
         uint32_t t;
-        if (a.k <= 32) t = wave_kth_key<2>(reinterpret_cast<const uint32_t(&)[2]>(all), a.k);
+        if (a.k <= 16) t = wave_kth_key<1>(reinterpret_cast<const uint32_t(&)[1]>(all), a.k);
+        else if (a.k <= 32) t = wave_kth_key<2>(reinterpret_cast<const uint32_t(&)[2]>(all), a.k);
         else if (a.k <= 64) t = wave_kth_key<4>(reinterpret_cast<const uint32_t(&)[4]>(all), a.k);
         else t = wave_kth_key<4 * PV>(all, a.k);
         if (t > score_key(-__builtin_inff())) list.prime(t);
-    }
+    };
+    if (R <= 2 && g0 < g1) prime_from_first_spans();   // (k <= 128)
 
     // The four scores of one 16-byte group; at most 4 * 64 words are staged.
     auto stage_group = [&](const float4& v, uint32_t col) {
