@@ -222,7 +222,7 @@ int dsx_knn_last_search_path(void) { return g_knn_last_path; }
 
 int dsx_knn_f16_set_sweep(int mode)
 {
-    DSX_CHECK_ARG(mode >= 0 && mode <= 2, "dsx_knn_f16_set_sweep: mode %d (0, 1 or 2)", mode);
+    DSX_CHECK_ARG(mode >= 0 && mode <= 3, "dsx_knn_f16_set_sweep: mode %d (0 to 3)", mode);
     g_knn_f16_sweep = mode;
     return DSX_OK;
 }

@@ -336,6 +336,180 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         a.seg_count[(uint64_t)(row0 + tid) * kSweepCountStride + chunk] = min(row_state(tid)[0], a.seg_cap);
 }
 
+// Candidate mode for long column ranges when the vectors have at most 256 components: the queries live in registers.
+// A wavefront keeps the operand fragments of its 64 queries for every k-step (KS * 8 registers), so the only operand that
+// moves during the sweep is the item: 64 items per stage, whole rows, staged in LDS once per workgroup of eight wavefronts
+// (512 queries) and read from there as the other MFMA operand — one 128-bit LDS read feeds two multiplications, where
+// knn_f16_sweep_kernel needs one read each, and a CU pulls in a quarter of the item bytes per multiplication.  The items are
+// the row operand, so a lane's sixteen results of a multiplication are sixteen items of ONE query: its bound is one register
+// and a few maxima and one compare are all a block without survivors costs.  The lists have the layout knn_f16_sweep_kernel
+// fills, with two lists per (query, chunk) — one for each of the two lanes that hold items of that query — whose fill counts
+// are registers; a full list spills into the query's shared list.  One workgroup per CU: two wavefronts per SIMD with 256
+// registers each.
+template <int KS>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void knn_f16_wide_kernel(KnnF16SweepArgs a)
+{
+    constexpr int BQ = 512, BI = 64, LD = KS * 16, PITCH = LD + 8, THREADS = 512;
+    constexpr int PIECES = BI * (LD / 8) / THREADS;   // 16-byte pieces of a stage per lane
+    static_assert(BI * (LD / 8) % THREADS == 0, "a stage is a whole number of 16-byte pieces per lane");
+    extern __shared__ __attribute__((aligned(16))) unsigned char wide_lds[];
+    typedef _Float16 (*StagePtr)[BI][PITCH];
+    StagePtr sI = reinterpret_cast<StagePtr>(wide_lds);   // two stages of items
+
+    // Workgroups that sweep the same chunk sit on the same XCD: an item stage comes from HBM once and from that XCD's L2 for
+    // the others.
+    const uint32_t total = a.tiles_m * a.chunks;
+    uint32_t wg = blockIdx.x;
+    {
+        const uint32_t per_xcd = (total + kF16Xcds - 1) / kF16Xcds;
+        const uint32_t xcd = wg % kF16Xcds, local = wg / kF16Xcds;
+        wg = xcd * per_xcd + local;
+        if (local >= per_xcd || wg >= total) return;
+    }
+    const uint32_t tm = wg % a.tiles_m, chunk = wg / a.tiles_m;
+    const uint32_t row0 = tm * BQ;
+    const uint32_t s0 = chunk * a.tiles_per_chunk;                 // stages of BI items
+    const uint32_t s1 = min(s0 + a.tiles_per_chunk, a.tiles_n);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, lhi = lane >> 5;
+    if (s0 >= s1) {   // more chunks than stages: two empty lists per query
+        if (row0 + tid < a.batch) {
+            a.seg_count[(uint64_t)(row0 + tid) * kSweepCountStride + 2 * chunk] = 0;
+            a.seg_count[(uint64_t)(row0 + tid) * kSweepCountStride + 2 * chunk + 1] = 0;
+        }
+        return;
+    }
+
+    // this lane's two queries: operand fragments for all k-steps, and their bounds (key 0: no bound yet, every number passes)
+    const uint32_t rows_stored = (a.batch + 255) / 256 * 256;   // rows the query array holds (zero filled beyond the batch)
+    uint32_t q[2];
+    uint64_t* my_seg[2];   // list (query, 2 * chunk + lhi) of seg_cap words
+    half8 bq[2][KS];
+    float bound[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        q[h] = row0 + wave * 64 + h * 32 + l32;
+        my_seg[h] = a.seg + ((uint64_t)q[h] * (2 * a.chunks) + 2 * chunk + lhi) * a.seg_cap;
+        const _Float16* qp = a.A + (uint64_t)min(q[h], rows_stored - 1) * LD + lhi * 8;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) bq[h][ks] = *reinterpret_cast<const half8*>(qp + ks * 16);
+        bound[h] = __builtin_inff();   // queries beyond the batch admit nothing
+        if (q[h] < a.batch) {
+            const uint32_t key = a.cand.row_bound[q[h]];
+            bound[h] = key ? key_score(key) : -__builtin_inff();
+        }
+    }
+
+    // A stage is BI whole rows: one contiguous piece of the table.
+    const uint4* gI = reinterpret_cast<const uint4*>(a.B + (uint64_t)s0 * BI * LD) + tid;
+    // (named registers, not an array: an array that a conditional load fills ends up in scratch memory)
+    uint4 st0 = {}, st1 = {}, st2 = {}, st3 = {};
+    static_assert(PIECES >= 1 && PIECES <= 4, "one to four pieces per lane");
+    auto load_stage = [&]() __attribute__((always_inline)) {
+        st0 = gI[0];
+        if constexpr (PIECES > 1) st1 = gI[THREADS];
+        if constexpr (PIECES > 2) st2 = gI[2 * THREADS];
+        if constexpr (PIECES > 3) st3 = gI[3 * THREADS];
+        gI += BI * (LD / 8);
+    };
+    auto store_piece = [&](int buf, int j, const uint4& v) __attribute__((always_inline)) {
+        const int p = tid + j * THREADS;
+        *reinterpret_cast<uint4*>(&sI[buf][p / (LD / 8)][(p % (LD / 8)) * 8]) = v;
+    };
+    auto store_stage = [&](int buf) __attribute__((always_inline)) {
+        store_piece(buf, 0, st0);
+        if constexpr (PIECES > 1) store_piece(buf, 1, st1);
+        if constexpr (PIECES > 2) store_piece(buf, 2, st2);
+        if constexpr (PIECES > 3) store_piece(buf, 3, st3);
+    };
+    // The 32 x 32 scores of one query block against one item block.  A lane holds sixteen items of one query, and the two
+    // lanes that share a query (rows 4 * lhi + ...) each own a list of their own — (query, 2 * chunk + lhi) — so a
+    // survivor costs a store and a register increment, no atomic.  The largest of the sixteen first (three-way maxima by
+    // groups of four), then only the groups and scores that reach the bound.
+    uint32_t fill[2] = {0, 0};
+    auto compare = [&](const floatx16& acc, int h, uint32_t item0) __attribute__((always_inline)) {
+        float gm[4];
+#pragma unroll
+        for (int g = 0; g < 4; g++) gm[g] = fmaxf(fmaxf(fmaxf(acc[4 * g], acc[4 * g + 1]), acc[4 * g + 2]), acc[4 * g + 3]);
+        const float top = fmaxf(fmaxf(fmaxf(gm[0], gm[1]), gm[2]), gm[3]);
+        if (__builtin_amdgcn_ballot_w64(top >= bound[h]) == 0) return;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            if (__builtin_amdgcn_ballot_w64(gm[g] >= bound[h]) == 0) continue;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float x = acc[4 * g + e];
+                asm volatile("" : "+v"(x));
+                const uint32_t col = item0 + 8 * g + e;
+                if (x >= bound[h] && col < a.n) {   // (items beyond the range are zero padding)
+                    const uint64_t word = ((uint64_t)score_key(x) << 32) | (uint32_t)~(a.cand.col_offset + col);
+                    if (fill[h] < a.seg_cap) {
+                        my_seg[h][fill[h]] = word;
+                    } else {   // this list is full: the query's shared list
+                        const uint32_t p2 = atomicAdd(&a.cand.cand_count[q[h]], 1u);
+                        if (p2 < a.cand.cand_cap) a.cand.cand[(uint64_t)q[h] * a.cand.cand_cap + p2] = word;
+                        else *a.cand.overflow = 1u;
+                    }
+                    fill[h]++;
+                }
+            }
+        }
+    };
+
+    load_stage();
+    store_stage(0);
+    __syncthreads();
+    for (uint32_t s = s0; s < s1; s++) {
+        const int buf = (int)((s - s0) & 1u);
+        const bool more = s + 1 < s1;
+        if (more) load_stage();
+        // The item fragment of step ks + AHEAD is requested before step ks multiplies, so that the LDS latency is paid once per
+        // item block and not once per step.
+        constexpr int AHEAD = (KS < 6) ? KS : 6, RING = 8;
+#pragma unroll 1
+        for (int sub = 0; sub < BI / 32; sub++) {
+            const _Float16* ip = &sI[buf][sub * 32 + l32][lhi * 8];
+            half8 av[RING];
+#pragma unroll
+            for (int t = 0; t < AHEAD; t++) av[t % RING] = *reinterpret_cast<const half8*>(ip + t * 16);
+            __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);   // the first AHEAD reads,
+            floatx16 acc0, acc1;
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc0[v] = acc1[v] = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                if (ks + AHEAD < KS) av[(ks + AHEAD) % RING] = *reinterpret_cast<const half8*>(ip + (ks + AHEAD) * 16);
+                acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[ks % RING], bq[0][ks], acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[ks % RING], bq[1][ks], acc1, 0, 0, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                        // then two multiplications
+                if (ks + AHEAD < KS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // and one more read, in turn
+            }
+            const uint32_t item0 = s * BI + sub * 32 + 4 * lhi;
+            compare(acc0, 0, item0);
+            compare(acc1, 1, item0);
+        }
+        if (more) store_stage(buf ^ 1);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+        if (q[h] < a.batch) a.seg_count[(uint64_t)q[h] * kSweepCountStride + 2 * chunk + lhi] = min(fill[h], a.seg_cap);
+}
+
+template <int KS> static int launch_wide(const KnnF16SweepArgs& a, uint32_t grid)
+{
+    constexpr size_t lds = 2 * 64 * (KS * 16 + 8) * sizeof(_Float16);
+    static bool sized[64] = {};   // per device: the kernel's LDS limit is raised once
+    const int dev = ctx().device;
+    if (dev < 0 || dev >= 64 || !sized[dev]) {
+        DSX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&knn_f16_wide_kernel<KS>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        if (dev >= 0 && dev < 64) sized[dev] = true;
+    }
+    hipLaunchKernelGGL((knn_f16_wide_kernel<KS>), dim3(grid), dim3(512), lds, ctx().stream, a);
+    DSX_LAUNCH_CHECK("knn_f16_wide_kernel");
+    return DSX_OK;
+}
+
 // fp32 -> fp16, round to nearest even (__float2half), into the padded row-major layout.  src is either column-major
 // (items: src[d * src_ld + row]) or row-major (queries: src[row * src_ld + d]); rows >= rows_valid and components >= dim
 // become zero.  One lane per 8 output halves.
@@ -420,32 +594,54 @@ int knn_f16_scores_run(const void* queries16, const void* items16, uint32_t ld, 
 }
 
 // Candidate mode of a column range of n items for `batch` queries.  mode 0: one workgroup per tile (knn_f16_kernel); 1: a
-// sweep (knn_f16_sweep_kernel) when it has workgroups for every CU and at least four tiles per chunk; 2: a sweep whenever every
-// chunk gets a tile (tests at small sizes).  *chunks_used: the chunks of the sweep, 0 when the range went through
-// knn_f16_kernel and only the shared lists were appended to.
+// sweep when it has workgroups for (half of) the CUs and enough items per chunk — knn_f16_wide_kernel for vectors of at most 256
+// components, knn_f16_sweep_kernel otherwise; 2: knn_f16_sweep_kernel whenever every chunk gets a tile, 3: knn_f16_wide_kernel
+// whenever every chunk gets a stage (tests at small sizes).  *chunks_used: the chunks of the sweep, 0 when the range went
+// through knn_f16_kernel and only the shared lists were appended to.
 int knn_f16_candidates_run(const void* queries16, const void* items16, uint32_t ld, uint32_t batch, uint32_t n, const CandArgs& cand,
                            uint64_t* seg, uint32_t* seg_count, uint32_t seg_words, int mode, uint32_t* chunks_used)
 {
     *chunks_used = 0;
     const uint32_t cus = (uint32_t)ctx().num_cus;
-    const uint32_t tiles_m = (batch + 127) / 128, tiles_n = (n + 127) / 128;
-    const uint32_t chunks = std::min<uint32_t>(kSweepCountStride, (4 * cus + tiles_m - 1) / tiles_m);   // every CU four times over
-    const bool sweep = seg && seg_count && (mode == 2 ? tiles_n >= chunks : (mode == 1 && tiles_m * chunks >= 2 * cus && tiles_n >= 4 * chunks));
-    if (!sweep) return knn_f16_scores_run(queries16, items16, ld, batch, n, nullptr, 0, &cand);
     KnnF16SweepArgs a{};
     a.A = (const _Float16*)queries16;
     a.B = (const _Float16*)items16;
     a.ld = ld;
     a.batch = batch;
     a.n = n;
+    a.seg = seg;
+    a.seg_count = seg_count;
+    a.cand = cand;
+    if (seg && seg_count && ld <= 256 && (mode == 1 || mode == 3)) {
+        // queries in registers: 512 per workgroup, stages of 64 items, one workgroup per CU
+        const uint32_t tiles_q = (batch + 511) / 512, stages = (n + 63) / 64;
+        const uint32_t chunks = std::min<uint32_t>(kSweepCountStride / 2, (cus + tiles_q - 1) / tiles_q);   // two lists per (query, chunk)
+        if (mode == 3 ? stages >= chunks : (2 * tiles_q * chunks >= cus && stages >= 8 * chunks)) {
+            a.tiles_m = tiles_q;
+            a.tiles_n = stages;
+            a.chunks = chunks;
+            a.tiles_per_chunk = (stages + chunks - 1) / chunks;
+            a.seg_cap = seg_words / (2 * chunks);
+            const uint32_t total = tiles_q * chunks;
+            const uint32_t grid = ((total + kF16Xcds - 1) / kF16Xcds) * kF16Xcds;
+            *chunks_used = 2 * chunks;
+            switch (ld) {
+            case 64: return launch_wide<4>(a, grid);
+            case 128: return launch_wide<8>(a, grid);
+            case 192: return launch_wide<12>(a, grid);
+            default: return launch_wide<16>(a, grid);
+            }
+        }
+    }
+    const uint32_t tiles_m = (batch + 127) / 128, tiles_n = (n + 127) / 128;
+    const uint32_t chunks = std::min<uint32_t>(kSweepCountStride, (4 * cus + tiles_m - 1) / tiles_m);   // every CU four times over
+    const bool sweep = seg && seg_count && (mode == 2 || mode == 3 ? tiles_n >= chunks : (mode == 1 && tiles_m * chunks >= 2 * cus && tiles_n >= 4 * chunks));
+    if (!sweep) return knn_f16_scores_run(queries16, items16, ld, batch, n, nullptr, 0, &cand);
     a.tiles_m = tiles_m;
     a.tiles_n = tiles_n;
     a.chunks = chunks;
     a.tiles_per_chunk = (tiles_n + chunks - 1) / chunks;
-    a.seg = seg;
-    a.seg_count = seg_count;
     a.seg_cap = seg_words / chunks;
-    a.cand = cand;
     const uint32_t total = a.tiles_m * a.chunks;
     const uint32_t grid = ((total + kF16Xcds - 1) / kF16Xcds) * kF16Xcds;
     hipLaunchKernelGGL(knn_f16_sweep_kernel, dim3(grid), dim3(256), 0, ctx().stream, a);

@@ -404,7 +404,7 @@ def knn_bench(args, pkg, lib):
     ms16 = (time.perf_counter() - t0) * 1e3 / args.steps
     step16(el)
     f16 = {"ms_per_step": round(ms16, 4), "value": round(Q / (ms16 / 1e3), 1), "unit": "queries/s", "dtype": "f16 operands, f32 sums",
-           "kernel": "knn_f16_sweep_kernel (+ knn_f16_kernel for the first block)", "bound": "mfma", "achieved": round(flops / el[0] / 1e9, 3), "peak": 2500.0, "unit_roofline": "TFLOP/s",
+           "kernel": "knn_f16_wide_kernel (+ knn_f16_kernel for the first block)", "bound": "mfma", "achieved": round(flops / el[0] / 1e9, 3), "peak": 2500.0, "unit_roofline": "TFLOP/s",
            "frac": round(flops / el[0] / 1e9 / 2500.0, 4), "scores_ms": round(el[0], 4), "topk_ms": round(el[1], 4),
            "path": {0: "blocks", 1: "candidate lists", 2: "candidate lists, redone block by block"}[lib.dsx_knn_last_search_path()]}
     cpu = None

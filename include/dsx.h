@@ -324,8 +324,10 @@ int dsx_knn_set_block_columns(uint32_t columns);
 int dsx_knn_last_search_path(void);
 /* No counterpart in the reference: how dsx_knn_search_f16 scores the column ranges after the first block.  1 (default): a
  * range with enough item tiles is swept by workgroups that keep their queries and walk a chunk of the range each (private
- * candidate lists, no atomics on device memory); 0: always one workgroup per tile; 2: sweep every range that has at least one
- * tile per chunk (for tests at small sizes).  The results are the same in every mode. */
+ * candidate lists, no atomics on device memory) — with the queries held in registers when the vectors have at most 256
+ * components, 128 queries per workgroup staged through LDS otherwise; 0: always one workgroup per tile; 2 and 3: the LDS sweep
+ * and the register sweep for every range that has at least one tile per chunk (for tests at small sizes).  The results are
+ * the same in every mode. */
 int dsx_knn_f16_set_sweep(int mode);
 
 #ifdef __cplusplus

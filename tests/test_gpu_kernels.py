@@ -751,11 +751,13 @@ def knn_case_f16(pkg, dsx, orc, items_m, queries_m, k):
 
 
 # sweep 0: one workgroup per tile of scores; 2: column ranges with at least a tile per chunk go through knn_f16_sweep_kernel
-# (with these few queries that is 64 chunks per row tile, so ranges from 8,192 columns on)
-@pytest.mark.parametrize("sweep", [0, 2])
+# (with these few queries that is 64 chunks per row tile, so ranges from 8,192 columns on); 3: through knn_f16_wide_kernel
+# (queries in registers; ranges from 4,096 columns on; 192 components is the one register layout the other cases leave out)
+@pytest.mark.parametrize("sweep", [0, 2, 3])
 @pytest.mark.parametrize("items,queries,dim,k,blocks", [(1003, 9, 24, 10, 0), (50000, 64, 256, 100, 0), (30011, 70, 64, 100, 1024),
                                                           (9000, 130, 250, 10, 1024), (26000, 33, 32, 200, 1024),
-                                                          (70001, 300, 100, 100, 2048), (60000, 520, 256, 50, 2048)])
+                                                          (70001, 300, 100, 100, 2048), (60000, 520, 256, 50, 2048),
+                                                          (20000, 600, 180, 20, 1024)])
 def test_knn_search_f16(pkg, dsx, orc, synth, items, queries, dim, k, blocks, sweep):
     say("knn fp16 items=%d queries=%d dim=%d k=%d first block=%d sweep=%d" % (items, queries, dim, k, blocks, sweep))
     p = synth.knn_config(seed=21, items=items, queries=queries, dim=dim, k=k)
@@ -777,8 +779,9 @@ def test_knn_search_f16(pkg, dsx, orc, synth, items, queries, dim, k, blocks, sw
     assert (np.diff(got_s, axis=1) <= 0).all()
 
 
+@pytest.mark.parametrize("sweep", [2, 3])
 @pytest.mark.parametrize("dim", [64, 128])
-def test_knn_search_f16_sweep_spills_clustered_items(pkg, dsx, orc, rng, dim):
+def test_knn_search_f16_sweep_spills_clustered_items(pkg, dsx, orc, rng, dim, sweep):
     """300 neighbouring items that all beat a query's bound land in two or three chunks of a sweep, whose lists hold 64 words
     each: the rest goes to the query's shared list, nothing is lost and the search is not redone."""
     items, queries, k = 40000, 70, 100
@@ -788,7 +791,7 @@ def test_knn_search_f16_sweep_spills_clustered_items(pkg, dsx, orc, rng, dim):
     for j in range(300):
         it[21000 + j] = u * (40.0 + 0.25 * j)   # far above anything else for query 5, all different
     dsx.dsx_knn_set_block_columns(1024)
-    pkg.check(dsx.dsx_knn_f16_set_sweep(2))
+    pkg.check(dsx.dsx_knn_f16_set_sweep(sweep))
     try:
         got_s, got_i, ref_s, ref_i, it16, q16, _ = knn_case_f16(pkg, dsx, orc, it, q, k)
         assert dsx.dsx_knn_last_search_path() == 1
@@ -821,7 +824,7 @@ def test_knn_f16_table_layout_and_rounding(pkg, dsx, rng):
     assert (t[items:] == 0).all() and (t[:, dim:] == 0).all()
 
 
-@pytest.mark.parametrize("sweep,dim", [(0, 16), (2, 16), (2, 128)])
+@pytest.mark.parametrize("sweep,dim", [(0, 16), (2, 16), (2, 128), (3, 16), (3, 128), (3, 250)])
 def test_knn_search_f16_exact_ties_and_full_lists(pkg, dsx, orc, rng, sweep, dim):
     """Small integers are exact in fp16 too: bit-identical to the oracle, including the query whose candidates all tie (with
     the sweep: its 64-word lists per chunk fill up and spill into the shared list, which fills up as well)."""
