@@ -346,10 +346,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 // fills, with two lists per (query, chunk) — one for each of the two lanes that hold items of that query — whose fill counts
 // are registers; a full list spills into the query's shared list.  One workgroup per CU: two wavefronts per SIMD with 256
 // registers each.
+constexpr int kWideStageItems = 128;
 template <int KS>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void knn_f16_wide_kernel(KnnF16SweepArgs a)
 {
-    constexpr int BQ = 512, BI = 64, LD = KS * 16, PITCH = LD + 8, THREADS = 512;
+    constexpr int BQ = 512, BI = kWideStageItems, LD = KS * 16, PITCH = LD + 8, THREADS = 512;
     constexpr int PIECES = BI * (LD / 8) / THREADS;   // 16-byte pieces of a stage per lane
     static_assert(BI * (LD / 8) % THREADS == 0, "a stage is a whole number of 16-byte pieces per lane");
     extern __shared__ __attribute__((aligned(16))) unsigned char wide_lds[];
@@ -403,13 +404,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // A stage is BI whole rows: one contiguous piece of the table.
     const uint4* gI = reinterpret_cast<const uint4*>(a.B + (uint64_t)s0 * BI * LD) + tid;
     // (named registers, not an array: an array that a conditional load fills ends up in scratch memory)
-    uint4 st0 = {}, st1 = {}, st2 = {}, st3 = {};
-    static_assert(PIECES >= 1 && PIECES <= 4, "one to four pieces per lane");
+    uint4 st0 = {}, st1 = {}, st2 = {}, st3 = {}, st4 = {}, st5 = {}, st6 = {}, st7 = {};
+    static_assert(PIECES >= 1 && PIECES <= 8, "one to eight pieces per lane");
     auto load_stage = [&]() __attribute__((always_inline)) {
         st0 = gI[0];
         if constexpr (PIECES > 1) st1 = gI[THREADS];
         if constexpr (PIECES > 2) st2 = gI[2 * THREADS];
         if constexpr (PIECES > 3) st3 = gI[3 * THREADS];
+        if constexpr (PIECES > 4) st4 = gI[4 * THREADS];
+        if constexpr (PIECES > 5) st5 = gI[5 * THREADS];
+        if constexpr (PIECES > 6) st6 = gI[6 * THREADS];
+        if constexpr (PIECES > 7) st7 = gI[7 * THREADS];
         gI += BI * (LD / 8);
     };
     auto store_piece = [&](int buf, int j, const uint4& v) __attribute__((always_inline)) {
@@ -421,6 +426,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if constexpr (PIECES > 1) store_piece(buf, 1, st1);
         if constexpr (PIECES > 2) store_piece(buf, 2, st2);
         if constexpr (PIECES > 3) store_piece(buf, 3, st3);
+        if constexpr (PIECES > 4) store_piece(buf, 4, st4);
+        if constexpr (PIECES > 5) store_piece(buf, 5, st5);
+        if constexpr (PIECES > 6) store_piece(buf, 6, st6);
+        if constexpr (PIECES > 7) store_piece(buf, 7, st7);
     };
     // The 32 x 32 scores of one query block against one item block.  A lane holds sixteen items of one query, and the two
     // lanes that share a query (rows 4 * lhi + ...) each own a list of their own — (query, 2 * chunk + lhi) — so a
@@ -498,7 +507,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 template <int KS> static int launch_wide(const KnnF16SweepArgs& a, uint32_t grid)
 {
-    constexpr size_t lds = 2 * 64 * (KS * 16 + 8) * sizeof(_Float16);
+    constexpr size_t lds = 2 * kWideStageItems * (KS * 16 + 8) * sizeof(_Float16);
     static bool sized[64] = {};   // per device: the kernel's LDS limit is raised once
     const int dev = ctx().device;
     if (dev < 0 || dev >= 64 || !sized[dev]) {
@@ -614,7 +623,7 @@ int knn_f16_candidates_run(const void* queries16, const void* items16, uint32_t 
     a.cand = cand;
     if (seg && seg_count && ld <= 256 && (mode == 1 || mode == 3)) {
         // queries in registers: 512 per workgroup, stages of 64 items, one workgroup per CU
-        const uint32_t tiles_q = (batch + 511) / 512, stages = (n + 63) / 64;
+        const uint32_t tiles_q = (batch + 511) / 512, stages = (n + kWideStageItems - 1) / kWideStageItems;
         const uint32_t chunks = std::min<uint32_t>(kSweepCountStride / 2, (cus + tiles_q - 1) / tiles_q);   // two lists per (query, chunk)
         if (mode == 3 ? stages >= chunks : (2 * tiles_q * chunks >= cus && stages >= 8 * chunks)) {
             a.tiles_m = tiles_q;
