@@ -729,7 +729,7 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
     static_assert(E * kTopkThreads <= kGuidedMaxSegs, "at most kGuidedMaxSegs segments");
     __shared__ uint64_t sStage[kTopkWaves][List::kStageWords];
     __shared__ uint32_t sPrime[kTopkWaves][kGuidedMaxK];
-    __shared__ uint32_t sListCount;
+    __shared__ uint32_t sListCount, sBound;
     extern __shared__ uint32_t sDyn[];   // segments to read [nseg] | their maxima [nseg] | best listed score per segment [nseg] | bitmap of listed columns
     uint32_t* sList = sDyn;
     uint32_t* sListKey = sDyn + a.nseg;
@@ -772,14 +772,8 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
     bool light = false;   // the same for the whole workgroup
     if constexpr (FILTERED) {
         light = !a.fmul && (fe - fs) * 2 <= a.nseg;
-        const uint32_t words = (a.width + 31) / 32;
-        for (uint32_t i = threadIdx.x; i < words; i += kTopkThreads) sBitmap[i] = 0;
-        for (uint32_t i = threadIdx.x; i < a.nseg; i += kTopkThreads) sFiltMax[i] = 0;
-        __syncthreads();
-        auto mark = [&](uint32_t c, float v) {
-            atomicOr(&sBitmap[c >> 5], 1u << (c & 31));
-            if (v == v) atomicMax(&sFiltMax[c / kGuidedSegWidth], score_key(v));   // a NaN is never a segment's maximum
-        };
+        // (the listed columns are requested before the barrier below, which waits for everything in flight: the row's range,
+        // the maxima and the first listed columns then cost two round trips, not three)
 #pragma unroll
         for (int u = 0; u < kFU; u++) {
             const uint64_t t = fs + (uint64_t)u * kTopkThreads + threadIdx.x;
@@ -790,6 +784,14 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
                 if (a.fmul) fm[u] = a.fmul[t];
             }
         }
+        const uint32_t words = (a.width + 31) / 32;
+        for (uint32_t i = threadIdx.x; i < words; i += kTopkThreads) sBitmap[i] = 0;
+        for (uint32_t i = threadIdx.x; i < a.nseg; i += kTopkThreads) sFiltMax[i] = 0;
+        __syncthreads();
+        auto mark = [&](uint32_t c, float v) {
+            atomicOr(&sBitmap[c >> 5], 1u << (c & 31));
+            if (v == v) atomicMax(&sFiltMax[c / kGuidedSegWidth], score_key(v));   // a NaN is never a segment's maximum
+        };
         if (light) {   // (at most nseg / 2 <= 1024 listed columns: they are all in fcol)
 #pragma unroll
             for (int u = 0; u < kFU; u++) {
@@ -848,13 +850,23 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
             published += (uint32_t)__popcll(pm);
         }
         __syncthreads();
-        uint32_t all[4];
+        // (one wavefront searches, the others wait: four workgroups share a CU, and what the searches of sixteen wavefronts
+        // cost is instruction issue, not latency)
+        if (wave == 0) {
+            uint32_t all[4];
 #pragma unroll
-        for (int n = 0; n < 4; n++) {
-            const uint32_t i = n * kWave + lane;
-            all[n] = (i < kTopkWaves * a.k) ? sPrime[i / a.k][i % a.k] : 0u;
+            for (int n = 0; n < 4; n++) {
+                const uint32_t i = n * kWave + lane;
+                all[n] = (i < kTopkWaves * a.k) ? sPrime[i / a.k][i % a.k] : 0u;
+            }
+            uint32_t t;
+            if (a.k <= 16) t = wave_kth_key<1>(reinterpret_cast<const uint32_t(&)[1]>(all), a.k);
+            else if (a.k <= 32) t = wave_kth_key<2>(reinterpret_cast<const uint32_t(&)[2]>(all), a.k);
+            else t = wave_kth_key<4>(all, a.k);
+            if (lane == 0) sBound = t;
         }
-        const uint32_t t = (a.k <= 32) ? wave_kth_key<2>(reinterpret_cast<const uint32_t(&)[2]>(all), a.k) : wave_kth_key<4>(all, a.k);
+        __syncthreads();
+        const uint32_t t = sBound;
         if (t > score_key(-__builtin_inff())) {
             bound = t;
             list.prime(t);
@@ -884,16 +896,18 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
     // segment reaches the bound, but once a wavefront holds k of them, later segments that only tie are out.
     const uint32_t count = sListCount;
     constexpr int kSegsInFlight = 8;
-    for (uint32_t i0 = wave * kSegsInFlight; i0 < count; i0 += kTopkWaves * kSegsInFlight) {
+    // (the listed segments are dealt out one at a time: the usual dozen or two then keep all four wavefronts busy)
+    for (uint32_t i0 = wave; i0 < count; i0 += kTopkWaves * kSegsInFlight) {
         float v[kSegsInFlight];
         uint32_t col[kSegsInFlight];
 #pragma unroll
         for (int u = 0; u < kSegsInFlight; u++) {
             v[u] = __uint_as_float(0x7fc00000u);   // NaN fails the compare below
             col[u] = 0;
-            if (i0 + u < count) {
-                const uint32_t first = sList[i0 + u] * kGuidedSegWidth;
-                if (key_score(sListKey[i0 + u]) >= list.admission_score(first)) {   // wave-uniform
+            const uint32_t i = i0 + u * kTopkWaves;
+            if (i < count) {
+                const uint32_t first = sList[i] * kGuidedSegWidth;
+                if (key_score(sListKey[i]) >= list.admission_score(first)) {   // wave-uniform
                     col[u] = first + lane;
                     if (col[u] < a.width) v[u] = row[col[u]];
                 }
