@@ -5,6 +5,7 @@
 // with VEC consecutive fp32 columns per lane (128-bit gathers when VEC = 4), and the groups walk the non-zeros interleaved
 // (group g takes non-zeros g, g+G, ...), up to sixteen gathers in flight per lane.  The G partial sums are combined through LDS in
 // group order, so the result does not depend on scheduling.  Bias and activation can be applied in the same kernel.
+#include <type_traits>
 #include "dsx_device.h"
 #include "dsx_internal.h"
 
@@ -93,8 +94,11 @@ struct SparseZArgs {
 
 // T: storage type of the non-zero values; UNITVAL: every value is exactly 1 (Boolean, unweighted): no multiply;
 // FUSED: unit = act(bias + sum) instead of unit = beta * unit + sum.
-template <typename T, bool BOOLEAN, bool UNITVAL, int VEC, bool FUSED>
-__global__ __launch_bounds__(kSparseThreads) void sparse_z_kernel(SparseZArgs a)
+// DEEP: sixteen gathers per lane in flight (96 registers, five workgroups per CU) — what a launch of many rounds wants, where
+// the longest rows set the time; otherwise eight (at most 64 registers, eight workgroups per CU): a launch that then fits the
+// GPU in one round does without a second round's start-up.
+template <typename T, bool BOOLEAN, bool UNITVAL, int VEC, bool FUSED, bool DEEP>
+__global__ __launch_bounds__(kSparseThreads, DEEP ? 4 : 8) void sparse_z_kernel(SparseZArgs a)
 {
     __builtin_amdgcn_s_setprio(3);   // short kernels issue ahead of a GEMM's wavefronts that share their SIMD
     __shared__ uint32_t sIdx[kSparseChunk];
@@ -136,6 +140,16 @@ __global__ __launch_bounds__(kSparseThreads) void sparse_z_kernel(SparseZArgs a)
     float acc[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; v++) acc[v] = 0.0f;
+    // (the bias is requested now: asked for after the sums, it would be one more memory round trip at the very end)
+    float bz[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; v++) bz[v] = 0.0f;
+    if constexpr (FUSED) {
+        if (g == 0 && active && a.bias) {
+#pragma unroll
+            for (int v = 0; v < VEC; v++) bz[v] = a.bias[col + v];
+        }
+    }
 
     const float* wcol = a.weight + col;
     for (uint64_t cs = start; cs < end; cs += kSparseChunk) {
@@ -153,7 +167,8 @@ __global__ __launch_bounds__(kSparseThreads) void sparse_z_kernel(SparseZArgs a)
         __syncthreads();
         if (active) {
             uint32_t t = g;
-            for (; t + 15 * G < n; t += 16 * G) gather_block<16, VEC, UNITVAL>(wcol, a.stride, sIdx, sVal, t, G, acc);
+            constexpr int U = DEEP ? 16 : 8;
+            for (; t + (U - 1) * G < n; t += U * G) gather_block<U, VEC, UNITVAL>(wcol, a.stride, sIdx, sVal, t, G, acc);
             for (; t + 3 * G < n; t += 4 * G) gather_block<4, VEC, UNITVAL>(wcol, a.stride, sIdx, sVal, t, G, acc);
             for (; t < n; t += G) gather_block<1, VEC, UNITVAL>(wcol, a.stride, sIdx, sVal, t, G, acc);
         }
@@ -165,9 +180,27 @@ __global__ __launch_bounds__(kSparseThreads) void sparse_z_kernel(SparseZArgs a)
         for (int v = 0; v < VEC; v++) sRed[(g * lpr + lane) * VEC + v] = acc[v];
         __syncthreads();
         if (g == 0) {
-            for (uint32_t gg = 1; gg < G; gg++) {
+            // all partial sums are read at once and added in group order (G is 4, 8 or 16 with 64, 32 or 16 lanes per row)
+            auto combine = [&](auto groups_tag) __attribute__((always_inline)) {
+                constexpr int GG = decltype(groups_tag)::value;
+                float part[GG - 1][VEC];
 #pragma unroll
-                for (int v = 0; v < VEC; v++) acc[v] += sRed[(gg * lpr + lane) * VEC + v];
+                for (int gg = 1; gg < GG; gg++)
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) part[gg - 1][v] = sRed[(gg * lpr + lane) * VEC + v];
+#pragma unroll
+                for (int gg = 1; gg < GG; gg++)
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) acc[v] += part[gg - 1][v];
+            };
+            if (G == 16) combine(std::integral_constant<int, 16>());
+            else if (G == 8) combine(std::integral_constant<int, 8>());
+            else if (G == 4) combine(std::integral_constant<int, 4>());
+            else {
+                for (uint32_t gg = 1; gg < G; gg++) {
+#pragma unroll
+                    for (int v = 0; v < VEC; v++) acc[v] += sRed[(gg * lpr + lane) * VEC + v];
+                }
             }
         }
     }
@@ -176,7 +209,7 @@ __global__ __launch_bounds__(kSparseThreads) void sparse_z_kernel(SparseZArgs a)
         if constexpr (FUSED) {
 #pragma unroll
             for (int v = 0; v < VEC; v++) {
-                float x = (a.bias ? a.bias[col + v] : 0.0f) + acc[v];
+                float x = bz[v] + acc[v];
                 o[v] = activate_rt(x, a.act, a.slope, a.alpha, a.lambda);
             }
         } else {
@@ -218,11 +251,24 @@ static int launch_sparse_z(const SparseZArgs& a0, uint32_t batch)
     a.tile_major = batch <= 65535;   // (the second grid dimension ends there)
     dim3 grid = a.tile_major ? dim3(tiles, batch) : dim3(batch, tiles);
     hipStream_t s = ctx().stream;
+    // (values that are not all 1 need registers for the values as well: only the deep form)
+    const bool deep = !UNITVAL || (uint64_t)tiles * batch > 8ull * (uint64_t)ctx().num_cus;   // more than one round of eight workgroups per CU
+#define DSX_SPARSE_CASE(V)                                                                                                            \
+    case V:                                                                                                                           \
+        if constexpr (UNITVAL) {                                                                                                      \
+            if (!deep) {                                                                                                              \
+                hipLaunchKernelGGL((sparse_z_kernel<T, BOOLEAN, UNITVAL, V, FUSED, false>), grid, dim3(kSparseThreads), 0, s, a);     \
+                break;                                                                                                                \
+            }                                                                                                                         \
+        }                                                                                                                             \
+        hipLaunchKernelGGL((sparse_z_kernel<T, BOOLEAN, UNITVAL, V, FUSED, true>), grid, dim3(kSparseThreads), 0, s, a);              \
+        break;
     switch (vec) {
-    case 4: hipLaunchKernelGGL((sparse_z_kernel<T, BOOLEAN, UNITVAL, 4, FUSED>), grid, dim3(kSparseThreads), 0, s, a); break;
-    case 2: hipLaunchKernelGGL((sparse_z_kernel<T, BOOLEAN, UNITVAL, 2, FUSED>), grid, dim3(kSparseThreads), 0, s, a); break;
-    default: hipLaunchKernelGGL((sparse_z_kernel<T, BOOLEAN, UNITVAL, 1, FUSED>), grid, dim3(kSparseThreads), 0, s, a); break;
+        DSX_SPARSE_CASE(4)
+        DSX_SPARSE_CASE(2)
+        DSX_SPARSE_CASE(1)
     }
+#undef DSX_SPARSE_CASE
     DSX_LAUNCH_CHECK("sparse_z_kernel");
     return DSX_OK;
 }
