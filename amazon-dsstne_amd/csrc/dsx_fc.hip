@@ -581,7 +581,10 @@ int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int trans
             a.nseg = (n + 63) / 64;
             *seg_width = 64;
         }
-        launch_fc_shape<2, 2, 16>(a, xv, wv, transposed != 0);
+        // Short sums (the wide layer behind a narrow one) are staged eight k-steps at a time: the multiplications cost the same,
+        // and the kernels of other streams that share the CUs find 17 KiB of LDS taken per workgroup instead of 34.
+        if (k <= 256) launch_fc_shape<2, 2, 8>(a, xv, wv, transposed != 0);
+        else launch_fc_shape<2, 2, 16>(a, xv, wv, transposed != 0);
     } else if (!transposed && !accumulate && xv == 4 && (k == 128 || k == 256) && (uint64_t)batch * n <= (1u << 20)) {
         if (k == 128) launch_fc_small<32>(a);   // latency bound: all operands in one round trip
         else launch_fc_small<64>(a);
