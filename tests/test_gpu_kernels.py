@@ -349,7 +349,11 @@ def test_topk_testsort_shapes(pkg, dsx, orc, rng, batch, k, nfeat):
 # misaligned (odd widths), more slots than columns, one workgroup per row and several.
 @pytest.mark.parametrize("batch,width,k", [(5, 1, 1), (3, 2, 4), (9, 7, 3), (4, 64, 64), (6, 65, 65), (7, 255, 128), (3, 257, 129),
                                            (2, 1000, 256), (33, 4099, 10), (1024, 27278, 10), (3, 1000003, 100), (1, 300000, 256),
-                                           (16, 50001, 200)])
+                                           (16, 50001, 200),
+                                           # k on both sides of every width of the primed bound's key search (16, 32, 64, 128 keys
+                                           # per lane group), rows of two full spans and more and rows shorter than one span
+                                           (12, 27278, 16), (12, 27278, 17), (12, 27278, 33), (12, 27278, 65), (12, 27278, 128),
+                                           (12, 27278, 129), (9, 5000, 16), (9, 5000, 17), (7, 70000, 32), (7, 70000, 64)])
 def test_topk_random(pkg, dsx, orc, rng, batch, width, k):
     say("topk random batch=%d width=%d k=%d" % (batch, width, k))
     scores = rng.standard_normal((batch, width)).astype(np.float32)
@@ -462,9 +466,11 @@ def run_guided(pkg, dsx, scores, k, seg_max, position=0, index=None, start=None,
 
 
 @pytest.mark.parametrize("batch,width,k", [(16, 27278, 10), (5, 64, 8), (7, 65, 32), (9, 1000, 1), (4, 131072, 32), (3, 40, 32),
-                                           (6, 5000, 64), (8, 27278, 50), (5, 5000, 100), (2, 200000, 10)])
+                                           (6, 5000, 64), (8, 27278, 50), (5, 5000, 100), (2, 200000, 10),
+                                           (9, 27278, 16), (9, 27278, 17), (9, 27278, 33), (9, 130000, 16)])
 def test_topk_guided_plain(pkg, dsx, orc, rng, batch, width, k):
-    # the last two shapes are outside the guided kernel's range (k > 64, more than 2048 segments): the call scans instead
+    # (5, 5000, 100) and (2, 200000, 10) are outside the guided kernel's range (k > 64, more than 2048 segments): the call scans
+    # instead; the shapes after them put k on both sides of the widths of the bound's key search
     say("topk_guided batch=%d width=%d k=%d" % (batch, width, k))
     scores = rng.standard_normal((batch, width), dtype=np.float32)
     keys, idx = run_guided(pkg, dsx, scores, k, segment_maxima(scores))
