@@ -404,10 +404,11 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
                 }
                 __syncthreads();
             };
-            if constexpr (BK >= 16) {
+            if constexpr (BK >= 16 && CAND != 2) {
                 // Two k-steps per trip: each step's LDS buffer is then a constant and its addresses are immediate offsets, a
                 // dozen vector instructions less per step (1.5-1.8 % at k = 512 and 1,024; with steps of 8 the longer loop body
-                // costs more than that saves).
+                // costs more than that saves, and the layer's candidate mode, which also keeps its bounds and the bias in
+                // registers, would spill).
                 uint32_t kt = 0;
                 for (; kt + 1 < nk; kt += 2) {
                     k_step(kt, 0);
