@@ -82,6 +82,8 @@ SIGNATURES = {
                                  C.POINTER(ActParams), _vp],
     "dsx_fc_forward": [_vp, _u32, _vp, _int, _vp, _vp, _u32, _u32, _u32, _u32, _int, _u32, C.POINTER(ActParams)],
     "dsx_fc_forward_segmax": [_vp, _u32, _vp, _int, _vp, _vp, _u32, _u32, _u32, _u32, _u32, C.POINTER(ActParams), _vp, C.POINTER(_u32)],
+    "dsx_fc_split": [_vp, _u32, _int, _u32, _u32, _vp],
+    "dsx_fc_forward_split": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _int, _u32, C.POINTER(ActParams), _vp, C.POINTER(_u32)],
     "dsx_activation": [_vp, _u32, _u32, _u32, C.POINTER(ActParams)],
     "dsx_add_buffers": [_vp, _vp, _u64],
     "dsx_topk": [_vp, _vp, _vp, _u32, _u32, _u32],
@@ -104,9 +106,10 @@ SIGNATURES = {
     "dsx_knn_f16_set_sweep": [_int],
 }
 SPECIAL_RESTYPES = {"dsx_last_error": C.c_char_p, "dsx_stream": C.c_void_p, "dsx_knn_workspace_bytes": C.c_size_t,
-                    "dsx_knn_workspace_bytes_f16": C.c_size_t, "dsx_knn_f16_table_bytes": C.c_size_t}
+                    "dsx_knn_workspace_bytes_f16": C.c_size_t, "dsx_knn_f16_table_bytes": C.c_size_t, "dsx_fc_split_bytes": _u64}
 SPECIAL_ARGTYPES = {"dsx_last_error": [], "dsx_stream": [], "dsx_knn_workspace_bytes": [_u32, _u32, _u32, _u32],
-                    "dsx_knn_workspace_bytes_f16": [_u32, _u32, _u32, _u32], "dsx_knn_f16_table_bytes": [_u32, _u32]}
+                    "dsx_knn_workspace_bytes_f16": [_u32, _u32, _u32, _u32], "dsx_knn_f16_table_bytes": [_u32, _u32],
+                    "dsx_fc_split_bytes": [_u32, _u32]}
 
 _lib = None
 

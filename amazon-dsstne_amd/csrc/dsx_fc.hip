@@ -657,6 +657,199 @@ int fc_layer_candidates_run(const float* X, uint32_t ldx, const float* W, uint32
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
+// fp32 products from bf16 matrix instructions (a mode the caller asks for; the kernels above multiply in fp32).
+// An fp32 value is the exact sum of three bf16 values, hi + mid + lo (3 x 8 significant bits, each rounded to nearest from what
+// the ones before left).  Of the nine products of two such sums, the six that reach 2^-24 of the full product are accumulated
+// in fp32 by v_mfma_f32_32x32x16_bf16, smallest first: twelve matrix-core cycles per k and 32 x 32 block where
+// v_mfma_f32_32x32x2_f32 takes thirty-two.  What is dropped (mid.lo, lo.mid, lo.lo) is below 2^-25 of a product, less than the
+// rounding of the product itself in fp32; measured against fp64, the sums are as close as the fp32 kernel's.
+// Operands come pre-split ("planes"): plane p, block kb of eight consecutive k, row r (a row of X or a column of W) is one
+// 16-byte unit at ((p * kblocks + kb) * rows_padded + r), rows padded to 128 and k to 16 with zeros, so that a lane's MFMA
+// operand is one 128-bit read, the 128 rows of a tile are 2 KiB of consecutive memory and no load needs a bounds check.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // (a native vector: arrays of it stay in registers)
+
+__device__ __forceinline__ uint32_t bf16_rn_bits(float x)
+{
+    const uint32_t u = __float_as_uint(x);
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+
+// src element (r, kk) is src[r * stride_r + kk * stride_k].  One lane per (block of eight k, row); consecutive lanes take
+// consecutive rows (a [k][n] weight matrix is read along n, the planes are written 16 bytes per lane, consecutively).
+__global__ __launch_bounds__(256) void fc_split_kernel(const float* __restrict__ src, uint64_t stride_r, uint64_t stride_k, uint32_t rows,
+                                                        uint32_t k, uint32_t rows_padded, uint32_t kblocks, uint4* __restrict__ planes)
+{
+    const uint64_t id = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (id >= (uint64_t)rows_padded * kblocks) return;
+    const uint32_t r = (uint32_t)(id % rows_padded), kb = (uint32_t)(id / rows_padded);
+    uint32_t h[8], m[8], l[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const uint32_t kk = kb * 8 + e;
+        float x = 0.0f;
+        if (r < rows && kk < k) x = src[r * stride_r + kk * stride_k];
+        if (!(fabsf(x) < 3.0e38f)) {   // infinities, NaN and what would round up to infinity stay in the first plane alone
+            h[e] = __float_as_uint(x) >> 16; m[e] = 0; l[e] = 0;
+            if (x != x) h[e] |= 0x40;
+            continue;
+        }
+        h[e] = bf16_rn_bits(x);
+        const float r1 = x - __uint_as_float(h[e] << 16);   // exact
+        m[e] = bf16_rn_bits(r1);
+        const float r2 = r1 - __uint_as_float(m[e] << 16);  // exact
+        l[e] = bf16_rn_bits(r2);
+    }
+    const uint64_t unit = (uint64_t)kb * rows_padded + r, plane = (uint64_t)kblocks * rows_padded;
+    planes[unit] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+    planes[plane + unit] = make_uint4(m[0] | (m[1] << 16), m[2] | (m[3] << 16), m[4] | (m[5] << 16), m[6] | (m[7] << 16));
+    planes[2 * plane + unit] = make_uint4(l[0] | (l[1] << 16), l[2] | (l[3] << 16), l[4] | (l[5] << 16), l[6] | (l[7] << 16));
+}
+
+struct FcSplitArgs {
+    const u32x4* Xs;
+    const u32x4* Ws;
+    uint32_t xrows, wrows, kblocks;   // padded rows of the two sets of planes; blocks of eight k (an even number)
+};
+
+// Z = act(acc? + bias + X . W) as fc_gemm_kernel<2, 2, ...> computes it (same tile order, same epilogue), from planes.
+// A k-step is one MFMA depth (16): 24 KiB of operands (3 planes x 2 blocks of k x (128 + 128) rows x 16 bytes), double
+// buffered in LDS; every lane moves one unit of each plane of each operand per step.
+template <int ACT>
+__global__ __launch_bounds__(kFcThreads, 3) void fc_gemm_split_kernel(FcArgs a, FcSplitArgs sp)
+{
+    __shared__ u32x4 sA[2][3][2][128];
+    __shared__ u32x4 sB[2][3][2][128];
+    const uint32_t total = a.tiles_m * a.tiles_n;
+    uint32_t wg = blockIdx.x;
+    {
+        const uint32_t per_xcd = (total + kXcds - 1) / kXcds;
+        const uint32_t xcd = wg % kXcds, local = wg / kXcds;
+        wg = xcd * per_xcd + local;
+        if (local >= per_xcd || wg >= total) return;
+    }
+    const uint32_t tm = wg % a.tiles_m, tn = a.tiles_n - 1 - wg / a.tiles_m;
+    const uint32_t row0 = tm * 128, col0 = tn * 128;
+    __builtin_amdgcn_s_setprio(1);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, lhi = lane >> 5;
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    const int srow = tid & 127, shalf = tid >> 7;
+    const uint64_t xplane = (uint64_t)sp.kblocks * sp.xrows, wplane = (uint64_t)sp.kblocks * sp.wrows;
+    const u32x4* xa = sp.Xs + (uint64_t)shalf * sp.xrows + row0 + srow;
+    const u32x4* wb = sp.Ws + (uint64_t)shalf * sp.wrows + col0 + srow;
+    u32x4 ra[3], rb[3];
+    auto load = [&](uint32_t kt) __attribute__((always_inline)) {
+#pragma unroll
+        for (int p = 0; p < 3; p++) {
+            ra[p] = xa[p * xplane + (uint64_t)(2 * kt) * sp.xrows];
+            rb[p] = wb[p * wplane + (uint64_t)(2 * kt) * sp.wrows];
+        }
+    };
+    auto store = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int p = 0; p < 3; p++) {
+            sA[buf][p][shalf][srow] = ra[p];
+            sB[buf][p][shalf][srow] = rb[p];
+        }
+    };
+    auto multiply = [&](int buf) __attribute__((always_inline)) {
+        bf16x8 fa[2][3], fb[2][3];
+#pragma unroll
+        for (int p = 0; p < 3; p++) {
+#pragma unroll
+            for (int i = 0; i < 2; i++) fa[i][p] = __builtin_bit_cast(bf16x8, sA[buf][p][lhi][wm * 64 + i * 32 + l32]);
+#pragma unroll
+            for (int j = 0; j < 2; j++) fb[j][p] = __builtin_bit_cast(bf16x8, sB[buf][p][lhi][wn * 64 + j * 32 + l32]);
+        }
+        // (plane of X, plane of W): lo.hi, hi.lo, mid.mid, mid.hi, hi.mid, hi.hi
+#define DSX_TERM(PX, PW)                                                                                                   \
+    _Pragma("unroll") for (int i = 0; i < 2; i++) _Pragma("unroll") for (int j = 0; j < 2; j++)                            \
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][PX], fb[j][PW], acc[i][j], 0, 0, 0);
+        DSX_TERM(2, 0) DSX_TERM(0, 2) DSX_TERM(1, 1) DSX_TERM(1, 0) DSX_TERM(0, 1) DSX_TERM(0, 0)
+#undef DSX_TERM
+    };
+    const uint32_t nk = sp.kblocks / 2;
+    load(0);
+    store(0);
+    __syncthreads();
+    for (uint32_t kt = 0; kt < nk; kt++) {
+        const int buf = kt & 1;
+        // (unconditional, so that the staging registers stay registers: the last step's reload goes where nobody reads it)
+        load(kt + 1 < nk ? kt + 1 : kt);
+        multiply(buf);
+        store(buf ^ 1);
+        __syncthreads();
+    }
+    __builtin_amdgcn_s_setprio(0);
+    static_assert(sizeof(sA) >= 2 * 512 * sizeof(float) && sizeof(sB) >= 2 * 512 * sizeof(float),
+                  "the segment maxima are transposed through the operand tiles' LDS, two wavefronts in each");
+    fc_epilogue<2, 2, ACT>(acc, a, row0 + wm * 64, col0 + wn * 64, lane,
+                           reinterpret_cast<float*>((wave < 2) ? &sA[0][0][0][0] : &sB[0][0][0][0]) + (wave & 1) * 512);
+}
+
+static inline uint32_t split_rows_padded(uint32_t rows) { return (rows + 127) / 128 * 128; }
+static inline uint32_t split_kblocks(uint32_t k) { return (k + 15) / 16 * 2; }
+
+static int fc_split_planes_run(const float* src, uint64_t stride_r, uint64_t stride_k, uint32_t rows, uint32_t k, void* planes)
+{
+    const uint32_t rp = split_rows_padded(rows), kb = split_kblocks(k);
+    const uint64_t units = (uint64_t)rp * kb;
+    hipLaunchKernelGGL(fc_split_kernel, dim3((uint32_t)((units + 255) / 256)), dim3(256), 0, ctx().stream, src, stride_r, stride_k, rows, k, rp,
+                       kb, reinterpret_cast<uint4*>(planes));
+    DSX_LAUNCH_CHECK("fc_split_kernel");
+    return DSX_OK;
+}
+
+static int fc_split_run(const void* Xs, const void* Ws, const float* bias, float* Z, uint32_t ldz, uint32_t batch, uint32_t k, uint32_t n,
+                 int accumulate, uint32_t activation, const dsx_act_params* params, float* seg_max, uint32_t* seg_width)
+{
+    if (seg_width) *seg_width = 0;
+    FcArgs a{};
+    a.bias = bias; a.Z = Z; a.ldz = ldz;
+    a.batch = batch; a.k = k; a.n = n;
+    a.accumulate = accumulate;
+    a.act = activation;
+    a.slope = params ? params->slope : 0.01f;
+    a.alpha = params ? params->alpha : 1.0f;
+    a.lambda = params ? params->lambda : 1.0f;
+    a.tiles_m = (batch + 127) / 128;
+    a.tiles_n = (n + 127) / 128;
+    if (seg_max && seg_width && !accumulate) {
+        a.seg_max = seg_max;
+        a.nseg = (n + 63) / 64;
+        *seg_width = 64;
+    }
+    FcSplitArgs sp{reinterpret_cast<const u32x4*>(Xs), reinterpret_cast<const u32x4*>(Ws), split_rows_padded(batch), split_rows_padded(n),
+                   split_kblocks(k)};
+    const uint32_t total = a.tiles_m * a.tiles_n;
+    const dim3 grid(((total + kXcds - 1) / kXcds) * kXcds);
+    hipStream_t s = ctx().stream;
+#define DSX_ACT_CASE(A) case A: hipLaunchKernelGGL((fc_gemm_split_kernel<A>), grid, dim3(kFcThreads), 0, s, a, sp); break;
+    switch (a.act) {
+        DSX_ACT_CASE(DSX_ACT_SIGMOID)
+        DSX_ACT_CASE(DSX_ACT_TANH)
+        DSX_ACT_CASE(DSX_ACT_RELU)
+        DSX_ACT_CASE(DSX_ACT_LRELU)
+        DSX_ACT_CASE(DSX_ACT_ELU)
+        DSX_ACT_CASE(DSX_ACT_SELU)
+    default: hipLaunchKernelGGL((fc_gemm_split_kernel<DSX_ACT_LINEAR>), grid, dim3(kFcThreads), 0, s, a, sp); break;
+    }
+#undef DSX_ACT_CASE
+    DSX_LAUNCH_CHECK("fc_gemm_split_kernel");
+    return DSX_OK;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
 // Stand-alone activations (used when a layer has several sources, so the GEMM epilogue cannot apply them).
 
 __global__ __launch_bounds__(256) void activation_kernel(float* z, uint64_t size, uint32_t act, float slope, float alpha, float lambda)
@@ -719,6 +912,34 @@ int dsx_fc_forward_segmax(const float* X, uint32_t ldx, const float* W, int tran
     *seg_width = 0;
     if (batch == 0) return DSX_OK;
     return fc_run(X, ldx, W, transposed ? k : n, transposed, bias, Z, ldz, batch, k, n, 0, activation, params, seg_max, seg_width);
+}
+
+uint64_t dsx_fc_split_bytes(uint32_t rows, uint32_t k)
+{
+    return 3ull * split_rows_padded(rows) * split_kblocks(k) * 16;
+}
+
+int dsx_fc_split(const float* src, uint32_t ld, int k_major, uint32_t rows, uint32_t k, void* planes)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(src && planes, "dsx_fc_split: null device pointer");
+    DSX_CHECK_ARG(((uintptr_t)planes % 16) == 0, "dsx_fc_split: planes must be 16-byte aligned");
+    DSX_CHECK_ARG(rows > 0 && k > 0 && ld >= (k_major ? rows : k), "dsx_fc_split: rows = %u, k = %u, ld = %u", rows, k, ld);
+    return k_major ? fc_split_planes_run(src, 1, ld, rows, k, planes) : fc_split_planes_run(src, ld, 1, rows, k, planes);
+}
+
+int dsx_fc_forward_split(const void* x_planes, const void* w_planes, const float* bias, float* Z, uint32_t ldz, uint32_t batch, uint32_t k,
+                         uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params, float* seg_max, uint32_t* seg_width)
+{
+    DSX_REQUIRE_INIT();
+    if (seg_width) *seg_width = 0;
+    DSX_CHECK_ARG(x_planes && w_planes && Z, "dsx_fc_forward_split: null device pointer");
+    DSX_CHECK_ARG(((uintptr_t)x_planes % 16) == 0 && ((uintptr_t)w_planes % 16) == 0, "dsx_fc_forward_split: planes must be 16-byte aligned");
+    DSX_CHECK_ARG(k > 0 && n > 0 && ldz >= n, "dsx_fc_forward_split: k = %u, n = %u, ldz = %u", k, n, ldz);
+    DSX_CHECK_ARG(is_elementwise_activation(activation), "dsx_fc_forward_split: activation %u is a row operation; pass DSX_ACT_LINEAR and call dsx_activation", activation);
+    DSX_CHECK_ARG((seg_max == NULL) == (seg_width == NULL), "dsx_fc_forward_split: seg_max and seg_width go together");
+    if (batch == 0) return DSX_OK;
+    return fc_split_run(x_planes, w_planes, bias, Z, ldz, batch, k, n, accumulate, activation, params, seg_max, seg_width);
 }
 
 int dsx_activation(float* unit, uint32_t batch, uint32_t stride, uint32_t activation, const dsx_act_params* params)

@@ -12,8 +12,9 @@ from . import ACT_SOFTMAX, ActParams, DeviceArray, check, load_library, ptr
 
 
 class DevicePipeline:
-    def __init__(self, problem, lib=None, guided=False):
-        """guided: the output layer also leaves segment maxima (dsx_fc_forward_segmax) and the top-K uses them."""
+    def __init__(self, problem, lib=None, guided=False, split=False):
+        """guided: the output layer also leaves segment maxima (dsx_fc_forward_segmax) and the top-K uses them.
+        split: the output layer forms its fp32 products from bf16 matrix instructions (dsx_fc_split / dsx_fc_forward_split)."""
         self.lib = lib or load_library()
         p = self.p = problem
         self.guided = guided
@@ -31,6 +32,12 @@ class DevicePipeline:
         self.keys = DeviceArray((p.batch, 256), np.float32, self.lib)
         self.vals = DeviceArray((p.batch, 256), np.uint32, self.lib)
         self.params = ActParams(0.01, 1.0, 1.0)
+        self.split = split
+        if split:
+            k, n = p.widths[-2], p.widths[-1]
+            self.w_planes = DeviceArray((self.lib.dsx_fc_split_bytes(n, k) // 4,), np.uint32, self.lib)
+            self.x_planes = DeviceArray((self.lib.dsx_fc_split_bytes(p.batch, k) // 4,), np.uint32, self.lib)
+            check(self.lib.dsx_fc_split(ptr(self.W[-1]), n, 1, n, k, ptr(self.w_planes)))   # weights: once
 
     def forward(self, position=0, batch=None):
         """All layers; returns nothing (activations stay in self.units)."""
@@ -46,6 +53,15 @@ class DevicePipeline:
             k, n = p.widths[l], p.widths[l + 1]
             act = p.acts[l]
             fused = act if act != ACT_SOFTMAX else 3
+            if self.split and l == len(self.W) - 1:
+                check(lib.dsx_fc_split(ptr(self.units[l - 1]), k, 0, batch, k, ptr(self.x_planes)))
+                g = self.guided and act != ACT_SOFTMAX
+                check(lib.dsx_fc_forward_split(ptr(self.x_planes), ptr(self.w_planes), ptr(self.b[l]), ptr(self.units[l]), n, batch, k, n, 0,
+                                               fused, C.byref(self.params), ptr(self.seg_max) if g else None,
+                                               C.byref(self.seg_width) if g else None))
+                if act == ACT_SOFTMAX:
+                    check(lib.dsx_activation(ptr(self.units[l]), batch, n, act, C.byref(self.params)))
+                continue
             if self.guided and l == len(self.W) - 1 and act != ACT_SOFTMAX:
                 check(lib.dsx_fc_forward_segmax(ptr(self.units[l - 1]), k, ptr(self.W[l]), 0, ptr(self.b[l]), ptr(self.units[l]), n, batch, k,
                                                 n, fused, C.byref(self.params), ptr(self.seg_max), C.byref(self.seg_width)))

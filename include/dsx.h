@@ -206,6 +206,26 @@ int dsx_fc_forward_segmax(const float* X, uint32_t ldx, const float* W, int tran
                           uint32_t batch, uint32_t k, uint32_t n, uint32_t activation, const dsx_act_params* params, float* seg_max,
                           uint32_t* seg_width);
 
+/* The same layer with every fp32 product formed from bf16 matrix instructions: a mode the caller asks for, with no counterpart
+ * in the reference (whose cublasSgemm, engine/NNLayer.cpp:1056-1096, multiplies in fp32, as dsx_fc_forward does).  An fp32
+ * value is the exact sum of three bf16 values; six of the nine products of two such sums, accumulated in fp32, carry
+ * everything above 2^-25 of the full product, so the sums are as close to the exact ones as dsx_fc_forward's (the tests
+ * compare both with fp64), at 12 instead of 32 matrix-core cycles per k.  They are not bit-identical to dsx_fc_forward's.
+ *
+ * Operands are passed pre-split.  dsx_fc_split writes the planes of `rows` vectors of k values each:
+ *   k_major == 0: vector r is src[r * ld + 0 .. k)        (X, a [batch x k] unit buffer; W stored [n x k], i.e. transposed)
+ *   k_major != 0: vector r is src[0 .. k) * ld + r         (W stored [k x n])
+ * into `planes`, dsx_fc_split_bytes(rows, k) bytes of 16-byte aligned device memory (3 x 2 bytes per value, rows padded to
+ * 128 and k to 16).  Weights are split once, a layer's input once per batch.  Inf and NaN inputs stay Inf / NaN; finite values
+ * from 3.0e38 up are kept to bf16 precision only.
+ * dsx_fc_forward_split then computes Z as dsx_fc_forward (accumulate, bias, activation) and, with seg_max / seg_width non-NULL
+ * and accumulate == 0, the segment maxima as dsx_fc_forward_segmax (*seg_width = 64 for every shape). */
+uint64_t dsx_fc_split_bytes(uint32_t rows, uint32_t k);
+int dsx_fc_split(const float* src, uint32_t ld, int k_major, uint32_t rows, uint32_t k, void* planes);
+int dsx_fc_forward_split(const void* x_planes, const void* w_planes, const float* bias, float* Z, uint32_t ldz, uint32_t batch, uint32_t k,
+                         uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params, float* seg_max,
+                         uint32_t* seg_width);
+
 /* kCalculateSigmoidActivation ... kCalculateSELUActivation (engine/kActivation.cu:46-153) and
  * kCalculateSoftMaxActivation (engine/kActivation.cu:155-236), in place on a [batch x stride] buffer. */
 int dsx_activation(float* unit, uint32_t batch, uint32_t stride, uint32_t activation, const dsx_act_params* params);

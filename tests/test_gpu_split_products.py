@@ -1,0 +1,186 @@
+"""The dense layer with fp32 products formed from bf16 matrix instructions (dsx_fc_split / dsx_fc_forward_split) against the
+CPU oracle, against fp64, and against the fp32 kernel it stands in for (needs an MI355X).
+
+Tolerance: 1e-4 relative to the scale of the sums, as for dsx_fc_forward; on top of that the mode has to be as close to the
+fp64 product as the fp32 kernel is (it claims fp32 accuracy, not only the tolerance)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from parity import assert_close, assert_topk_parity, assert_units_close
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print("[case] " + msg, flush=True)
+
+
+def dev(pkg, a):
+    return None if a is None else pkg.DeviceArray.from_numpy(a)
+
+
+def planes_of(pkg, dsx, d, ld, k_major, rows, k):
+    planes = pkg.DeviceArray((dsx.dsx_fc_split_bytes(rows, k) // 4,), np.uint32)
+    pkg.check(dsx.dsx_fc_split(d.ptr, ld, k_major, rows, k, planes.ptr))
+    return planes
+
+
+def bf16_planes_to_float(words, rows, k):
+    """Undo the layout of dsx_fc_split on the host: returns the three planes as float64 arrays [rows][k]."""
+    rp, kb = (rows + 127) // 128 * 128, (k + 15) // 16 * 2
+    halves = words.view(np.uint16).reshape(3, kb, rp, 8)
+    f = (halves.astype(np.uint32) << 16).view(np.float32).astype(np.float64)      # [p][kb][r][8]
+    f = f.transpose(0, 2, 1, 3).reshape(3, rp, kb * 8)
+    return f, rp, kb * 8
+
+
+@pytest.mark.parametrize("rows,k,k_major", [(5, 3, 0), (130, 17, 0), (257, 40, 1), (128, 16, 1), (1, 129, 1)])
+def test_split_planes_sum_back_to_the_input(pkg, dsx, rng, rows, k, k_major):
+    """hi + mid + lo is the fp32 input exactly (three times eight significant bits), the padding is zero, and each plane is what
+    rounding to nearest-even leaves of the one before (so that |mid| <= ulp_bf16(hi) / 2 and so on)."""
+    say("split planes rows=%d k=%d k_major=%d" % (rows, k, k_major))
+    x = (rng.standard_normal((rows, k)) * np.exp(4 * rng.standard_normal((rows, k)))).astype(np.float32)
+    x[0, 0] = 0.0
+    x[rows - 1, k - 1] = np.float32(1.0) + np.float32(2.0 ** -23)      # needs all three planes
+    ld = (rows if k_major else k) + 3
+    src = np.zeros((k, ld) if k_major else (rows, ld), dtype=np.float32)
+    if k_major:
+        src[:, :rows] = x.T
+    else:
+        src[:, :k] = x
+    d = dev(pkg, src)
+    planes = planes_of(pkg, dsx, d, ld, k_major, rows, k)
+    f, rp, kp = bf16_planes_to_float(planes.numpy(), rows, k)
+    total = f[0] + f[1] + f[2]
+    assert np.array_equal(total[:rows, :k], x.astype(np.float64))
+    assert not total[rows:].any() and not total[:, k:].any()
+    hi = f[0][:rows, :k]
+    nz = hi != 0
+    assert np.all(np.abs(f[1][:rows, :k][nz]) <= np.abs(hi[nz]) * 2.0 ** -8)
+    assert np.all(np.abs(f[2][:rows, :k][nz]) <= np.abs(hi[nz]) * 2.0 ** -16)
+
+
+def test_split_planes_special_values(pkg, dsx):
+    x = np.array([[np.inf, -np.inf, np.nan, 3.3e38, -3.4e38, 1e-40, -0.0, 65504.0]], dtype=np.float32)
+    d = dev(pkg, x)
+    planes = planes_of(pkg, dsx, d, 8, 0, 1, 8)
+    f, _, _ = bf16_planes_to_float(planes.numpy(), 1, 8)
+    total = (f[0] + f[1] + f[2])[0, :8]
+    assert total[0] == np.inf and total[1] == -np.inf and np.isnan(total[2])
+    assert np.isfinite(total[3]) and abs(total[3] / 3.3e38 - 1) < 2.0 ** -7          # kept to bf16 precision, not turned into inf
+    assert np.isfinite(total[4]) and abs(total[4] / -3.4e38 - 1) < 2.0 ** -7
+    assert total[7] == 65504.0 and total[6] == 0.0
+    assert abs(total[5] - 1e-40) <= 2.0 ** -134                                         # subnormal: to half a bf16 subnormal step
+
+
+SHAPES = [(300, 100, 1000), (130, 17, 257), (1, 128, 129), (257, 130, 128), (64, 512, 3000), (1024, 128, 5000)]
+
+
+@pytest.mark.parametrize("B,k,n", SHAPES)
+def test_fc_split_vs_oracle_fp64_and_fp32_kernel(pkg, dsx, orc, rng, B, k, n):
+    say("fc_forward_split B=%d k=%d n=%d" % (B, k, n))
+    X = (rng.standard_normal((B, k)) * np.exp(rng.standard_normal((B, k)))).astype(np.float32)
+    W = (rng.standard_normal((k, n)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    dX, dW, db = dev(pkg, X), dev(pkg, W), dev(pkg, bias)
+    xp = planes_of(pkg, dsx, dX, k, 0, B, k)
+    wp = planes_of(pkg, dsx, dW, n, 1, n, k)
+    Z = pkg.DeviceArray.from_numpy(np.full((B, n + 3), 55.0, dtype=np.float32))
+    pkg.check(dsx.dsx_fc_forward_split(xp.ptr, wp.ptr, db.ptr, Z.ptr, n + 3, B, k, n, 0, 3, None, None, None))
+    got = Z.numpy()
+    assert np.all(got[:, n:] == 55.0)                                   # nothing written past n
+    got = got[:, :n]
+    ref = orc.sgemm_acc(X, W, orc.clear_unit([bias], n, B))
+    scale = np.abs(X).astype(np.float64) @ np.abs(W).astype(np.float64) + np.abs(bias)   # what the rounding errors scale with
+    assert_close(got, ref, "split fc vs oracle", rel=1e-4, abs_floor=max(0.1 * float(scale.max()), 1e-2))
+    exact = X.astype(np.float64) @ W.astype(np.float64) + bias
+    Zf = pkg.DeviceArray.from_numpy(np.zeros((B, n), dtype=np.float32))
+    pkg.check(dsx.dsx_fc_forward(dX.ptr, k, dW.ptr, 0, db.ptr, Zf.ptr, n, B, k, n, 0, 3, None))
+    err_split = float((np.abs(got - exact) / scale).max())
+    err_f32 = float((np.abs(Zf.numpy() - exact) / scale).max())
+    say("  max error / sum |x||w|: split %.3e, fp32 kernel %.3e" % (err_split, err_f32))
+    assert err_split <= 1.5 * err_f32 + 2.0 ** -24                      # as close to fp64 as fp32 multiplication is
+    assert err_split < 2e-6
+
+
+@pytest.mark.parametrize("act", [0, 1, 2, 10, 11, 12])
+@pytest.mark.parametrize("accumulate", [0, 1])
+def test_fc_split_epilogue(pkg, dsx, orc, rng, act, accumulate):
+    B, k, n = 70, 48, 150
+    X = rng.standard_normal((B, k)).astype(np.float32)
+    W = (rng.standard_normal((k, n)) * 0.3).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    Z0 = rng.standard_normal((B, n)).astype(np.float32)
+    params = pkg.ActParams(0.2, 1.5, 1.05)
+    dX, dW, db = dev(pkg, X), dev(pkg, W), dev(pkg, bias)
+    xp = planes_of(pkg, dsx, dX, k, 0, B, k)
+    wp = planes_of(pkg, dsx, dW, n, 1, n, k)
+    Z = pkg.DeviceArray.from_numpy(Z0)
+    pkg.check(dsx.dsx_fc_forward_split(xp.ptr, wp.ptr, db.ptr, Z.ptr, n, B, k, n, accumulate, act, C.byref(params), None, None))
+    pre = orc.clear_unit([bias], n, B) + (Z0 if accumulate else 0)
+    ref = orc.activation(orc.sgemm_acc(X, W, pre), act, 0.2, 1.5, 1.05)
+    # (sums of 48 products of size 0.3 that cancel to almost nothing carry the rounding of their terms: 1e-4 of a tenth of a typical sum)
+    assert_close(Z.numpy(), ref, "split fc epilogue", rel=1e-4, abs_floor=0.1)
+
+
+def test_fc_split_transposed_weights_and_pitched_input(pkg, dsx, orc, rng):
+    B, k, n = 90, 70, 130
+    X = rng.standard_normal((B, k + 6)).astype(np.float32)       # row pitch larger than k
+    Wt = (rng.standard_normal((n, k)) * 0.2).astype(np.float32)  # [n][k]: shared transposed weight (engine/NNLayer.cpp:1065-1072)
+    dX, dW = dev(pkg, X), dev(pkg, Wt)
+    xp = planes_of(pkg, dsx, dX, k + 6, 0, B, k)
+    wp = planes_of(pkg, dsx, dW, k, 0, n, k)                      # a column of W is a row of the stored matrix
+    Z = pkg.DeviceArray.from_numpy(np.zeros((B, n), dtype=np.float32))
+    pkg.check(dsx.dsx_fc_forward_split(xp.ptr, wp.ptr, None, Z.ptr, n, B, k, n, 0, 3, None, None, None))
+    ref = orc.sgemm_acc(np.ascontiguousarray(X[:, :k]), Wt, np.zeros((B, n), dtype=np.float32), transposed=True)
+    assert_close(Z.numpy(), ref, "split fc, transposed weights", rel=1e-4, abs_floor=0.5)
+
+
+def test_fc_split_segment_maxima_and_arguments(pkg, dsx, rng):
+    B, k, n = 200, 64, 1000
+    X = rng.standard_normal((B, k)).astype(np.float32)
+    W = (rng.standard_normal((k, n)) * 0.2).astype(np.float32)
+    dX, dW = dev(pkg, X), dev(pkg, W)
+    xp = planes_of(pkg, dsx, dX, k, 0, B, k)
+    wp = planes_of(pkg, dsx, dW, n, 1, n, k)
+    Z = pkg.DeviceArray((B, n), np.float32)
+    nseg = (n + 63) // 64
+    sm = pkg.DeviceArray((B, nseg), np.float32)
+    sw = C.c_uint32(7)
+    pkg.check(dsx.dsx_fc_forward_split(xp.ptr, wp.ptr, None, Z.ptr, n, B, k, n, 0, 0, None, sm.ptr, C.byref(sw)))
+    assert sw.value == 64
+    unit = Z.numpy()
+    pad = np.full((B, nseg * 64), -np.inf, dtype=np.float32)
+    pad[:, :n] = unit
+    assert np.array_equal(sm.numpy(), pad.reshape(B, nseg, 64).max(axis=2))
+    # argument errors are reported, not run
+    assert dsx.dsx_fc_forward_split(None, wp.ptr, None, Z.ptr, n, B, k, n, 0, 0, None, None, None) != 0
+    assert dsx.dsx_fc_forward_split(xp.ptr, wp.ptr, None, Z.ptr, n - 1, B, k, n, 0, 0, None, None, None) != 0
+    assert dsx.dsx_fc_forward_split(xp.ptr, wp.ptr, None, Z.ptr, n, B, k, n, 0, 7, None, None, None) != 0      # softmax is a row operation
+    assert dsx.dsx_fc_forward_split(xp.ptr, wp.ptr, None, Z.ptr, n, B, k, n, 0, 0, None, sm.ptr, None) != 0
+    assert dsx.dsx_fc_split(dX.ptr, k - 1, 0, B, k, xp.ptr) != 0
+    assert dsx.dsx_fc_forward_split(xp.ptr, wp.ptr, None, Z.ptr, n, 0, k, n, 0, 0, None, None, None) == 0       # empty batch: nothing to do
+
+
+def test_cfg2_with_split_products_matches_the_oracle(pkg, dsx, orc, synth):
+    """Config 2 end to end with the output layer in this mode, scanning and guided top-K: activations within 1e-4 of the oracle's,
+    indexes the oracle's except where its scores are closer than 1e-5."""
+    from amazon_dsstne_amd.pipeline import DevicePipeline
+    p = synth.config(2)
+    _, ref_unit, _, _ = orc.forward(p, 0, None, filtered=False, want_unit=True, want_topk=False)
+    _, _, ref_keys, ref_idx = orc.forward(p, 0, None, filtered=True)
+    ref_scores = ref_unit.copy()
+    orc.lib().orc_apply_filter(ref_scores.ctypes.data, p.batch, ref_scores.shape[1], 0, 0, None, p.start.ctypes.data, p.end.ctypes.data,
+                               p.sparse_index.ctypes.data, None)
+    for guided in (False, True):
+        pipe = DevicePipeline(p, dsx, guided=guided, split=True)
+        pipe.step()
+        keys, idx = pipe.results()
+        unit = pipe.output_unit()
+        assert_units_close(unit, ref_unit, p, 0, "cfg2 output activations (split products)")
+        nd = assert_topk_parity(keys, idx, ref_keys, ref_idx, ref_scores, "cfg2 split products guided=%s" % guided)
+        say("cfg2 split products, guided=%s: parity ok (%d tie-equivalent index differences)" % (guided, nd))
+        rows = np.arange(p.batch)[:, None]
+        assert np.array_equal(unit[rows, idx], keys)
