@@ -71,6 +71,7 @@ private:
     struct LaneSet {
         unique_ptr<GpuBuffer<NNFloat>> unit;
         unique_ptr<GpuBuffer<NNFloat>> segMax;
+        unique_ptr<GpuBuffer<uint32_t>> splitInput;
         uint32_t segWidth = 0;
         bool deferred = false;
         uint32_t deferredBatch = 0;
@@ -83,6 +84,17 @@ private:
     // whoever asks for the units themselves (NNNetwork::GetUnitBuffer, GetUnits) has them computed at that moment (Materialise).
     // _deferred: the units of the current batch have not been computed yet; _deferredBatch: its rows.
     bool _bDeferOutput = true;   // NNNetwork::SetDeferredOutput
+    // NNNetwork::SetSplitProducts: this layer's input as bf16 planes (dsx_fc_split), written before the layer's kernel on the
+    // same stream; one buffer per lane, like the units.
+    bool _bSplitProducts = false;
+    uint32_t _splitMinTiles = 0;
+    unique_ptr<GpuBuffer<uint32_t>> _pbSplitInput;
+    bool UseSplitProducts(uint32_t batch) const
+    {
+        return _bSplitProducts && (uint64_t)((batch + 127) / 128) * ((_localStride + 127) / 128) >= _splitMinTiles;
+    }
+    // Z = act(bias + X.W) of a single-source layer through dsx_fc_split + dsx_fc_forward_split (segment maxima on request).
+    void ForwardSplit(uint32_t batch, NNFloat* pSegMax, uint32_t* pSegWidth);
     bool _deferred = false;
     uint32_t _deferredBatch = 0;
     void Materialise();
@@ -92,12 +104,14 @@ private:
         LaneSet& mine = _parked[_currentLane];
         mine.unit.swap(_pbUnit);
         mine.segMax.swap(_pbSegMax);
+        mine.splitInput.swap(_pbSplitInput);
         mine.segWidth = _segWidth;
         mine.deferred = _deferred;
         mine.deferredBatch = _deferredBatch;
         LaneSet& next = _parked[lane];
         _pbUnit.swap(next.unit);
         _pbSegMax.swap(next.segMax);
+        _pbSplitInput.swap(next.splitInput);
         _segWidth = next.segWidth;
         _deferred = next.deferred;
         _deferredBatch = next.deferredBatch;

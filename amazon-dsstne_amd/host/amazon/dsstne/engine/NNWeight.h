@@ -40,6 +40,13 @@ private:
     vector<NNFloat> _vBias;
     unique_ptr<GpuBuffer<NNFloat>> _pbWeight;
     unique_ptr<GpuBuffer<NNFloat>> _pbBias;
+    // NNNetwork::SetSplitProducts: the weights as three planes of bf16 (dsx_fc_split) for the dense kernel that forms its fp32
+    // products from bf16 matrix instructions; one set per orientation in which layers use the matrix ([0]: stored [k][n],
+    // [1]: stored [n][k]), built on first use and again after CopyWeights / SetWeights / Randomize / a load from file.
+    unique_ptr<GpuBuffer<uint32_t>> _pbSplit[2];
+    bool _bSplitValid[2] = {false, false};
+    const void* SplitPlanes(bool bTransposed, uint32_t k, uint32_t n);
+    void InvalidateSplit() { _bSplitValid[0] = _bSplitValid[1] = false; }
 
     NNWeight(NNLayer& inputLayer, NNLayer& outputLayer, bool bShared = false, bool bTransposed = false, bool bLocked = false,
              NNFloat maxNorm = 0.0f);

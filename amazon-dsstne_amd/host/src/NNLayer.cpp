@@ -166,7 +166,7 @@ void NNLayer::ForwardPropagateFullyConnected(uint32_t position, uint32_t batch, 
         } else if (_kind == Output && _localStride >= kSegMaxMinWidth) {
             // Wide output layer that feeds no other layer: what usually follows is a top-K, which can run together with the layer
             // without the layer's result ever being stored.  The layer is computed when somebody asks for it.
-            if (_bDeferOutput && _localStride >= kDeferMinWidth && !w->_bTransposed && _vOutgoingLayer.empty() && _vOutgoingSkip.empty() &&
+            if (_bDeferOutput && !UseSplitProducts(batch) && _localStride >= kDeferMinWidth && !w->_bTransposed && _vOutgoingLayer.empty() && _vOutgoingSkip.empty() &&
                 dsx_fc_topk_supported(src->_stride, src->GetUnitBuffer(), (uint32_t)_activation, &params, NULL)) {
                 if (dsx_fc_topk_flagged(0)) {
                     // rows whose survivor lists filled up had to be recomputed one by one: this data (thousands of scores tied at the
@@ -181,6 +181,8 @@ void NNLayer::ForwardPropagateFullyConnected(uint32_t position, uint32_t batch, 
             }
             _deferredBatch = batch;
             Materialise();
+        } else if (UseSplitProducts(batch)) {
+            ForwardSplit(batch, NULL, NULL);
         } else {
             dsxFatal(dsx_fc_forward(src->GetUnitBuffer(), src->_stride, wsrc->_pbWeight->_pDevData, w->_bTransposed ? 1 : 0,
                                     w->_pbBias->_pDevData, pUnit, _stride, batch, src->_stride, _localStride, 0, (uint32_t)_activation, &params),
@@ -218,9 +220,29 @@ void NNLayer::Materialise()
     dsx_act_params params = {_RELUSlope, _ELUAlpha, _SELULambda};
     const size_t need = (size_t)_batch * ((_localStride + 63) / 64);
     if (!_pbSegMax || _pbSegMax->_length < need) _pbSegMax.reset(new GpuBuffer<NNFloat>(need));
+    if (UseSplitProducts(_deferredBatch)) {
+        ForwardSplit(_deferredBatch, _pbSegMax->_pDevData, &_segWidth);
+        return;
+    }
     dsxFatal(dsx_fc_forward_segmax(src->GetUnitBuffer(), src->_stride, wsrc->_pbWeight->_pDevData, w->_bTransposed ? 1 : 0,
                                    w->_pbBias->_pDevData, GetIncomingUnitBuffer(), _stride, _deferredBatch, src->_stride, _localStride,
                                    (uint32_t)_activation, &params, _pbSegMax->_pDevData, &_segWidth),
+             "NNLayer::ForwardPropagate: GEMM failure");
+}
+
+void NNLayer::ForwardSplit(uint32_t batch, NNFloat* pSegMax, uint32_t* pSegWidth)
+{
+    NNLayer* src = _vIncomingLayer[0];
+    NNWeight* w = _vIncomingWeight[0];
+    NNWeight* wsrc = w->_bShared ? w->_pSharedWeight : w;
+    dsx_act_params params = {_RELUSlope, _ELUAlpha, _SELULambda};
+    const uint32_t k = src->_stride;
+    const void* pWeightPlanes = wsrc->SplitPlanes(w->_bTransposed, k, _localStride);
+    const size_t words = (size_t)(dsx_fc_split_bytes(_batch, k) / sizeof(uint32_t));
+    if (!_pbSplitInput || _pbSplitInput->_length < words) _pbSplitInput.reset(new GpuBuffer<uint32_t>(words));
+    dsxFatal(dsx_fc_split(src->GetUnitBuffer(), src->_stride, 0, batch, k, _pbSplitInput->_pDevData), "NNLayer::ForwardPropagate: input planes");
+    dsxFatal(dsx_fc_forward_split(_pbSplitInput->_pDevData, pWeightPlanes, w->_pbBias->_pDevData, GetIncomingUnitBuffer(), _stride, batch, k,
+                                  _localStride, 0, (uint32_t)_activation, &params, pSegMax, pSegWidth),
              "NNLayer::ForwardPropagate: GEMM failure");
 }
 

@@ -95,6 +95,7 @@ NNNetwork::NNNetwork(NNNetworkDescriptor& d, uint32_t batch)
                 fatal("NNNetwork::NNNetwork: too few weight values between layers %s and %s.", wd._inputLayer.c_str(), wd._outputLayer.c_str());
             std::copy(wd._vWeight.begin(), wd._vWeight.begin() + pWeight->_vWeight.size(), pWeight->_vWeight.begin());
             pWeight->_pbWeight->Upload(pWeight->_vWeight.data());
+            pWeight->InvalidateSplit();
         }
         if (!wd._vBias.empty()) {
             if (wd._vBias.size() < pWeight->_vBias.size())
@@ -320,6 +321,25 @@ void NNNetwork::LayerWithTopK(NNLayer* pLayer, uint32_t k, uint32_t batch, const
                          pLayer->_localStride, (uint32_t)pLayer->_activation, &params, k, pKey, pValue, _position, pIndex, pFilterStart,
                          pFilterEnd, pFilterIndex),
              "NNNetwork::CalculateTopK: output layer with top-K");
+}
+
+bool NNNetwork::SetSplitProducts(bool bSplit)
+{
+    dsx_device_info info;
+    dsxFatal(dsx_get_device_info(&info), "NNNetwork::SetSplitProducts");
+    for (auto l : _vLayer) {
+        l->_bSplitProducts = bSplit;
+        l->_splitMinTiles = 2u * info.compute_units;
+    }
+    // (also the way to say that weights were written through NNWeight::GetWeightBuffer: the planes are built again on next use)
+    for (auto w : _vWeight) {
+        w->InvalidateSplit();
+        if (!bSplit) {
+            w->_pbSplit[0].reset();
+            w->_pbSplit[1].reset();
+        }
+    }
+    return true;
 }
 
 bool NNNetwork::SetDeferredOutput(bool bDefer)

@@ -121,6 +121,7 @@ void NNWeight::Randomize()
             std::fill(_vWeight.begin(), _vWeight.end(), -shift);
         }
         _pbWeight->Upload(_vWeight.data());
+        InvalidateSplit();
     }
     std::fill(_vBias.begin(), _vBias.end(), _outputLayer._biasInit);
     _pbBias->Upload(_vBias.data());
@@ -141,6 +142,7 @@ bool NNWeight::CopyWeights(const NNWeight* pSrcWeight)
     pDstWeight->_vWeight = pSrc->_vWeight;
     _vBias = pSrcWeight->_vBias;
     if (pDstWeight->_pbWeight) pDstWeight->_pbWeight->Upload(pDstWeight->_vWeight.data());
+    pDstWeight->InvalidateSplit();
     if (_pbBias) _pbBias->Upload(_vBias.data());
     return true;
 }
@@ -154,7 +156,25 @@ bool NNWeight::SetWeights(const vector<NNFloat>& vWeight)
     }
     std::copy(vWeight.begin(), vWeight.begin() + pWeight->_vWeight.size(), pWeight->_vWeight.begin());
     if (pWeight->_pbWeight) pWeight->_pbWeight->Upload(pWeight->_vWeight.data());
+    pWeight->InvalidateSplit();
     return true;
+}
+
+// The matrix as dsx_fc_forward_split wants it, for a layer that multiplies [batch x k] inputs into n units: column j of the
+// product's W is row j of the planes.  Built on the calling lane's stream; every lane waits for it once (dsx_sync), after that
+// the planes are only read.
+const void* NNWeight::SplitPlanes(bool bTransposed, uint32_t k, uint32_t n)
+{
+    const int o = bTransposed ? 1 : 0;
+    if (!_bSplitValid[o]) {
+        const size_t words = (size_t)(dsx_fc_split_bytes(n, k) / sizeof(uint32_t));
+        if (!_pbSplit[o] || _pbSplit[o]->_length < words) _pbSplit[o].reset(new GpuBuffer<uint32_t>(words));
+        dsxFatal(dsx_fc_split(_pbWeight->_pDevData, bTransposed ? k : n, bTransposed ? 0 : 1, n, k, _pbSplit[o]->_pDevData),
+                 "NNWeight::SplitPlanes");
+        dsxFatal(dsx_sync(), "NNWeight::SplitPlanes");
+        _bSplitValid[o] = true;
+    }
+    return _pbSplit[o]->_pDevData;
 }
 
 bool NNWeight::SetBiases(const vector<NNFloat>& vBias)

@@ -381,6 +381,13 @@ int dsstne_set_lanes(dsstne_context* c, uint32_t lanes)
     CAPI_CATCH(-1)
 }
 
+int dsstne_set_split_products(dsstne_context* c, int split)
+{
+    CAPI_TRY
+    return c->net()->SetSplitProducts(split != 0) ? 0 : fail("dsstne_set_split_products failed");
+    CAPI_CATCH(-1)
+}
+
 int dsstne_set_deferred_output(dsstne_context* c, int defer)
 {
     CAPI_TRY

@@ -44,6 +44,7 @@ SIGNATURES = {
     "dsstne_get_topk_previous": ([_vp, _cp, _u32, _u32, _vp, _vp], _int),
     "dsstne_set_lanes": ([_vp, _u32], _int),
     "dsstne_set_deferred_output": ([_vp, _int], _int),
+    "dsstne_set_split_products": ([_vp, _int], _int),
     "dsstne_knn_create_typed": ([_u32, _u32, _cp], _vp),
     "dsstne_knn_search": ([_vp, _u32, _vp, _u32, _vp, _vp], _int),
     "dsstne_knn_elapsed": ([_vp, C.POINTER(_f32), C.POINTER(_f32)], _int),
@@ -158,6 +159,10 @@ class Network:
     def set_deferred_output(self, defer):
         """NNNetwork::SetDeferredOutput: False stores the output layer in predict_batch, as the reference does."""
         _check(self.lib.dsstne_set_deferred_output(self.ctx, 1 if defer else 0))
+
+    def set_split_products(self, split):
+        """NNNetwork::SetSplitProducts: True forms the wide dense layers' fp32 products from bf16 matrix instructions."""
+        _check(self.lib.dsstne_set_split_products(self.ctx, 1 if split else 0))
 
     def units(self, layer="Output", rows=None, width=None):
         width = width or self.p.widths[-1]

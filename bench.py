@@ -152,6 +152,13 @@ def network_bench(args, pkg, lib):
     settle(pkg, lib, step)
     ms_stored = float(np.median(timed_windows(step, net.sync, args.steps, 3)))
     net.set_deferred_output(True)
+    # ... and with the wide dense layers' fp32 products formed from bf16 matrix instructions (NNNetwork::SetSplitProducts: three
+    # bf16 planes per operand, six MFMA terms per product, fp32 sums; as close to fp64 as the fp32 kernel, not bit-identical to
+    # it).  A mode the caller asks for: reported beside `value`, never as `value`.
+    net.set_split_products(True)
+    settle(pkg, lib, step)
+    ms_split = float(np.median(timed_windows(step, net.sync, args.steps, 3)))
+    net.set_split_products(False)
     net.sync()
     net.close()
 
@@ -352,6 +359,9 @@ def network_bench(args, pkg, lib):
                      "note": "NNNetwork::SetLanes(1): one set of buffers, one stream, batches strictly one after the other"},
         "stored_output": {"ms_per_step": round(ms_stored, 5), "value": rate(ms_stored), "unit": "samples/s",
                           "note": "NNNetwork::SetDeferredOutput(false): PredictBatch stores the output layer, the top-K reads it back (the same as the default below 131,072 output units)"},
+        "split_products": {"ms_per_step": round(ms_split, 5), "value": rate(ms_split), "unit": "samples/s",
+                           "dtype": "f32 products as six bf16 x bf16 MFMA terms, f32 sums",
+                           "note": "NNNetwork::SetSplitProducts(true), off by default: dense layers of at least two 128 x 128 tiles per compute unit run fc_gemm_split_kernel (a wide output layer is then always stored); results within the same tolerance of the oracle, as close to fp64 as the fp32 kernel's"},
         "with_input_upload": {"ms_per_step": round(ms_upload, 5), "value": rate(ms_upload), "unit": "samples/s",
                               "note": "the batch's CSR arrays handed over as host memory before every step (NNDataSet::LoadSparseData; PCIe-inclusive): uploads go to alternating sets of device arrays on the lane of the batch they belong to"},
         "request_round_trip": {"ms": round(ms_request, 5), "value": rate(ms_request), "unit": "samples/s",

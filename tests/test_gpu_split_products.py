@@ -184,3 +184,63 @@ def test_cfg2_with_split_products_matches_the_oracle(pkg, dsx, orc, synth):
         say("cfg2 split products, guided=%s: parity ok (%d tie-equivalent index differences)" % (guided, nd))
         rows = np.arange(p.batch)[:, None]
         assert np.array_equal(unit[rows, idx], keys)
+
+
+def host_forward_split(orc, p, lanes=2, batches=(0,)):
+    """PredictBatch + filtered top-K through the class API with NNNetwork::SetSplitProducts(true), compared with the oracle."""
+    from amazon_dsstne_amd import host_api
+    net = host_api.Network(p, max_k=p.k)
+    try:
+        net.set_lanes(lanes)
+        net.set_split_products(True)
+        net.bind_input()
+        for position in batches:
+            rows = min(p.batch, p.examples - position)
+            net.predict_batch(position)
+            net.topk(p.k, filter_dataset="input")
+            keys, idx = net.get_topk(rows)
+            unit = net.units(rows=p.batch)[:rows]
+            _, ref_unit, _, _ = orc.forward(p, position, rows, filtered=False, want_unit=True, want_topk=False)
+            _, _, ref_keys, ref_idx = orc.forward(p, position, rows, filtered=True)
+            assert_units_close(unit, ref_unit, p, position, p.name + " units, split products")
+            ref_scores = ref_unit.copy()
+            orc.lib().orc_apply_filter(ref_scores.ctypes.data, rows, ref_scores.shape[1], 0, position,
+                                       p.index.ctypes.data if p.index is not None else None, p.start.ctypes.data, p.end.ctypes.data,
+                                       p.sparse_index.ctypes.data, None)
+            nd = assert_topk_parity(keys, idx, ref_keys, ref_idx, ref_scores, p.name + " split products")
+            say("%s at %d, %d lanes, split products through NNNetwork: parity ok (%d tie-equivalent)" % (p.name, position, lanes, nd))
+        return net
+    except Exception:
+        net.close()
+        raise
+
+
+def test_network_api_split_products_cfg2(pkg, dsx, orc, synth):
+    p = synth.config(2, batches=3)
+    for lanes in (1, 2):
+        host_forward_split(orc, p, lanes=lanes, batches=(0, 1024, 2048)).close()
+
+
+def test_network_api_split_products_hidden_layer_and_new_weights(pkg, dsx, orc, synth):
+    """A network whose hidden layers are wide enough for the mode too (4096 rows x 2048 units: 512 tiles of 128 x 128), and weights replaced
+    after the planes were built: the next batch must be computed from the new weights."""
+    p = synth.autoencoder("split-wide-hidden", 31, 5000, [256, 2048], 4096, 10, 1, 1.0, 40, 0.8, (1, 300), bias_std=0.1)
+    net = host_forward_split(orc, p)
+    try:
+        rng = np.random.default_rng(5)
+        p.weights[1] = (rng.standard_normal(p.weights[1].shape) * 0.02).astype(np.float32)
+        p.weights[2] = (rng.standard_normal(p.weights[2].shape) * 0.02).astype(np.float32)
+        net.set_weights("Hidden1", "Hidden2", weights=p.weights[1])
+        net.set_weights("Hidden2", "Output", weights=p.weights[2])
+        net.predict_batch(0)
+        unit = net.units(rows=p.batch)
+        _, ref_unit, _, _ = orc.forward(p, 0, p.batch, filtered=False, want_unit=True, want_topk=False)
+        assert_units_close(unit, ref_unit, p, 0, "units after SetWeights, split products")
+        # and back: the fp32 kernels give the same within the tolerance
+        net.set_split_products(False)
+        net.predict_batch(0)
+        plain = net.units(rows=p.batch)
+        assert_units_close(plain, ref_unit, p, 0, "units with the mode switched off again")
+        assert not np.array_equal(plain, unit)          # (the two modes round differently: the first pass did take the other kernel)
+    finally:
+        net.close()
