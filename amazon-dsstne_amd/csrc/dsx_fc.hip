@@ -743,17 +743,28 @@ __global__ __launch_bounds__(kFcThreads, 3) void fc_gemm_split_kernel(FcArgs a, 
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
+    // Every load is "plane base (uniform) + this lane's 32-bit byte offset", the offset advancing by a uniform step per k-step
+    // (a plane is smaller than 4 GiB, the host checks): two vector additions per step instead of 64-bit address arithmetic.
     const int srow = tid & 127, shalf = tid >> 7;
-    const uint64_t xplane = (uint64_t)sp.kblocks * sp.xrows, wplane = (uint64_t)sp.kblocks * sp.wrows;
-    const u32x4* xa = sp.Xs + (uint64_t)shalf * sp.xrows + row0 + srow;
-    const u32x4* wb = sp.Ws + (uint64_t)shalf * sp.wrows + col0 + srow;
+    const uint64_t xplane = (uint64_t)sp.kblocks * sp.xrows * 16, wplane = (uint64_t)sp.kblocks * sp.wrows * 16;
+    const char* xbase[3];
+    const char* wbase[3];
+#pragma unroll
+    for (int p = 0; p < 3; p++) {
+        xbase[p] = reinterpret_cast<const char*>(sp.Xs) + p * xplane;
+        wbase[p] = reinterpret_cast<const char*>(sp.Ws) + p * wplane;
+    }
+    uint32_t xoff = (shalf * sp.xrows + row0 + srow) * 16u, woff = (shalf * sp.wrows + col0 + srow) * 16u;
+    const uint32_t xstep = 2u * sp.xrows * 16u, wstep = 2u * sp.wrows * 16u;
     u32x4 ra[3], rb[3];
-    auto load = [&](uint32_t kt) __attribute__((always_inline)) {
+    auto load = [&]() __attribute__((always_inline)) {   // the next k-step's units
 #pragma unroll
         for (int p = 0; p < 3; p++) {
-            ra[p] = xa[p * xplane + (uint64_t)(2 * kt) * sp.xrows];
-            rb[p] = wb[p * wplane + (uint64_t)(2 * kt) * sp.wrows];
+            ra[p] = *reinterpret_cast<const u32x4*>(xbase[p] + xoff);
+            rb[p] = *reinterpret_cast<const u32x4*>(wbase[p] + woff);
         }
+        xoff += xstep;
+        woff += wstep;
     };
     auto store = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
@@ -779,13 +790,18 @@ __global__ __launch_bounds__(kFcThreads, 3) void fc_gemm_split_kernel(FcArgs a, 
 #undef DSX_TERM
     };
     const uint32_t nk = sp.kblocks / 2;
-    load(0);
+    load();
     store(0);
     __syncthreads();
     for (uint32_t kt = 0; kt < nk; kt++) {
         const int buf = kt & 1;
-        // (unconditional, so that the staging registers stay registers: the last step's reload goes where nobody reads it)
-        load(kt + 1 < nk ? kt + 1 : kt);
+        // (unconditional, so that the staging registers stay registers: the last step loads its own units again, and they go
+        // where nobody reads them)
+        if (kt + 1 == nk) {
+            xoff -= xstep;
+            woff -= wstep;
+        }
+        load();
         multiply(buf);
         store(buf ^ 1);
         __syncthreads();
@@ -831,6 +847,9 @@ static int fc_split_run(const void* Xs, const void* Ws, const float* bias, float
     }
     FcSplitArgs sp{reinterpret_cast<const u32x4*>(Xs), reinterpret_cast<const u32x4*>(Ws), split_rows_padded(batch), split_rows_padded(n),
                    split_kblocks(k)};
+    if ((uint64_t)sp.kblocks * sp.xrows * 16 >= (1ull << 32) || (uint64_t)sp.kblocks * sp.wrows * 16 >= (1ull << 32)) {
+        return set_error(DSX_EINVAL, "dsx_fc_forward_split: a plane of 4 GiB or more (rows padded to 128 x k padded to 16 x 2 bytes)");
+    }
     const uint32_t total = a.tiles_m * a.tiles_n;
     const dim3 grid(((total + kXcds - 1) / kXcds) * kXcds);
     hipStream_t s = ctx().stream;
