@@ -713,12 +713,15 @@ struct FcSplitArgs {
 };
 
 // Z = act(acc? + bias + X . W) as fc_gemm_kernel<2, 2, ...> computes it (same tile order, same epilogue), from planes.
-// A k-step is one MFMA depth (16): 24 KiB of operands (3 planes x 2 blocks of k x (128 + 128) rows x 16 bytes), double
-// buffered in LDS; every lane moves one unit of each plane of each operand per step.
-template <int ACT>
-__global__ __launch_bounds__(kFcThreads, 3) void fc_gemm_split_kernel(FcArgs a, FcSplitArgs sp)
+// A k-step is one MFMA depth (16), its operand units double buffered in LDS.  MH = 1: a 128 x 128 tile, 2 x 2 wavefronts of
+// 64 x 64, 24 KiB of units per step, three workgroups per CU.  MH = 2: a 256 x 128 tile, wavefronts of 128 x 64 (eight
+// accumulators: 0.375 fragment reads per MFMA instead of 0.5, and three quarters of the operand traffic per product), 36 KiB
+// per step, two workgroups per CU.
+template <int ACT, int MH>
+__global__ __launch_bounds__(kFcThreads, MH == 1 ? 3 : 2) void fc_gemm_split_kernel(FcArgs a, FcSplitArgs sp)
 {
-    __shared__ u32x4 sA[2][3][2][128];
+    constexpr int BM = 128 * MH;
+    __shared__ u32x4 sA[2][3][2][BM];
     __shared__ u32x4 sB[2][3][2][128];
     const uint32_t total = a.tiles_m * a.tiles_n;
     uint32_t wg = blockIdx.x;
@@ -729,22 +732,25 @@ __global__ __launch_bounds__(kFcThreads, 3) void fc_gemm_split_kernel(FcArgs a, 
         if (local >= per_xcd || wg >= total) return;
     }
     const uint32_t tm = wg % a.tiles_m, tn = a.tiles_n - 1 - wg / a.tiles_m;
-    const uint32_t row0 = tm * 128, col0 = tn * 128;
+    const uint32_t row0 = tm * BM, col0 = tn * 128;
     __builtin_amdgcn_s_setprio(1);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, lhi = lane >> 5;
 
-    floatx16 acc[2][2];
+    floatx16 acc[MH][2][2];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int h = 0; h < MH; h++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int i = 0; i < 2; i++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[h][i][j][v] = 0.0f;
 
     // Every load is "plane base (uniform) + this lane's 32-bit byte offset", the offset advancing by a uniform step per k-step
     // (a plane is smaller than 4 GiB, the host checks): two vector additions per step instead of 64-bit address arithmetic.
+    // W: lane (half, row) moves one unit per plane.  X: the same for MH = 1; for MH = 2 a lane moves both halves of its row.
     const int srow = tid & 127, shalf = tid >> 7;
     const uint64_t xplane = (uint64_t)sp.kblocks * sp.xrows * 16, wplane = (uint64_t)sp.kblocks * sp.wrows * 16;
     const char* xbase[3];
@@ -754,13 +760,20 @@ __global__ __launch_bounds__(kFcThreads, 3) void fc_gemm_split_kernel(FcArgs a, 
         xbase[p] = reinterpret_cast<const char*>(sp.Xs) + p * xplane;
         wbase[p] = reinterpret_cast<const char*>(sp.Ws) + p * wplane;
     }
-    uint32_t xoff = (shalf * sp.xrows + row0 + srow) * 16u, woff = (shalf * sp.wrows + col0 + srow) * 16u;
+    uint32_t xoff = (MH == 1) ? (shalf * sp.xrows + row0 + srow) * 16u : (row0 + tid) * 16u;
+    uint32_t woff = (shalf * sp.wrows + col0 + srow) * 16u;
+    const uint32_t xhalf = sp.xrows * 16u;
     const uint32_t xstep = 2u * sp.xrows * 16u, wstep = 2u * sp.wrows * 16u;
-    u32x4 ra[3], rb[3];
+    u32x4 ra[3 * MH], rb[3];
     auto load = [&]() __attribute__((always_inline)) {   // the next k-step's units
 #pragma unroll
         for (int p = 0; p < 3; p++) {
-            ra[p] = *reinterpret_cast<const u32x4*>(xbase[p] + xoff);
+            if constexpr (MH == 1) {
+                ra[p] = *reinterpret_cast<const u32x4*>(xbase[p] + xoff);
+            } else {
+                ra[2 * p] = *reinterpret_cast<const u32x4*>(xbase[p] + xoff);
+                ra[2 * p + 1] = *reinterpret_cast<const u32x4*>(xbase[p] + xoff + xhalf);
+            }
             rb[p] = *reinterpret_cast<const u32x4*>(wbase[p] + woff);
         }
         xoff += xstep;
@@ -769,25 +782,35 @@ __global__ __launch_bounds__(kFcThreads, 3) void fc_gemm_split_kernel(FcArgs a, 
     auto store = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int p = 0; p < 3; p++) {
-            sA[buf][p][shalf][srow] = ra[p];
+            if constexpr (MH == 1) {
+                sA[buf][p][shalf][srow] = ra[p];
+            } else {
+                sA[buf][p][0][tid] = ra[2 * p];
+                sA[buf][p][1][tid] = ra[2 * p + 1];
+            }
             sB[buf][p][shalf][srow] = rb[p];
         }
     };
     auto multiply = [&](int buf) __attribute__((always_inline)) {
-        bf16x8 fa[2][3], fb[2][3];
+        bf16x8 fb[2][3];
 #pragma unroll
-        for (int p = 0; p < 3; p++) {
-#pragma unroll
-            for (int i = 0; i < 2; i++) fa[i][p] = __builtin_bit_cast(bf16x8, sA[buf][p][lhi][wm * 64 + i * 32 + l32]);
+        for (int p = 0; p < 3; p++)
 #pragma unroll
             for (int j = 0; j < 2; j++) fb[j][p] = __builtin_bit_cast(bf16x8, sB[buf][p][lhi][wn * 64 + j * 32 + l32]);
-        }
-        // (plane of X, plane of W): lo.hi, hi.lo, mid.mid, mid.hi, hi.mid, hi.hi
+#pragma unroll
+        for (int h = 0; h < MH; h++) {
+            bf16x8 fa[2][3];
+#pragma unroll
+            for (int p = 0; p < 3; p++)
+#pragma unroll
+                for (int i = 0; i < 2; i++) fa[i][p] = __builtin_bit_cast(bf16x8, sA[buf][p][lhi][wm * 64 * MH + h * 64 + i * 32 + l32]);
+            // (plane of X, plane of W): lo.hi, hi.lo, mid.mid, mid.hi, hi.mid, hi.hi; the four accumulators take turns
 #define DSX_TERM(PX, PW)                                                                                                   \
     _Pragma("unroll") for (int i = 0; i < 2; i++) _Pragma("unroll") for (int j = 0; j < 2; j++)                            \
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][PX], fb[j][PW], acc[i][j], 0, 0, 0);
-        DSX_TERM(2, 0) DSX_TERM(0, 2) DSX_TERM(1, 1) DSX_TERM(1, 0) DSX_TERM(0, 1) DSX_TERM(0, 0)
+        acc[h][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i][PX], fb[j][PW], acc[h][i][j], 0, 0, 0);
+            DSX_TERM(2, 0) DSX_TERM(0, 2) DSX_TERM(1, 1) DSX_TERM(1, 0) DSX_TERM(0, 1) DSX_TERM(0, 0)
 #undef DSX_TERM
+        }
     };
     const uint32_t nk = sp.kblocks / 2;
     load();
@@ -809,11 +832,13 @@ __global__ __launch_bounds__(kFcThreads, 3) void fc_gemm_split_kernel(FcArgs a, 
     __builtin_amdgcn_s_setprio(0);
     static_assert(sizeof(sA) >= 2 * 512 * sizeof(float) && sizeof(sB) >= 2 * 512 * sizeof(float),
                   "the segment maxima are transposed through the operand tiles' LDS, two wavefronts in each");
-    fc_epilogue<2, 2, ACT>(acc, a, row0 + wm * 64, col0 + wn * 64, lane,
-                           reinterpret_cast<float*>((wave < 2) ? &sA[0][0][0][0] : &sB[0][0][0][0]) + (wave & 1) * 512);
+    float* sT = reinterpret_cast<float*>((wave < 2) ? &sA[0][0][0][0] : &sB[0][0][0][0]) + (wave & 1) * 512;
+#pragma unroll
+    for (int h = 0; h < MH; h++) fc_epilogue<2, 2, ACT>(acc[h], a, row0 + wm * 64 * MH + h * 64, col0 + wn * 64, lane, sT);
 }
 
-static inline uint32_t split_rows_padded(uint32_t rows) { return (rows + 127) / 128 * 128; }
+static uint32_t g_split_tile_rows = 0;   // dsx_fc_split_set_tile_rows: 0 = by shape
+static inline uint32_t split_rows_padded(uint32_t rows) { return (rows + 255) / 256 * 256; }
 static inline uint32_t split_kblocks(uint32_t k) { return (k + 15) / 16 * 2; }
 
 static int fc_split_planes_run(const float* src, uint64_t stride_r, uint64_t stride_k, uint32_t rows, uint32_t k, void* planes)
@@ -838,8 +863,12 @@ static int fc_split_run(const void* Xs, const void* Ws, const float* bias, float
     a.slope = params ? params->slope : 0.01f;
     a.alpha = params ? params->alpha : 1.0f;
     a.lambda = params ? params->lambda : 1.0f;
-    a.tiles_m = (batch + 127) / 128;
     a.tiles_n = (n + 127) / 128;
+    // 256-row tiles for long sums, when they still give every CU its two workgroups twice over (4,096 x 512 x 262,144: 5,410
+    // against 5,730 us; with k = 128 the epilogue dominates and the smaller tiles' third workgroup per CU is worth more)
+    int mh = (k >= 512 && (uint64_t)((batch + 255) / 256) * a.tiles_n >= 4ull * ctx().num_cus) ? 2 : 1;
+    if (g_split_tile_rows) mh = g_split_tile_rows == 256 ? 2 : 1;
+    a.tiles_m = (batch + 128 * mh - 1) / (128 * mh);
     if (seg_max && seg_width && !accumulate) {
         a.seg_max = seg_max;
         a.nseg = (n + 63) / 64;
@@ -853,7 +882,11 @@ static int fc_split_run(const void* Xs, const void* Ws, const float* bias, float
     const uint32_t total = a.tiles_m * a.tiles_n;
     const dim3 grid(((total + kXcds - 1) / kXcds) * kXcds);
     hipStream_t s = ctx().stream;
-#define DSX_ACT_CASE(A) case A: hipLaunchKernelGGL((fc_gemm_split_kernel<A>), grid, dim3(kFcThreads), 0, s, a, sp); break;
+#define DSX_ACT_CASE(A)                                                                                      \
+    case A:                                                                                                  \
+        if (mh == 2) hipLaunchKernelGGL((fc_gemm_split_kernel<A, 2>), grid, dim3(kFcThreads), 0, s, a, sp); \
+        else hipLaunchKernelGGL((fc_gemm_split_kernel<A, 1>), grid, dim3(kFcThreads), 0, s, a, sp);         \
+        break;
     switch (a.act) {
         DSX_ACT_CASE(DSX_ACT_SIGMOID)
         DSX_ACT_CASE(DSX_ACT_TANH)
@@ -861,7 +894,10 @@ static int fc_split_run(const void* Xs, const void* Ws, const float* bias, float
         DSX_ACT_CASE(DSX_ACT_LRELU)
         DSX_ACT_CASE(DSX_ACT_ELU)
         DSX_ACT_CASE(DSX_ACT_SELU)
-    default: hipLaunchKernelGGL((fc_gemm_split_kernel<DSX_ACT_LINEAR>), grid, dim3(kFcThreads), 0, s, a, sp); break;
+    default:
+        if (mh == 2) hipLaunchKernelGGL((fc_gemm_split_kernel<DSX_ACT_LINEAR, 2>), grid, dim3(kFcThreads), 0, s, a, sp);
+        else hipLaunchKernelGGL((fc_gemm_split_kernel<DSX_ACT_LINEAR, 1>), grid, dim3(kFcThreads), 0, s, a, sp);
+        break;
     }
 #undef DSX_ACT_CASE
     DSX_LAUNCH_CHECK("fc_gemm_split_kernel");
@@ -945,6 +981,13 @@ int dsx_fc_split(const float* src, uint32_t ld, int k_major, uint32_t rows, uint
     DSX_CHECK_ARG(((uintptr_t)planes % 16) == 0, "dsx_fc_split: planes must be 16-byte aligned");
     DSX_CHECK_ARG(rows > 0 && k > 0 && ld >= (k_major ? rows : k), "dsx_fc_split: rows = %u, k = %u, ld = %u", rows, k, ld);
     return k_major ? fc_split_planes_run(src, 1, ld, rows, k, planes) : fc_split_planes_run(src, ld, 1, rows, k, planes);
+}
+
+int dsx_fc_split_set_tile_rows(uint32_t rows)
+{
+    if (rows != 0 && rows != 128 && rows != 256) return set_error(DSX_EINVAL, "dsx_fc_split_set_tile_rows: %u (0, 128 or 256)", rows);
+    g_split_tile_rows = rows;
+    return DSX_OK;
 }
 
 int dsx_fc_forward_split(const void* x_planes, const void* w_planes, const float* bias, float* Z, uint32_t ldz, uint32_t batch, uint32_t k,

@@ -92,8 +92,8 @@ private:
     bool UseSplitProducts(uint32_t batch) const
     {
         if (!_bSplitProducts || _vIncomingLayer.empty()) return false;
-        // (a plane of the kernel's operands stays below 4 GiB: 2 bytes x inputs padded to 16 x units padded to 128)
-        const uint64_t plane = 2ull * ((_vIncomingLayer[0]->_stride + 15) / 16 * 16) * ((uint64_t)(_localStride + 127) / 128 * 128);
+        // (a plane of the kernel's operands stays below 4 GiB: 2 bytes x inputs padded to 16 x units padded to 256)
+        const uint64_t plane = 2ull * ((_vIncomingLayer[0]->_stride + 15) / 16 * 16) * ((uint64_t)(_localStride + 255) / 256 * 256);
         return plane < (1ull << 32) && (uint64_t)((batch + 127) / 128) * ((_localStride + 127) / 128) >= _splitMinTiles;
     }
     // Z = act(bias + X.W) of a single-source layer through dsx_fc_split + dsx_fc_forward_split (segment maxima on request).

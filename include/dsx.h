@@ -216,12 +216,17 @@ int dsx_fc_forward_segmax(const float* X, uint32_t ldx, const float* W, int tran
  *   k_major == 0: vector r is src[r * ld + 0 .. k)        (X, a [batch x k] unit buffer; W stored [n x k], i.e. transposed)
  *   k_major != 0: vector r is src[0 .. k) * ld + r         (W stored [k x n])
  * into `planes`, dsx_fc_split_bytes(rows, k) bytes of 16-byte aligned device memory (3 x 2 bytes per value, rows padded to
- * 128 and k to 16).  Weights are split once, a layer's input once per batch.  Inf and NaN inputs stay Inf / NaN; finite values
+ * 256 and k to 16).  Weights are split once, a layer's input once per batch.  Inf and NaN inputs stay Inf / NaN; finite values
  * from 3.0e38 up are kept to bf16 precision only.
  * dsx_fc_forward_split then computes Z as dsx_fc_forward (accumulate, bias, activation) and, with seg_max / seg_width non-NULL
- * and accumulate == 0, the segment maxima as dsx_fc_forward_segmax (*seg_width = 64 for every shape). */
+ * and accumulate == 0, the segment maxima as dsx_fc_forward_segmax (*seg_width = 64 for every shape).  A plane (2 bytes x rows
+ * padded x k padded) must stay below 4 GiB.
+ * dsx_fc_split_set_tile_rows(128 | 256) fixes the rows of a workgroup's tile (tests reach both kernels with small shapes);
+ * 0, the default, chooses by shape: 256 for k >= 512 when that still leaves four tiles per compute unit.  Results do not
+ * depend on it. */
 uint64_t dsx_fc_split_bytes(uint32_t rows, uint32_t k);
 int dsx_fc_split(const float* src, uint32_t ld, int k_major, uint32_t rows, uint32_t k, void* planes);
+int dsx_fc_split_set_tile_rows(uint32_t rows);
 int dsx_fc_forward_split(const void* x_planes, const void* w_planes, const float* bias, float* Z, uint32_t ldz, uint32_t batch, uint32_t k,
                          uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params, float* seg_max,
                          uint32_t* seg_width);

@@ -29,7 +29,7 @@ def planes_of(pkg, dsx, d, ld, k_major, rows, k):
 
 def bf16_planes_to_float(words, rows, k):
     """Undo the layout of dsx_fc_split on the host: returns the three planes as float64 arrays [rows][k]."""
-    rp, kb = (rows + 127) // 128 * 128, (k + 15) // 16 * 2
+    rp, kb = (rows + 255) // 256 * 256, (k + 15) // 16 * 2
     halves = words.view(np.uint16).reshape(3, kb, rp, 8)
     f = (halves.astype(np.uint32) << 16).view(np.float32).astype(np.float64)      # [p][kb][r][8]
     f = f.transpose(0, 2, 1, 3).reshape(3, rp, kb * 8)
@@ -78,9 +78,22 @@ def test_split_planes_special_values(pkg, dsx):
 SHAPES = [(300, 100, 1000), (130, 17, 257), (1, 128, 129), (257, 130, 128), (64, 512, 3000), (1024, 128, 5000)]
 
 
+@pytest.fixture(params=[128, 256])
+def tile_rows(request, pkg, dsx):
+    """Both tile heights of the kernel on every shape (by itself it takes 256 rows only for long sums over many tiles)."""
+    pkg.check(dsx.dsx_fc_split_set_tile_rows(request.param))
+    yield request.param
+    pkg.check(dsx.dsx_fc_split_set_tile_rows(0))
+
+
+def test_fc_split_tile_rows_argument(pkg, dsx):
+    assert dsx.dsx_fc_split_set_tile_rows(64) != 0
+    pkg.check(dsx.dsx_fc_split_set_tile_rows(0))
+
+
 @pytest.mark.parametrize("B,k,n", SHAPES)
-def test_fc_split_vs_oracle_fp64_and_fp32_kernel(pkg, dsx, orc, rng, B, k, n):
-    say("fc_forward_split B=%d k=%d n=%d" % (B, k, n))
+def test_fc_split_vs_oracle_fp64_and_fp32_kernel(pkg, dsx, orc, rng, tile_rows, B, k, n):
+    say("fc_forward_split B=%d k=%d n=%d, tiles of %d rows" % (B, k, n, tile_rows))
     X = (rng.standard_normal((B, k)) * np.exp(rng.standard_normal((B, k)))).astype(np.float32)
     W = (rng.standard_normal((k, n)) * 0.1).astype(np.float32)
     bias = rng.standard_normal(n).astype(np.float32)
@@ -107,7 +120,7 @@ def test_fc_split_vs_oracle_fp64_and_fp32_kernel(pkg, dsx, orc, rng, B, k, n):
 
 @pytest.mark.parametrize("act", [0, 1, 2, 10, 11, 12])
 @pytest.mark.parametrize("accumulate", [0, 1])
-def test_fc_split_epilogue(pkg, dsx, orc, rng, act, accumulate):
+def test_fc_split_epilogue(pkg, dsx, orc, rng, tile_rows, act, accumulate):
     B, k, n = 70, 48, 150
     X = rng.standard_normal((B, k)).astype(np.float32)
     W = (rng.standard_normal((k, n)) * 0.3).astype(np.float32)
@@ -138,8 +151,8 @@ def test_fc_split_transposed_weights_and_pitched_input(pkg, dsx, orc, rng):
     assert_close(Z.numpy(), ref, "split fc, transposed weights", rel=1e-4, abs_floor=0.5)
 
 
-def test_fc_split_segment_maxima_and_arguments(pkg, dsx, rng):
-    B, k, n = 200, 64, 1000
+def test_fc_split_segment_maxima_and_arguments(pkg, dsx, rng, tile_rows):
+    B, k, n = 300, 64, 1000
     X = rng.standard_normal((B, k)).astype(np.float32)
     W = (rng.standard_normal((k, n)) * 0.2).astype(np.float32)
     dX, dW = dev(pkg, X), dev(pkg, W)
