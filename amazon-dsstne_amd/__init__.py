@@ -103,14 +103,16 @@ SIGNATURES = {
     "dsx_knn_set_block_columns": [_u32],
     "dsx_knn_f16_convert_items": [_vp, _u32, _u32, _u32, _vp],
     "dsx_knn_search_f16": [_vp, _u32, _u32, _u32, _vp, _u32, _u32, _vp, _vp, _vp, _sz, C.POINTER(_f32)],
+    "dsx_knn_search_split": [_vp, _u32, _u32, _u32, _vp, _u32, _u32, _vp, _vp, _vp, _sz, C.POINTER(_f32)],
     "dsx_knn_last_search_path": [],
     "dsx_knn_f16_set_sweep": [_int],
 }
 SPECIAL_RESTYPES = {"dsx_last_error": C.c_char_p, "dsx_stream": C.c_void_p, "dsx_knn_workspace_bytes": C.c_size_t,
-                    "dsx_knn_workspace_bytes_f16": C.c_size_t, "dsx_knn_f16_table_bytes": C.c_size_t, "dsx_fc_split_bytes": _u64}
+                    "dsx_knn_workspace_bytes_f16": C.c_size_t, "dsx_knn_f16_table_bytes": C.c_size_t, "dsx_fc_split_bytes": _u64,
+                    "dsx_knn_workspace_bytes_split": C.c_size_t}
 SPECIAL_ARGTYPES = {"dsx_last_error": [], "dsx_stream": [], "dsx_knn_workspace_bytes": [_u32, _u32, _u32, _u32],
                     "dsx_knn_workspace_bytes_f16": [_u32, _u32, _u32, _u32], "dsx_knn_f16_table_bytes": [_u32, _u32],
-                    "dsx_fc_split_bytes": [_u32, _u32]}
+                    "dsx_fc_split_bytes": [_u32, _u32], "dsx_knn_workspace_bytes_split": [_u32, _u32, _u32, _u32]}
 
 _lib = None
 

@@ -710,6 +710,7 @@ struct FcSplitArgs {
     const u32x4* Xs;
     const u32x4* Ws;
     uint32_t xrows, wrows, kblocks;   // padded rows of the two sets of planes; blocks of eight k (an even number)
+    uint32_t wcol0;                   // the product's first column is row wcol0 of the W planes (a multiple of 128)
 };
 
 // Z = act(acc? + bias + X . W) as fc_gemm_kernel<2, 2, ...> computes it (same tile order, same epilogue), from planes.
@@ -717,9 +718,11 @@ struct FcSplitArgs {
 // 64 x 64, 24 KiB of units per step, three workgroups per CU.  MH = 2: a 256 x 128 tile, wavefronts of 128 x 64 (eight
 // accumulators: 0.375 fragment reads per MFMA instead of 0.5, and three quarters of the operand traffic per product), 36 KiB
 // per step, two workgroups per CU.
-template <int ACT, int MH>
+// CAND = 1 (MH = 1 only): candidate mode as in fc_gemm_kernel, the scores compared with the rows' bounds instead of stored.
+template <int ACT, int MH, int CAND = 0>
 __global__ __launch_bounds__(kFcThreads, MH == 1 ? 3 : 2) void fc_gemm_split_kernel(FcArgs a, FcSplitArgs sp)
 {
+    static_assert(CAND == 0 || MH == 1, "the candidate epilogue works on tiles of 128 rows");
     constexpr int BM = 128 * MH;
     __shared__ u32x4 sA[2][3][2][BM];
     __shared__ u32x4 sB[2][3][2][128];
@@ -747,6 +750,8 @@ __global__ __launch_bounds__(kFcThreads, MH == 1 ? 3 : 2) void fc_gemm_split_ker
             for (int j = 0; j < 2; j++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) acc[h][i][j][v] = 0.0f;
+    uint32_t bound_key = 0;
+    if constexpr (CAND) bound_key = candidate_bound_prefetch<2>(a.cand, row0, a.batch, tid);
 
     // Every load is "plane base (uniform) + this lane's 32-bit byte offset", the offset advancing by a uniform step per k-step
     // (a plane is smaller than 4 GiB, the host checks): two vector additions per step instead of 64-bit address arithmetic.
@@ -761,7 +766,7 @@ __global__ __launch_bounds__(kFcThreads, MH == 1 ? 3 : 2) void fc_gemm_split_ker
         wbase[p] = reinterpret_cast<const char*>(sp.Ws) + p * wplane;
     }
     uint32_t xoff = (MH == 1) ? (shalf * sp.xrows + row0 + srow) * 16u : (row0 + tid) * 16u;
-    uint32_t woff = (shalf * sp.wrows + col0 + srow) * 16u;
+    uint32_t woff = (shalf * sp.wrows + sp.wcol0 + col0 + srow) * 16u;
     const uint32_t xhalf = sp.xrows * 16u;
     const uint32_t xstep = 2u * sp.xrows * 16u, wstep = 2u * sp.wrows * 16u;
     u32x4 ra[3 * MH], rb[3];
@@ -814,6 +819,7 @@ __global__ __launch_bounds__(kFcThreads, MH == 1 ? 3 : 2) void fc_gemm_split_ker
     };
     const uint32_t nk = sp.kblocks / 2;
     load();
+    if constexpr (CAND) asm volatile("" ::"v"(bound_key));   // the bound's load is issued up here, not moved down to its use
     store(0);
     __syncthreads();
     for (uint32_t kt = 0; kt < nk; kt++) {
@@ -830,6 +836,13 @@ __global__ __launch_bounds__(kFcThreads, MH == 1 ? 3 : 2) void fc_gemm_split_ker
         __syncthreads();
     }
     __builtin_amdgcn_s_setprio(0);
+    if constexpr (CAND) {
+        static_assert(sizeof(sA) >= kCandLdsBytes<2>, "the epilogue reuses the X tile's LDS");
+        // (the k-loop ended with a barrier: every wavefront is done with sA)
+        candidate_epilogue<2, 2, 2, 2, false>(acc[0], reinterpret_cast<float*>(&sA[0][0][0][0]), a.cand, bound_key, row0, col0, a.batch, a.n, tid,
+                                              wm, wn, l32, lhi);
+        return;
+    }
     static_assert(sizeof(sA) >= 2 * 512 * sizeof(float) && sizeof(sB) >= 2 * 512 * sizeof(float),
                   "the segment maxima are transposed through the operand tiles' LDS, two wavefronts in each");
     float* sT = reinterpret_cast<float*>((wave < 2) ? &sA[0][0][0][0] : &sB[0][0][0][0]) + (wave & 1) * 512;
@@ -838,10 +851,11 @@ __global__ __launch_bounds__(kFcThreads, MH == 1 ? 3 : 2) void fc_gemm_split_ker
 }
 
 static uint32_t g_split_tile_rows = 0;   // dsx_fc_split_set_tile_rows: 0 = by shape
-static inline uint32_t split_rows_padded(uint32_t rows) { return (rows + 255) / 256 * 256; }
+uint32_t split_rows_padded(uint32_t rows) { return (rows + 255) / 256 * 256; }
 static inline uint32_t split_kblocks(uint32_t k) { return (k + 15) / 16 * 2; }
+uint64_t split_plane_bytes(uint32_t rows, uint32_t k) { return 3ull * split_rows_padded(rows) * split_kblocks(k) * 16; }
 
-static int fc_split_planes_run(const float* src, uint64_t stride_r, uint64_t stride_k, uint32_t rows, uint32_t k, void* planes)
+int fc_split_planes_run(const float* src, uint64_t stride_r, uint64_t stride_k, uint32_t rows, uint32_t k, void* planes)
 {
     const uint32_t rp = split_rows_padded(rows), kb = split_kblocks(k);
     const uint64_t units = (uint64_t)rp * kb;
@@ -851,8 +865,19 @@ static int fc_split_planes_run(const float* src, uint64_t stride_r, uint64_t str
     return DSX_OK;
 }
 
-static int fc_split_run(const void* Xs, const void* Ws, const float* bias, float* Z, uint32_t ldz, uint32_t batch, uint32_t k, uint32_t n,
-                 int accumulate, uint32_t activation, const dsx_act_params* params, float* seg_max, uint32_t* seg_width)
+static int split_planes_fit(uint32_t xrows, uint32_t wrows, uint32_t kblocks, uint32_t wcol0, uint32_t n)
+{
+    if ((uint64_t)kblocks * xrows * 16 >= (1ull << 32) || (uint64_t)kblocks * wrows * 16 >= (1ull << 32))
+        return set_error(DSX_EINVAL, "dsx_fc_forward_split: a plane of 4 GiB or more (rows padded to 256 x k padded to 16 x 2 bytes)");
+    if (wcol0 % 128 != 0 || (uint64_t)wcol0 + (n + 127) / 128 * 128 > wrows)
+        return set_error(DSX_EINVAL, "dsx_fc_forward_split: columns %u .. %u + %u of planes of %u rows", wcol0, wcol0, n, wrows);
+    return DSX_OK;
+}
+
+// Ws: planes of wrows (padded) rows; the product's n columns are rows wcol0 .. wcol0 + n of them.
+int fc_split_run(const void* Xs, const void* Ws, uint32_t wrows, uint32_t wcol0, const float* bias, float* Z, uint32_t ldz, uint32_t batch,
+                 uint32_t k, uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params, float* seg_max,
+                 uint32_t* seg_width)
 {
     if (seg_width) *seg_width = 0;
     FcArgs a{};
@@ -874,11 +899,8 @@ static int fc_split_run(const void* Xs, const void* Ws, const float* bias, float
         a.nseg = (n + 63) / 64;
         *seg_width = 64;
     }
-    FcSplitArgs sp{reinterpret_cast<const u32x4*>(Xs), reinterpret_cast<const u32x4*>(Ws), split_rows_padded(batch), split_rows_padded(n),
-                   split_kblocks(k)};
-    if ((uint64_t)sp.kblocks * sp.xrows * 16 >= (1ull << 32) || (uint64_t)sp.kblocks * sp.wrows * 16 >= (1ull << 32)) {
-        return set_error(DSX_EINVAL, "dsx_fc_forward_split: a plane of 4 GiB or more (rows padded to 128 x k padded to 16 x 2 bytes)");
-    }
+    FcSplitArgs sp{reinterpret_cast<const u32x4*>(Xs), reinterpret_cast<const u32x4*>(Ws), split_rows_padded(batch), wrows, split_kblocks(k), wcol0};
+    if (int rc = split_planes_fit(sp.xrows, sp.wrows, sp.kblocks, wcol0, n)) return rc;
     const uint32_t total = a.tiles_m * a.tiles_n;
     const dim3 grid(((total + kXcds - 1) / kXcds) * kXcds);
     hipStream_t s = ctx().stream;
@@ -901,6 +923,26 @@ static int fc_split_run(const void* Xs, const void* Ws, const float* bias, float
     }
 #undef DSX_ACT_CASE
     DSX_LAUNCH_CHECK("fc_gemm_split_kernel");
+    return DSX_OK;
+}
+
+// Candidate mode (exact KNN): scores of the queries' planes against columns wcol0 .. wcol0 + n of the item planes, compared with
+// the rows' bounds (CandArgs) instead of stored.
+int fc_split_candidates_run(const void* Xs, const void* Ws, uint32_t wrows, uint32_t wcol0, uint32_t batch, uint32_t k, uint32_t n,
+                            const CandArgs& cand)
+{
+    FcArgs a{};
+    a.batch = batch; a.k = k; a.n = n;
+    a.act = DSX_ACT_LINEAR;
+    a.cand = cand;
+    a.tiles_m = (batch + 127) / 128;
+    a.tiles_n = (n + 127) / 128;
+    FcSplitArgs sp{reinterpret_cast<const u32x4*>(Xs), reinterpret_cast<const u32x4*>(Ws), split_rows_padded(batch), wrows, split_kblocks(k), wcol0};
+    if (int rc = split_planes_fit(sp.xrows, sp.wrows, sp.kblocks, wcol0, n)) return rc;
+    const uint32_t total = a.tiles_m * a.tiles_n;
+    const dim3 grid(((total + kXcds - 1) / kXcds) * kXcds);
+    hipLaunchKernelGGL((fc_gemm_split_kernel<DSX_ACT_LINEAR, 1, 1>), grid, dim3(kFcThreads), 0, ctx().stream, a, sp);
+    DSX_LAUNCH_CHECK("fc_gemm_split_kernel (candidates)");
     return DSX_OK;
 }
 
@@ -971,7 +1013,7 @@ int dsx_fc_forward_segmax(const float* X, uint32_t ldx, const float* W, int tran
 
 uint64_t dsx_fc_split_bytes(uint32_t rows, uint32_t k)
 {
-    return 3ull * split_rows_padded(rows) * split_kblocks(k) * 16;
+    return split_plane_bytes(rows, k);
 }
 
 int dsx_fc_split(const float* src, uint32_t ld, int k_major, uint32_t rows, uint32_t k, void* planes)
@@ -1001,7 +1043,7 @@ int dsx_fc_forward_split(const void* x_planes, const void* w_planes, const float
     DSX_CHECK_ARG(is_elementwise_activation(activation), "dsx_fc_forward_split: activation %u is a row operation; pass DSX_ACT_LINEAR and call dsx_activation", activation);
     DSX_CHECK_ARG((seg_max == NULL) == (seg_width == NULL), "dsx_fc_forward_split: seg_max and seg_width go together");
     if (batch == 0) return DSX_OK;
-    return fc_split_run(x_planes, w_planes, bias, Z, ldz, batch, k, n, accumulate, activation, params, seg_max, seg_width);
+    return fc_split_run(x_planes, w_planes, split_rows_padded(n), 0, bias, Z, ldz, batch, k, n, accumulate, activation, params, seg_max, seg_width);
 }
 
 int dsx_activation(float* unit, uint32_t batch, uint32_t stride, uint32_t activation, const dsx_act_params* params)

@@ -85,6 +85,17 @@ int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int trans
 // per-row lists as packed words (CandArgs); nothing else is written.  knn_refresh folds a row's candidates into its best
 // list.  The caller guarantees 16-byte aligned operands with pitches that are multiples of four floats.
 struct CandArgs;
+// The same products from bf16 matrix instructions (dsx_fc_split / dsx_fc_forward_split): planes of an operand
+// (src element (r, kk) = src[r * stride_r + kk * stride_k]), their size and padded row count, the GEMM on a window of columns
+// of the W planes (wrows: their padded rows; wcol0: first column, a multiple of 128), and its candidate mode.
+uint32_t split_rows_padded(uint32_t rows);
+uint64_t split_plane_bytes(uint32_t rows, uint32_t k);
+int fc_split_planes_run(const float* src, uint64_t stride_r, uint64_t stride_k, uint32_t rows, uint32_t k, void* planes);
+int fc_split_run(const void* Xs, const void* Ws, uint32_t wrows, uint32_t wcol0, const float* bias, float* Z, uint32_t ldz, uint32_t batch,
+                 uint32_t k, uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params, float* seg_max,
+                 uint32_t* seg_width);
+int fc_split_candidates_run(const void* Xs, const void* Ws, uint32_t wrows, uint32_t wcol0, uint32_t batch, uint32_t k, uint32_t n,
+                            const CandArgs& cand);
 int fc_candidates_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, uint32_t batch, uint32_t k, uint32_t n,
                       const CandArgs& cand);
 // The same for a layer (pre-activation sums compared with bounds derived from activated scores, bias folded in).

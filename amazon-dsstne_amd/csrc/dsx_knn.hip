@@ -52,13 +52,14 @@ struct KnnWorkspace {
     uint32_t* cand_count;   // [queries]
     uint32_t* overflow;     // [1] (+ padding)
     uint64_t* cand;         // [queries][kCandCap]
-    void* queries16;        // fp16 storage only: the query batch, [queries rounded up to 256][ld] halves
+    void* queries16;        // fp16 storage: the query batch, [queries rounded up to 256][ld] halves; split products: its bf16 planes
     uint64_t* seg;          // fp16 storage only: [queries][chunks][kCandCap / chunks], the lists of a sweep (knn_f16_sweep_run)
     uint32_t* seg_count;    // fp16 storage only: [queries][64]
     size_t bytes;
 };
 
-static KnnWorkspace knn_layout(void* base, uint32_t rows_padded, uint32_t num_queries, uint32_t k, bool f16 = false, uint32_t dim = 0)
+static KnnWorkspace knn_layout(void* base, uint32_t rows_padded, uint32_t num_queries, uint32_t k, bool f16 = false, uint32_t dim = 0,
+                               bool split = false)
 {
     const uint32_t cb = knn_block_columns(rows_padded, num_queries);
     const uint32_t blocks = (rows_padded + cb - 1) / cb;
@@ -84,6 +85,7 @@ static KnnWorkspace knn_layout(void* base, uint32_t rows_padded, uint32_t num_qu
         w.seg_count = (uint32_t*)p;
         p += align256((size_t)num_queries * 64 * sizeof(uint32_t));
     }
+    if (split) p += align256((size_t)split_plane_bytes(num_queries, dim));
     w.bytes = (size_t)(p - (char*)base);
     return w;
 }
@@ -91,6 +93,9 @@ static KnnWorkspace knn_layout(void* base, uint32_t rows_padded, uint32_t num_qu
 // Where the scores of a column range come from: the fp32 table through fc_gemm_kernel, or the fp16 table through knn_f16_kernel.
 struct KnnOperands {
     bool f16 = false;
+    bool split = false;                 // fp32 products from bf16 matrix instructions: item_planes / query_planes (dsx_fc_split)
+    const void* item_planes = nullptr;
+    const void* query_planes = nullptr;
     const float* items = nullptr;       // fp32: column-major [dim][rows_padded]
     const float* queries = nullptr;     // fp32: [queries][dim]
     const char* items16 = nullptr;      // fp16: [rows rounded up to 256][ld]
@@ -100,6 +105,9 @@ struct KnnOperands {
     int into_matrix(uint32_t c0, uint32_t ncols, uint32_t num_queries, float* Z, uint32_t ldz) const
     {
         if (f16) return knn_f16_scores_run(queries16, items16 + (uint64_t)c0 * ld16 * 2, ld16, num_queries, ncols, Z, ldz, nullptr);
+        if (split)
+            return fc_split_run(query_planes, item_planes, split_rows_padded(rows_padded), c0, nullptr, Z, ldz, num_queries, dim, ncols, 0,
+                                DSX_ACT_LINEAR, nullptr, nullptr, nullptr);
         return fc_run(queries, dim, items + c0, rows_padded, 0, nullptr, Z, ldz, num_queries, dim, ncols, 0, DSX_ACT_LINEAR, nullptr);
     }
     // *chunks_used: how many (row, chunk) lists of seg the range filled besides the shared lists (0: none)
@@ -110,6 +118,7 @@ struct KnnOperands {
         if (f16)
             return knn_f16_candidates_run(queries16, items16 + (uint64_t)c0 * ld16 * 2, ld16, num_queries, ncols, cand, seg, seg_count, kCandCap,
                                           g_knn_f16_sweep, chunks_used);
+        if (split) return fc_split_candidates_run(query_planes, item_planes, split_rows_padded(rows_padded), c0, num_queries, dim, ncols, cand);
         return fc_candidates_run(queries, dim, items + c0, rows_padded, num_queries, dim, ncols, cand);
     }
 };
@@ -238,6 +247,11 @@ size_t dsx_knn_workspace_bytes_f16(uint32_t rows_padded, uint32_t dim, uint32_t 
     return knn_layout(nullptr, rows_padded, num_queries, k, true, dim).bytes;
 }
 
+size_t dsx_knn_workspace_bytes_split(uint32_t rows_padded, uint32_t dim, uint32_t num_queries, uint32_t k)
+{
+    return knn_layout(nullptr, rows_padded, num_queries, k, false, dim, true).bytes;
+}
+
 size_t dsx_knn_f16_table_bytes(uint32_t rows_padded, uint32_t dim) { return (size_t)knn_f16_rows(rows_padded) * knn_f16_ld(dim) * 2; }
 
 int dsx_knn_f16_convert_items(const float* items, uint32_t rows_padded, uint32_t padding, uint32_t dim, void* items_f16)
@@ -255,7 +269,7 @@ int dsx_knn_f16_convert_items(const float* items, uint32_t rows_padded, uint32_t
 static int knn_search_common(KnnOperands& op, uint32_t padding, uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, void* workspace,
                              size_t workspace_bytes, float* elapsed_ms, bool aligned, const float* queries_f32)
 {
-    const size_t need = knn_layout(nullptr, op.rows_padded, num_queries, k, op.f16, op.dim).bytes;
+    const size_t need = knn_layout(nullptr, op.rows_padded, num_queries, k, op.f16, op.dim, op.split).bytes;
     if (workspace) {
         DSX_CHECK_ARG(workspace_bytes >= need, "dsx_knn_search: workspace of %zu bytes, %zu needed", workspace_bytes, need);
         DSX_CHECK_ARG(((uintptr_t)workspace % 256) == 0, "dsx_knn_search: workspace is not 256-byte aligned");
@@ -264,7 +278,7 @@ static int knn_search_common(KnnOperands& op, uint32_t padding, uint32_t num_que
         if (int rc = lib_scratch_reserve(ws, need, "dsx_knn_search workspace")) return rc;
         workspace = ws.ptr;
     }
-    const KnnWorkspace w = knn_layout(workspace, op.rows_padded, num_queries, k, op.f16, op.dim);
+    const KnnWorkspace w = knn_layout(workspace, op.rows_padded, num_queries, k, op.f16, op.dim, op.split);
     const uint32_t M = op.rows_padded - padding;
     hipStream_t s = ctx().stream;
     KnnTimer t;
@@ -278,6 +292,12 @@ static int knn_search_common(KnnOperands& op, uint32_t padding, uint32_t num_que
         rc = knn_to_f16(queries_f32, false, op.dim, num_queries, op.dim, w.queries16, (uint32_t)knn_f16_rows(num_queries));
         t.stop(s, t.gemm);
         op.queries16 = w.queries16;
+    }
+    if (op.split) {   // the query batch as bf16 planes, counted as GEMM time too
+        t.start(s);
+        rc = fc_split_planes_run(queries_f32, op.dim, 1, num_queries, op.dim, w.queries16);
+        t.stop(s, t.gemm);
+        op.query_planes = w.queries16;
     }
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     hipStreamIsCapturing(s, &capturing);
@@ -313,6 +333,26 @@ int dsx_knn_search(const float* items, uint32_t rows_padded, uint32_t padding, u
     op.dim = dim;
     const bool aligned = ((uintptr_t)items % 16) == 0 && ((uintptr_t)queries % 16) == 0 && (rows_padded % 4) == 0 && (dim % 4) == 0;
     return knn_search_common(op, padding, num_queries, k, scores, indexes, workspace, workspace_bytes, elapsed_ms, aligned, nullptr);
+}
+
+int dsx_knn_search_split(const void* item_planes, uint32_t rows_padded, uint32_t padding, uint32_t dim, const float* queries,
+                         uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, void* workspace, size_t workspace_bytes,
+                         float* elapsed_ms)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(item_planes && queries && scores && indexes, "dsx_knn_search_split: null device pointer");
+    DSX_CHECK_ARG(((uintptr_t)item_planes % 16) == 0, "dsx_knn_search_split: the item planes are not 16-byte aligned");
+    DSX_CHECK_ARG(padding < rows_padded, "dsx_knn_search_split: padding %u leaves no item of %u", padding, rows_padded);
+    DSX_CHECK_ARG(dim > 0, "dsx_knn_search_split: dim is 0");
+    DSX_CHECK_ARG(k >= 1 && k <= 256, "dsx_knn_search_split: k = %u is outside 1..256", k);
+    DSX_CHECK_ARG((uint64_t)split_plane_bytes(rows_padded, dim) / 3 < (1ull << 32), "dsx_knn_search_split: a plane of the item table of 4 GiB or more");
+    if (num_queries == 0) return DSX_OK;
+    KnnOperands op;
+    op.split = true;
+    op.item_planes = item_planes;
+    op.rows_padded = rows_padded;
+    op.dim = dim;
+    return knn_search_common(op, padding, num_queries, k, scores, indexes, workspace, workspace_bytes, elapsed_ms, true, queries);
 }
 
 int dsx_knn_search_f16(const void* items_f16, uint32_t rows_padded, uint32_t padding, uint32_t dim, const float* queries,

@@ -417,6 +417,28 @@ def knn_bench(args, pkg, lib):
            "kernel": "knn_f16_wide_kernel (+ knn_f16_kernel for the first block)", "bound": "mfma", "achieved": round(flops / el[0] / 1e9, 3), "peak": 2500.0, "unit_roofline": "TFLOP/s",
            "frac": round(flops / el[0] / 1e9 / 2500.0, 4), "scores_ms": round(el[0], 4), "topk_ms": round(el[1], 4),
            "path": {0: "blocks", 1: "candidate lists", 2: "candidate lists, redone block by block"}[lib.dsx_knn_last_search_path()]}
+    del table
+    # ... and with the fp32 table's products formed from bf16 matrix instructions (dsx_knn_search_split: fp32-accurate, a mode the
+    # caller asks for; reported beside the fp32 figure)
+    planes = pkg.DeviceArray((lib.dsx_fc_split_bytes(rows, D) // 4,), np.uint32, lib)
+    pkg.check(lib.dsx_fc_split(dI.ptr, rows, 1, rows, D, planes.ptr))
+
+    def step_split(timing=None):
+        pkg.check(lib.dsx_knn_search_split(planes.ptr, rows, pad, D, dQ.ptr, Q, K, scores.ptr, idx.ptr, None, 0, timing))
+    for _ in range(max(1, args.warmup)):
+        step_split()
+    pkg.check(lib.dsx_sync())
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step_split()
+    pkg.check(lib.dsx_sync())
+    ms_split = (time.perf_counter() - t0) * 1e3 / args.steps
+    step_split(el)
+    split = {"ms_per_step": round(ms_split, 4), "value": round(Q / (ms_split / 1e3), 1), "unit": "queries/s",
+             "dtype": "f32 products as six bf16 x bf16 MFMA terms, f32 sums", "kernel": "fc_gemm_split_kernel (candidate mode)",
+             "scores_ms": round(el[0], 4), "topk_ms": round(el[1], 4),
+             "path": {0: "blocks", 1: "candidate lists", 2: "candidate lists, redone block by block"}[lib.dsx_knn_last_search_path()]}
+    del planes
     cpu = None
     if args.cpu_seconds > 0:
         orc = entry.load_oracle()
@@ -432,7 +454,7 @@ def knn_bench(args, pkg, lib):
             "unit": "queries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
             "config": {"workload": p.name, "queries": Q, "dim": D, "items": rows - pad, "top_k": K}, "roofline": roofline,
-            "cpu_baseline": cpu, "f16_storage": f16}
+            "cpu_baseline": cpu, "f16_storage": f16, "split_products": split}
 
 
 def main():

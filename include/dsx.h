@@ -339,6 +339,16 @@ int dsx_knn_search_f16(const void* items_f16, uint32_t rows_padded, uint32_t pad
                        uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, void* workspace, size_t workspace_bytes,
                        float* elapsed_ms);
 size_t dsx_knn_workspace_bytes_f16(uint32_t rows_padded, uint32_t dim, uint32_t num_queries, uint32_t k);
+
+/* dsx_knn_search with every fp32 product formed from bf16 matrix instructions (see dsx_fc_forward_split: as close to the exact
+ * inner products as fp32 multiplication, not bit-identical to it; no counterpart in the reference).  item_planes: the table
+ * as dsx_fc_split(items, rows_padded, 1, rows_padded, dim, item_planes) leaves it (dsx_fc_split_bytes(rows_padded, dim) bytes,
+ * 1.5 x the table; made once, the fp32 table can be freed afterwards); queries are fp32 and split in the workspace, which
+ * dsx_knn_workspace_bytes_split sizes.  Everything else as dsx_knn_search. */
+int dsx_knn_search_split(const void* item_planes, uint32_t rows_padded, uint32_t padding, uint32_t dim, const float* queries,
+                         uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, void* workspace, size_t workspace_bytes,
+                         float* elapsed_ms);
+size_t dsx_knn_workspace_bytes_split(uint32_t rows_padded, uint32_t dim, uint32_t num_queries, uint32_t k);
 /* No counterpart in the reference: width of the first column block (rounded down to a multiple of 1024, at least 1024;
  * 0 restores the default of about 1 GiB of scores).  Workspace sizes depend on it: set it before asking for them. */
 int dsx_knn_set_block_columns(uint32_t columns);

@@ -187,6 +187,24 @@ def test_cfg5_knn_full_size(pkg, dsx, orc, synth):
         assert gap.max() < 1e-5, "KNN indexes differ from the oracle outside near-ties (gap %g)" % gap.max()
     assert_close(s[picks], rs, "cfg5 scores of the sampled queries", rel=1e-4)
     say("cfg5: sampled queries agree with the oracle (%d tie-equivalent index differences)" % int(mism.sum()))
+    # fp32 products from bf16 matrix instructions on the same table (dsx_knn_search_split): the same checks against the same oracle results
+    planes = pkg.DeviceArray((dsx.dsx_fc_split_bytes(rows_padded, D) // 4,), np.uint32)
+    pkg.check(dsx.dsx_fc_split(d_items.ptr, rows_padded, 1, rows_padded, D, planes.ptr))
+    pkg.check(dsx.dsx_knn_search_split(planes.ptr, rows_padded, padding, D, d_q.ptr, Q, k, scores.ptr, idx.ptr, None, 0, None))
+    assert dsx.dsx_knn_last_search_path() == 1
+    ss, si = scores.numpy(), idx.numpy()
+    del planes
+    assert np.all(si < M) and np.all(np.diff(ss.astype(np.float64), axis=1) <= 0)
+    for q0 in range(0, Q, 512):
+        dots = np.einsum("qkd,qd->qk", p.items[si[q0:q0 + 256]].astype(np.float64), p.queries[q0:q0 + 256].astype(np.float64))
+        assert np.abs(dots - ss[q0:q0 + 256]).max() < 2e-6, "split products: a reported score is not the dot product with the reported item"
+    mism = si[picks] != ri
+    if mism.any():
+        gap = np.abs(ss[picks][mism].astype(np.float64) - rs[mism].astype(np.float64))
+        assert gap.max() < 1e-5, "split-product KNN indexes differ from the oracle outside near-ties (gap %g)" % gap.max()
+    assert_close(ss[picks], rs, "cfg5 split-product scores of the sampled queries", rel=1e-4)
+    say("cfg5 split products: sampled queries agree with the oracle (%d tie-equivalent index differences; %d of %d indexes differ from the fp32 search)"
+        % (int(mism.sum()), int((si != i).sum()), si.size))
     # fp16 storage on the same table: same checks against fp16-rounded operands for the sampled queries
     f16_bytes = dsx.dsx_knn_f16_table_bytes(rows_padded, D)
     t16 = pkg.DeviceArray((f16_bytes,), np.uint8)
