@@ -13,7 +13,10 @@
 namespace astdl {
 namespace knn {
 
-enum class DataType { FP32 = 0, FP16 = 1 };
+// FP32 and FP16 as in the reference (knn/KnnData.h).  FP32Split ("fp32-split") has no counterpart there: fp32 storage whose
+// inner products are formed from bf16 matrix instructions (dsx_knn_search_split): fp32-accurate scores, not bit-identical to
+// FP32's, about 1.5 times as fast; the table is kept as bf16 planes, 1.5 times its fp32 size.
+enum class DataType { FP32 = 0, FP16 = 1, FP32Split = 2 };
 
 std::string getDataTypeString(DataType dataType);
 DataType getDataTypeFromString(const std::string& dataTypeLiteral);

@@ -107,6 +107,7 @@ std::string getDataTypeString(DataType dataType)
     switch (dataType) {
     case DataType::FP32: return "fp32";
     case DataType::FP16: return "fp16";
+    case DataType::FP32Split: return "fp32-split";
     default: return "unknown";
     }
 }
@@ -115,6 +116,7 @@ DataType getDataTypeFromString(const std::string& s)
 {
     if (s == "fp32") return DataType::FP32;
     if (s == "fp16") return DataType::FP16;
+    if (s == "fp32-split") return DataType::FP32Split;
     throw std::invalid_argument("Unknown DataType " + s);
 }
 
@@ -214,6 +216,17 @@ void KnnData::load(int device, DataReader* dataReader)
         check(dsx_knn_f16_convert_items((const float*)dTmp.data, rows, rows - actualRows, (uint32_t)columns, table), "KnnData::load");
         check(dsx_sync(), "KnnData::load");
         freeMatrix(dTmp);
+    } else if (dataType == DataType::FP32Split) {
+        // the table as three planes of bf16 (dsx_fc_split of the column-major fp32 table, which only lives until then); its
+        // Matrix describes the logical shape (rows x columns of 3 x 2 bytes) over an allocation of dsx_fc_split_bytes
+        Matrix dTmp = allocateMatrixOnDevice(rows, columns, sizeof(float));
+        check(dsx_memcpy_h2d(dTmp.data, hTmpData, hTmp.getSizeInBytes()), "KnnData::load");
+        void* planes = nullptr;
+        check(dsx_malloc(&planes, dsx_fc_split_bytes(rows, (uint32_t)columns)), "KnnData::load");
+        dCollectionPartitions[device] = Matrix(planes, rows, columns, 6, MemoryType::Device);
+        check(dsx_fc_split((const float*)dTmp.data, rows, 1, rows, (uint32_t)columns, planes), "KnnData::load");
+        check(dsx_sync(), "KnnData::load");
+        freeMatrix(dTmp);
     } else {
         dCollectionPartitions[device] = allocateMatrixOnDevice(rows, columns, sizeof(float));
         check(dsx_memcpy_h2d(dCollectionPartitions[device].data, hTmpData, hTmp.getSizeInBytes()), "KnnData::load");
@@ -224,8 +237,9 @@ void KnnData::load(int device, DataReader* dataReader)
     dResultIndexes[device] = allocateMatrixOnDevice(batchSize, maxK, sizeof(uint32_t));
     hResultScores[device] = allocateMatrixOnHost(batchSize, maxK, sizeof(float));
     hResultIndexes[device] = allocateMatrixOnHost(batchSize, maxK, sizeof(uint32_t));
-    const size_t ws = dataType == DataType::FP16 ? dsx_knn_workspace_bytes_f16(rows, columns, batchSize, maxK)
-                                                 : dsx_knn_workspace_bytes(rows, columns, batchSize, maxK);
+    const size_t ws = dataType == DataType::FP16        ? dsx_knn_workspace_bytes_f16(rows, columns, batchSize, maxK)
+                      : dataType == DataType::FP32Split ? dsx_knn_workspace_bytes_split(rows, columns, batchSize, maxK)
+                                                        : dsx_knn_workspace_bytes(rows, columns, batchSize, maxK);
     dWorkspaces[device] = allocateMatrixOnDevice(1, 1, ws);
     dsx_device_info info;
     check(dsx_get_device_info(&info), "KnnData::load");
@@ -304,6 +318,11 @@ void KnnExactGpu::search(int k, const float* inputs, int size, std::string* keys
         check(dsx_knn_search_f16(items.data, items.numRows, data->collectionRowsPadded[device], (uint32_t)D, (const float*)dIn.data,
                                  (uint32_t)size, (uint32_t)maxK, dScores, dIndexes, data->dWorkspaces[device].data,
                                  data->dWorkspaces[device].elementSize, elapsed),
+              "KnnExactGpu::search");
+    else if (data->dataType == DataType::FP32Split)
+        check(dsx_knn_search_split(items.data, items.numRows, data->collectionRowsPadded[device], (uint32_t)D, (const float*)dIn.data,
+                                   (uint32_t)size, (uint32_t)maxK, dScores, dIndexes, data->dWorkspaces[device].data,
+                                   data->dWorkspaces[device].elementSize, elapsed),
               "KnnExactGpu::search");
     else
         check(dsx_knn_search((const float*)items.data, items.numRows, data->collectionRowsPadded[device], (uint32_t)D, (const float*)dIn.data,

@@ -120,6 +120,8 @@ dsstne_knn* dsstne_knn_create(uint32_t batch, uint32_t max_k);
 /* The same with the item storage named like the JNI's dataType argument ("fp32" or "fp16": astdl::knn::getDataTypeFromString,
  * knn/KnnData.cpp:81-91; an unknown name fails). */
 dsstne_knn* dsstne_knn_create_typed(uint32_t batch, uint32_t max_k, const char* data_type);
+/* (data_type "fp32-split", which the reference does not have: fp32 storage with the inner products formed from bf16 matrix
+ * instructions, dsx_knn_search_split in dsx.h) */
 /* KnnData::load from rows in memory: items is [rows][dim] row-major; keys may be NULL (row numbers are used). */
 int dsstne_knn_load(dsstne_knn* knn, const float* items, uint32_t rows, uint32_t dim, const char* const* keys);
 /* KnnData::load from a text file "key<kv_delim>v0<vec_delim>v1..." */

@@ -224,6 +224,7 @@ static void testKnnHost(const string& dir)
     CHECK(out[0] == 0.9f && out[1] == 0.9f && out[2] == 0.7f);
     CHECK(outk[0] == "a0" && outk[1] == "b0" && outk[2] == "b1");
     CHECK(getDataTypeFromString("fp32") == DataType::FP32 && getDataTypeString(DataType::FP16) == "fp16");
+    CHECK(getDataTypeFromString("fp32-split") == DataType::FP32Split && getDataTypeString(DataType::FP32Split) == "fp32-split");
     checkThrows<std::invalid_argument>("bad data type", [] { getDataTypeFromString("int8"); });
 }
 

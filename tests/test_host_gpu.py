@@ -279,6 +279,32 @@ def test_knn_api(pkg, dsx, orc, synth, tmp_path):
         lib.dsstne_knn_destroy(knn)
 
 
+def test_knn_api_split_products(pkg, dsx, orc, synth):
+    """KnnData(…, DataType::FP32Split): the fp32 table as bf16 planes, scores as exact as fp32 storage gives them."""
+    from amazon_dsstne_amd import host_api
+    lib = host_api.load_host_library()
+    p = synth.knn_config(seed=7, items=23456, queries=50, dim=72, k=24)
+    knn = lib.dsstne_knn_create_typed(64, 32, b"fp32-split")
+    assert knn, lib.dsstne_last_error()
+    try:
+        items = np.ascontiguousarray(p.items)
+        assert lib.dsstne_knn_load(knn, items.ctypes.data, items.shape[0], items.shape[1], None) == 0, lib.dsstne_last_error()
+        scores = np.empty((50, 24), dtype=np.float32)
+        idx = np.empty((50, 24), dtype=np.uint32)
+        q = np.ascontiguousarray(p.queries)
+        assert lib.dsstne_knn_search(knn, 24, q.ctypes.data, 50, scores.ctypes.data, idx.ctypes.data) == 0, lib.dsstne_last_error()
+        full = p.queries.astype(np.float64) @ p.items.astype(np.float64).T
+        order = np.argsort(-full, axis=1, kind="stable")[:, :24]
+        mism = idx != order
+        if mism.any():
+            r, c = np.nonzero(mism)
+            assert np.abs(full[r, idx[r, c]] - full[r, order[r, c]]).max() < 1e-5
+        # fp32 accuracy: unit vectors, so the scores are within a few fp32 roundings of the exact ones
+        assert np.abs(scores - np.take_along_axis(full, idx.astype(np.int64), axis=1)).max() < 2e-6
+    finally:
+        lib.dsstne_knn_destroy(knn)
+
+
 def test_knn_api_fp16_storage(pkg, dsx, orc, synth):
     """KnnData(…, DataType::FP16) + KnnExactGpu::search: table and queries rounded to fp16, fp32 scores (knn/KnnData.cpp:209-216,
     knn/KnnExactGpu.cu:108-116); a partial batch (size < batchSize) as the JNI passes it."""
