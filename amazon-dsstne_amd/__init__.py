@@ -95,6 +95,7 @@ SIGNATURES = {
     "dsx_topk_filtered_static": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp],
     "dsx_topk_guided": [_vp, _vp, _vp, _u32, _u32, _u32, _vp, _u32, _u32, _vp, _vp, _vp, _vp, _vp],
     "dsx_fc_topk": [_vp, _u32, _vp, _vp, _u32, _u32, _u32, _u32, C.POINTER(ActParams), _u32, _vp, _vp, _u32, _vp, _vp, _vp, _vp],
+    "dsx_fc_topk_split": [_vp, _u32, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, C.POINTER(ActParams), _u32, _vp, _vp, _u32, _vp, _vp, _vp, _vp],
     "dsx_fc_topk_supported": [_u32, _vp, _u32, C.POINTER(ActParams), _vp],
     "dsx_fc_topk_flagged": [_int],
     "dsx_fc_topk_set_first_columns": [_u32],

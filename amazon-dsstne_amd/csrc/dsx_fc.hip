@@ -718,7 +718,8 @@ struct FcSplitArgs {
 // 64 x 64, 24 KiB of units per step, three workgroups per CU.  MH = 2: a 256 x 128 tile, wavefronts of 128 x 64 (eight
 // accumulators: 0.375 fragment reads per MFMA instead of 0.5, and three quarters of the operand traffic per product), 36 KiB
 // per step, two workgroups per CU.
-// CAND = 1 (MH = 1 only): candidate mode as in fc_gemm_kernel, the scores compared with the rows' bounds instead of stored.
+// CAND (MH = 1 only): the candidate modes of fc_gemm_kernel, the scores compared with the rows' bounds instead of stored:
+// 1 = exact KNN, 2 = a layer (the sums start from the bias, pre-activation sums against bounds derived from activated scores).
 template <int ACT, int MH, int CAND = 0>
 __global__ __launch_bounds__(kFcThreads, MH == 1 ? 3 : 2) void fc_gemm_split_kernel(FcArgs a, FcSplitArgs sp)
 {
@@ -743,13 +744,19 @@ __global__ __launch_bounds__(kFcThreads, MH == 1 ? 3 : 2) void fc_gemm_split_ker
 
     floatx16 acc[MH][2][2];
 #pragma unroll
-    for (int h = 0; h < MH; h++)
+    for (int j = 0; j < 2; j++) {
+        float start = 0.0f;
+        if constexpr (CAND == 2) {   // every register of a lane belongs to column l32 of its block: the sums start from the bias
+            const uint32_t c = col0 + wn * 64 + j * 32 + l32;
+            if (a.bias && c < a.n) start = a.bias[c];
+        }
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int h = 0; h < MH; h++)
 #pragma unroll
-            for (int j = 0; j < 2; j++)
+            for (int i = 0; i < 2; i++)
 #pragma unroll
-                for (int v = 0; v < 16; v++) acc[h][i][j][v] = 0.0f;
+                for (int v = 0; v < 16; v++) acc[h][i][j][v] = start;
+    }
     uint32_t bound_key = 0;
     if constexpr (CAND) bound_key = candidate_bound_prefetch<2>(a.cand, row0, a.batch, tid);
 
@@ -839,8 +846,8 @@ __global__ __launch_bounds__(kFcThreads, MH == 1 ? 3 : 2) void fc_gemm_split_ker
     if constexpr (CAND) {
         static_assert(sizeof(sA) >= kCandLdsBytes<2>, "the epilogue reuses the X tile's LDS");
         // (the k-loop ended with a barrier: every wavefront is done with sA)
-        candidate_epilogue<2, 2, 2, 2, false>(acc[0], reinterpret_cast<float*>(&sA[0][0][0][0]), a.cand, bound_key, row0, col0, a.batch, a.n, tid,
-                                              wm, wn, l32, lhi);
+        candidate_epilogue<2, 2, 2, 2, CAND == 2>(acc[0], reinterpret_cast<float*>(&sA[0][0][0][0]), a.cand, bound_key, row0, col0, a.batch, a.n,
+                                                  tid, wm, wn, l32, lhi);
         return;
     }
     static_assert(sizeof(sA) >= 2 * 512 * sizeof(float) && sizeof(sB) >= 2 * 512 * sizeof(float),
@@ -926,12 +933,14 @@ int fc_split_run(const void* Xs, const void* Ws, uint32_t wrows, uint32_t wcol0,
     return DSX_OK;
 }
 
-// Candidate mode (exact KNN): scores of the queries' planes against columns wcol0 .. wcol0 + n of the item planes, compared with
-// the rows' bounds (CandArgs) instead of stored.
+// Candidate modes: scores of X's planes against columns wcol0 .. wcol0 + n of the W planes, compared with the rows' bounds
+// (CandArgs) instead of stored.  layer: Z = act(bias + X.W) as fc_layer_candidates_run (cand.act etc. describe the activation,
+// bias points at the window's first column); otherwise plain inner products (exact KNN).
 int fc_split_candidates_run(const void* Xs, const void* Ws, uint32_t wrows, uint32_t wcol0, uint32_t batch, uint32_t k, uint32_t n,
-                            const CandArgs& cand)
+                            const CandArgs& cand, bool layer, const float* bias)
 {
     FcArgs a{};
+    a.bias = bias;   // layer mode: of the window's first column
     a.batch = batch; a.k = k; a.n = n;
     a.act = DSX_ACT_LINEAR;
     a.cand = cand;
@@ -941,7 +950,8 @@ int fc_split_candidates_run(const void* Xs, const void* Ws, uint32_t wrows, uint
     if (int rc = split_planes_fit(sp.xrows, sp.wrows, sp.kblocks, wcol0, n)) return rc;
     const uint32_t total = a.tiles_m * a.tiles_n;
     const dim3 grid(((total + kXcds - 1) / kXcds) * kXcds);
-    hipLaunchKernelGGL((fc_gemm_split_kernel<DSX_ACT_LINEAR, 1, 1>), grid, dim3(kFcThreads), 0, ctx().stream, a, sp);
+    if (layer) hipLaunchKernelGGL((fc_gemm_split_kernel<DSX_ACT_LINEAR, 1, 2>), grid, dim3(kFcThreads), 0, ctx().stream, a, sp);
+    else hipLaunchKernelGGL((fc_gemm_split_kernel<DSX_ACT_LINEAR, 1, 1>), grid, dim3(kFcThreads), 0, ctx().stream, a, sp);
     DSX_LAUNCH_CHECK("fc_gemm_split_kernel (candidates)");
     return DSX_OK;
 }

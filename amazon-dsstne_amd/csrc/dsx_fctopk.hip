@@ -115,9 +115,14 @@ int dsx_fc_topk_supported(uint32_t ldx, const float* X, uint32_t activation, con
     return layer_activation_supported(activation, params) && filter_mul == nullptr && ((uintptr_t)X % 16) == 0 && (ldx % 4) == 0;
 }
 
-int dsx_fc_topk(const float* X, uint32_t ldx, const float* W, const float* bias, uint32_t batch, uint32_t kdim, uint32_t n,
-                uint32_t activation, const dsx_act_params* params, uint32_t k, float* keys, uint32_t* values, uint32_t position,
-                const uint32_t* index, const uint64_t* filter_start, const uint64_t* filter_end, const uint32_t* filter_index)
+}  // extern "C"
+
+// x_planes / w_planes (both or neither): the operands as dsx_fc_split leaves them; the products then come from the split-product
+// kernel.  X and W are needed either way (rows whose lists fill up are recomputed from them, in fp32).
+static int fc_topk_common(const float* X, uint32_t ldx, const float* W, const float* bias, uint32_t batch, uint32_t kdim, uint32_t n,
+                          uint32_t activation, const dsx_act_params* params, uint32_t k, float* keys, uint32_t* values, uint32_t position,
+                          const uint32_t* index, const uint64_t* filter_start, const uint64_t* filter_end, const uint32_t* filter_index,
+                          const void* x_planes, const void* w_planes)
 {
     DSX_REQUIRE_INIT();
     DSX_CHECK_ARG(X && W && keys && values, "dsx_fc_topk: null device pointer");
@@ -144,7 +149,9 @@ int dsx_fc_topk(const float* X, uint32_t ldx, const float* W, const float* bias,
     hipStream_t s = ctx().stream;
 
     // first block: the layer as a matrix, then the scanning top-K (filtered: indexes beyond the block are ignored)
-    int rc = fc_run(X, ldx, W, n, 0, bias, w.block_scores, ld0, batch, kdim, n0, 0, activation, params);
+    const uint32_t wrows = split_rows_padded(n);
+    int rc = x_planes ? fc_split_run(x_planes, w_planes, wrows, 0, bias, w.block_scores, ld0, batch, kdim, n0, 0, activation, params, nullptr, nullptr)
+                      : fc_run(X, ldx, W, n, 0, bias, w.block_scores, ld0, batch, kdim, n0, 0, activation, params);
     if (rc) return rc;
     if (!ranges)
         return topk_run(w.block_scores, ld0, n0, batch, k, keys, values, position, index, filter_start, filter_end, filter_index, nullptr, 0,
@@ -174,7 +181,8 @@ int dsx_fc_topk(const float* X, uint32_t ldx, const float* W, const float* bias,
         cand.slope = params ? params->slope : 0.01f;
         cand.alpha = params ? params->alpha : 1.0f;
         cand.lambda = params ? params->lambda : 1.0f;
-        rc = fc_layer_candidates_run(X, ldx, W + done, n, bias ? bias + done : nullptr, batch, kdim, ncols, cand);
+        rc = x_planes ? fc_split_candidates_run(x_planes, w_planes, wrows, done, batch, kdim, ncols, cand, true, bias ? bias + done : nullptr)
+                      : fc_layer_candidates_run(X, ldx, W + done, n, bias ? bias + done : nullptr, batch, kdim, ncols, cand);
         if (rc) return rc;
         done += ncols;
         LayerRefresh r{};
@@ -191,6 +199,27 @@ int dsx_fc_topk(const float* X, uint32_t ldx, const float* W, const float* bias,
         if (rc) return rc;
     }
     return DSX_OK;
+}
+
+extern "C" {
+
+int dsx_fc_topk(const float* X, uint32_t ldx, const float* W, const float* bias, uint32_t batch, uint32_t kdim, uint32_t n,
+                uint32_t activation, const dsx_act_params* params, uint32_t k, float* keys, uint32_t* values, uint32_t position,
+                const uint32_t* index, const uint64_t* filter_start, const uint64_t* filter_end, const uint32_t* filter_index)
+{
+    return fc_topk_common(X, ldx, W, bias, batch, kdim, n, activation, params, k, keys, values, position, index, filter_start, filter_end,
+                          filter_index, nullptr, nullptr);
+}
+
+int dsx_fc_topk_split(const float* X, uint32_t ldx, const float* W, const void* x_planes, const void* w_planes, const float* bias,
+                      uint32_t batch, uint32_t kdim, uint32_t n, uint32_t activation, const dsx_act_params* params, uint32_t k, float* keys,
+                      uint32_t* values, uint32_t position, const uint32_t* index, const uint64_t* filter_start, const uint64_t* filter_end,
+                      const uint32_t* filter_index)
+{
+    DSX_CHECK_ARG(x_planes && w_planes, "dsx_fc_topk_split: null planes");
+    DSX_CHECK_ARG(((uintptr_t)x_planes % 16) == 0 && ((uintptr_t)w_planes % 16) == 0, "dsx_fc_topk_split: planes must be 16-byte aligned");
+    return fc_topk_common(X, ldx, W, bias, batch, kdim, n, activation, params, k, keys, values, position, index, filter_start, filter_end,
+                          filter_index, x_planes, w_planes);
 }
 
 }  // extern "C"

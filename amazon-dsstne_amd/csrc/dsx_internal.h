@@ -95,7 +95,7 @@ int fc_split_run(const void* Xs, const void* Ws, uint32_t wrows, uint32_t wcol0,
                  uint32_t k, uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params, float* seg_max,
                  uint32_t* seg_width);
 int fc_split_candidates_run(const void* Xs, const void* Ws, uint32_t wrows, uint32_t wcol0, uint32_t batch, uint32_t k, uint32_t n,
-                            const CandArgs& cand);
+                            const CandArgs& cand, bool layer = false, const float* bias = nullptr);
 int fc_candidates_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, uint32_t batch, uint32_t k, uint32_t n,
                       const CandArgs& cand);
 // The same for a layer (pre-activation sums compared with bounds derived from activated scores, bias folded in).

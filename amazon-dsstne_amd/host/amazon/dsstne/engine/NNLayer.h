@@ -98,6 +98,7 @@ private:
     }
     // Z = act(bias + X.W) of a single-source layer through dsx_fc_split + dsx_fc_forward_split (segment maxima on request).
     void ForwardSplit(uint32_t batch, NNFloat* pSegMax, uint32_t* pSegWidth);
+    const void* SplitInput(uint32_t batch);   // the source layer's units of this batch as planes (this lane's buffer)
     bool _deferred = false;
     uint32_t _deferredBatch = 0;
     void Materialise();

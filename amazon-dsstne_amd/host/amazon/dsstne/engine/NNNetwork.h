@@ -86,7 +86,7 @@ public:
     // No counterpart in the reference.  SetSplitProducts(true): dense layers wide enough for the tiled kernel (at least two
     // 128 x 128 tiles per compute unit) form every fp32 product from six bf16 matrix instructions (dsx_fc_forward_split): sums as
     // close to the exact ones as fp32 multiplication gives, not bit-identical to it, about 1.5 times as fast; the weights of those
-    // layers are kept a second time as bf16 planes (1.5 times their size), and a wide output layer is always stored.  A caller
+    // layers are kept a second time as bf16 planes (1.5 times their size).  A caller
     // that writes weights through NNWeight::GetWeightBuffer calls it again afterwards.  Off by default.
     bool SetSplitProducts(bool bSplit);
     uint32_t GetLanes() const { return _lanes; }

@@ -166,7 +166,7 @@ void NNLayer::ForwardPropagateFullyConnected(uint32_t position, uint32_t batch, 
         } else if (_kind == Output && _localStride >= kSegMaxMinWidth) {
             // Wide output layer that feeds no other layer: what usually follows is a top-K, which can run together with the layer
             // without the layer's result ever being stored.  The layer is computed when somebody asks for it.
-            if (_bDeferOutput && !UseSplitProducts(batch) && _localStride >= kDeferMinWidth && !w->_bTransposed && _vOutgoingLayer.empty() && _vOutgoingSkip.empty() &&
+            if (_bDeferOutput && _localStride >= kDeferMinWidth && !w->_bTransposed && _vOutgoingLayer.empty() && _vOutgoingSkip.empty() &&
                 dsx_fc_topk_supported(src->_stride, src->GetUnitBuffer(), (uint32_t)_activation, &params, NULL)) {
                 if (dsx_fc_topk_flagged(0)) {
                     // rows whose survivor lists filled up had to be recomputed one by one: this data (thousands of scores tied at the
@@ -238,12 +238,20 @@ void NNLayer::ForwardSplit(uint32_t batch, NNFloat* pSegMax, uint32_t* pSegWidth
     dsx_act_params params = {_RELUSlope, _ELUAlpha, _SELULambda};
     const uint32_t k = src->_stride;
     const void* pWeightPlanes = wsrc->SplitPlanes(w->_bTransposed, k, _localStride);
+    const void* pInputPlanes = SplitInput(batch);
+    dsxFatal(dsx_fc_forward_split(pInputPlanes, pWeightPlanes, w->_pbBias->_pDevData, GetIncomingUnitBuffer(), _stride, batch, k,
+                                  _localStride, 0, (uint32_t)_activation, &params, pSegMax, pSegWidth),
+             "NNLayer::ForwardPropagate: GEMM failure");
+}
+
+const void* NNLayer::SplitInput(uint32_t batch)
+{
+    NNLayer* src = _vIncomingLayer[0];
+    const uint32_t k = src->_stride;
     const size_t words = (size_t)(dsx_fc_split_bytes(_batch, k) / sizeof(uint32_t));
     if (!_pbSplitInput || _pbSplitInput->_length < words) _pbSplitInput.reset(new GpuBuffer<uint32_t>(words));
     dsxFatal(dsx_fc_split(src->GetUnitBuffer(), src->_stride, 0, batch, k, _pbSplitInput->_pDevData), "NNLayer::ForwardPropagate: input planes");
-    dsxFatal(dsx_fc_forward_split(_pbSplitInput->_pDevData, pWeightPlanes, w->_pbBias->_pDevData, GetIncomingUnitBuffer(), _stride, batch, k,
-                                  _localStride, 0, (uint32_t)_activation, &params, pSegMax, pSegWidth),
-             "NNLayer::ForwardPropagate: GEMM failure");
+    return _pbSplitInput->_pDevData;
 }
 
 void NNLayer::CalculateActivation(uint32_t batch)

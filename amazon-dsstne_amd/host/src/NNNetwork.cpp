@@ -317,6 +317,15 @@ void NNNetwork::LayerWithTopK(NNLayer* pLayer, uint32_t k, uint32_t batch, const
     NNWeight* w = pLayer->_vIncomingWeight[0];
     NNWeight* wsrc = w->_bShared ? w->_pSharedWeight : w;
     dsx_act_params params = {pLayer->_RELUSlope, pLayer->_ELUAlpha, pLayer->_SELULambda};
+    if (pLayer->UseSplitProducts(batch)) {
+        const void* pInputPlanes = pLayer->SplitInput(batch);
+        dsxFatal(dsx_fc_topk_split(src->GetUnitBuffer(), src->_stride, wsrc->_pbWeight->_pDevData, pInputPlanes,
+                                   wsrc->SplitPlanes(false, src->_stride, pLayer->_localStride), w->_pbBias->_pDevData, batch, src->_stride,
+                                   pLayer->_localStride, (uint32_t)pLayer->_activation, &params, k, pKey, pValue, _position, pIndex,
+                                   pFilterStart, pFilterEnd, pFilterIndex),
+                 "NNNetwork::CalculateTopK: output layer with top-K");
+        return;
+    }
     dsxFatal(dsx_fc_topk(src->GetUnitBuffer(), src->_stride, wsrc->_pbWeight->_pDevData, w->_pbBias->_pDevData, batch, src->_stride,
                          pLayer->_localStride, (uint32_t)pLayer->_activation, &params, k, pKey, pValue, _position, pIndex, pFilterStart,
                          pFilterEnd, pFilterIndex),

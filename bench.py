@@ -361,7 +361,7 @@ def network_bench(args, pkg, lib):
                           "note": "NNNetwork::SetDeferredOutput(false): PredictBatch stores the output layer, the top-K reads it back (the same as the default below 131,072 output units)"},
         "split_products": {"ms_per_step": round(ms_split, 5), "value": rate(ms_split), "unit": "samples/s",
                            "dtype": "f32 products as six bf16 x bf16 MFMA terms, f32 sums",
-                           "note": "NNNetwork::SetSplitProducts(true), off by default: dense layers of at least two 128 x 128 tiles per compute unit run fc_gemm_split_kernel (a wide output layer is then always stored); results within the same tolerance of the oracle, as close to fp64 as the fp32 kernel's"},
+                           "note": "NNNetwork::SetSplitProducts(true), off by default: dense layers of at least two 128 x 128 tiles per compute unit run fc_gemm_split_kernel (a deferred output layer: dsx_fc_topk_split); results within the same tolerance of the oracle, as close to fp64 as the fp32 kernel's"},
         "with_input_upload": {"ms_per_step": round(ms_upload, 5), "value": rate(ms_upload), "unit": "samples/s",
                               "note": "the batch's CSR arrays handed over as host memory before every step (NNDataSet::LoadSparseData; PCIe-inclusive): uploads go to alternating sets of device arrays on the lane of the batch they belong to"},
         "request_round_trip": {"ms": round(ms_request, 5), "value": rate(ms_request), "unit": "samples/s",

@@ -95,8 +95,8 @@ int dsstne_set_lanes(dsstne_context* ctx, uint32_t lanes);
 int dsstne_set_deferred_output(dsstne_context* ctx, int defer);
 /* No counterpart in the reference (NNNetwork::SetSplitProducts).  split != 0: dense layers wide enough for the tiled kernel form
  * their fp32 products from bf16 matrix instructions (dsx_fc_forward_split in dsx.h): as close to the exact sums as fp32
- * multiplication, not bit-identical to it, about 1.5 times as fast; those layers' weights are kept a second time as bf16 planes
- * and a wide output layer is always stored.  Off by default. */
+ * multiplication, not bit-identical to it, about 1.5 times as fast; those layers' weights are kept a second time as bf16 planes.
+ * Off by default. */
 int dsstne_set_split_products(dsstne_context* ctx, int split);
 /* Dsstne.predict in one call: position 0, predict, unfiltered (filter_dataset NULL) or filtered top-k, copy back. */
 int dsstne_predict(dsstne_context* ctx, const char* layer, uint32_t k, const char* filter_dataset, float* scores, uint32_t* indexes);

@@ -305,6 +305,12 @@ int dsx_topk_guided(const float* in, float* keys, uint32_t* values, uint32_t bat
 int dsx_fc_topk(const float* X, uint32_t ldx, const float* W, const float* bias, uint32_t batch, uint32_t k_dim, uint32_t n,
                 uint32_t activation, const dsx_act_params* params, uint32_t k, float* keys, uint32_t* values, uint32_t position,
                 const uint32_t* index, const uint64_t* filter_start, const uint64_t* filter_end, const uint32_t* filter_index);
+/* dsx_fc_topk with the products formed from bf16 matrix instructions (dsx_fc_forward_split): x_planes = dsx_fc_split of X,
+ * w_planes = dsx_fc_split of W (k_major).  X and W are still needed: rows whose survivor lists fill up are recomputed from them. */
+int dsx_fc_topk_split(const float* X, uint32_t ldx, const float* W, const void* x_planes, const void* w_planes, const float* bias,
+                      uint32_t batch, uint32_t k_dim, uint32_t n, uint32_t activation, const dsx_act_params* params, uint32_t k, float* keys,
+                      uint32_t* values, uint32_t position, const uint32_t* index, const uint64_t* filter_start, const uint64_t* filter_end,
+                      const uint32_t* filter_index);
 int dsx_fc_topk_supported(uint32_t ldx, const float* X, uint32_t activation, const dsx_act_params* params, const float* filter_mul);
 /* 1 if any row of any dsx_fc_topk call so far had to be recomputed (reset != 0 clears the mark). */
 int dsx_fc_topk_flagged(int reset);

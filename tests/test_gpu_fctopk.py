@@ -21,10 +21,17 @@ def dev(pkg, a):
     return None if a is None else pkg.DeviceArray.from_numpy(a)
 
 
-@pytest.fixture
-def knobs(dsx):
+MODE = {"split": False}
+
+
+@pytest.fixture(params=["fp32", "split"])
+def knobs(request, dsx):
+    """Every test runs twice: dsx_fc_topk, and dsx_fc_topk_split (the same call with the products formed from bf16 matrix
+    instructions; the two-call path it is compared with stays the fp32 one)."""
+    MODE["split"] = request.param == "split"
     dsx.dsx_fc_topk_flagged(1)
     yield dsx
+    MODE["split"] = False
     dsx.dsx_fc_topk_set_first_columns(0)
     dsx.dsx_fc_topk_set_candidate_capacity(0)
     dsx.dsx_fc_topk_flagged(1)
@@ -40,8 +47,16 @@ def run_both(pkg, dsx, orc, X, W, bias, act, k, position=0, index=None, start=No
     params = pkg.ActParams(0.01, 1.0, 1.0)
     keys = pkg.DeviceArray.from_numpy(np.full((batch, k), 7.0, dtype=np.float32))
     vals = pkg.DeviceArray.from_numpy(np.full((batch, k), 7, dtype=np.uint32))
-    pkg.check(dsx.dsx_fc_topk(dX.ptr, kdim, dW.ptr, pkg.ptr(db), batch, kdim, n, act, C.byref(params), k, keys.ptr, vals.ptr, position,
-                              pkg.ptr(di), pkg.ptr(ds), pkg.ptr(de), pkg.ptr(dx)))
+    if MODE["split"]:
+        xp = pkg.DeviceArray((dsx.dsx_fc_split_bytes(batch, kdim) // 4,), np.uint32)
+        wp = pkg.DeviceArray((dsx.dsx_fc_split_bytes(n, kdim) // 4,), np.uint32)
+        pkg.check(dsx.dsx_fc_split(dX.ptr, kdim, 0, batch, kdim, xp.ptr))
+        pkg.check(dsx.dsx_fc_split(dW.ptr, n, 1, n, kdim, wp.ptr))
+        pkg.check(dsx.dsx_fc_topk_split(dX.ptr, kdim, dW.ptr, xp.ptr, wp.ptr, pkg.ptr(db), batch, kdim, n, act, C.byref(params), k, keys.ptr,
+                                        vals.ptr, position, pkg.ptr(di), pkg.ptr(ds), pkg.ptr(de), pkg.ptr(dx)))
+    else:
+        pkg.check(dsx.dsx_fc_topk(dX.ptr, kdim, dW.ptr, pkg.ptr(db), batch, kdim, n, act, C.byref(params), k, keys.ptr, vals.ptr, position,
+                                  pkg.ptr(di), pkg.ptr(ds), pkg.ptr(de), pkg.ptr(dx)))
     Z = pkg.DeviceArray((batch, n), np.float32)
     pkg.check(dsx.dsx_fc_forward(dX.ptr, kdim, dW.ptr, 0, pkg.ptr(db), Z.ptr, n, batch, kdim, n, 0, act, C.byref(params)))
     k2 = pkg.DeviceArray((batch, k), np.float32)
@@ -120,7 +135,8 @@ def test_fc_topk_small_layers_and_short_rows(pkg, dsx, orc, rng, knobs):
         X, W, bias = layer(rng, batch, kdim, n)
         start, end, fidx = random_csr(rng, batch, n, min(n - 1, 50))
         gk, gi, _, tk, ti = run_both(pkg, dsx, orc, X, W, bias, ACT_SIGMOID, k, 0, None, start, end, fidx, "n=%d" % n)
-        assert np.array_equal(gi, ti) and np.array_equal(gk.view(np.uint32), tk.view(np.uint32))
+        if not MODE["split"]:      # the same kernel, the same scan: bit for bit (split products round differently: parity rules, above)
+            assert np.array_equal(gi, ti) and np.array_equal(gk.view(np.uint32), tk.view(np.uint32))
 
 
 def test_fc_topk_ties_and_full_lists_are_recomputed_exactly(pkg, dsx, orc, rng, knobs):

@@ -150,6 +150,26 @@ def test_cfg4_full_size(pkg, dsx, orc, synth):
     _, ref_scores, ref_keys, ref_idx = oracle_rows(orc, p, picks, p.k)
     assert_topk_parity(gk[picks], gi[picks], ref_keys, ref_idx, ref_scores, "cfg4 fused vs oracle")
     assert dsx.dsx_fc_topk_flagged(1) == 0
+    # the same call with the products formed from bf16 matrix instructions (dsx_fc_topk_split)
+    k_dim, n = p.widths[1], p.widths[2]
+    xp = pkg.DeviceArray((dsx.dsx_fc_split_bytes(p.batch, k_dim) // 4,), np.uint32)
+    wp = pkg.DeviceArray((dsx.dsx_fc_split_bytes(n, k_dim) // 4,), np.uint32)
+    pkg.check(dsx.dsx_fc_split(pipe.units[0].ptr, k_dim, 0, p.batch, k_dim, xp.ptr))
+    pkg.check(dsx.dsx_fc_split(pipe.W[1].ptr, n, 1, n, k_dim, wp.ptr))
+    pkg.check(dsx.dsx_fc_topk_split(pipe.units[0].ptr, k_dim, pipe.W[1].ptr, xp.ptr, wp.ptr, pipe.b[1].ptr, p.batch, k_dim, n, p.acts[1],
+                                    C.byref(pipe.params), p.k, fk.ptr, fi.ptr, 0, None, pipe.start.ptr, pipe.end.ptr, pipe.sidx.ptr))
+    sk, si = fk.numpy(), fi.numpy()
+    del xp, wp
+    say("cfg4 fused, split products: %d of %d indexes differ from the stored fp32 path, rows recomputed: %d"
+        % (int((si != idx).sum()), si.size, dsx.dsx_fc_topk_flagged(0)))
+    check_batch_properties(p, sk, si)
+    assert_close(sk, keys, "cfg4 fused split-product scores vs stored fp32 path", rel=1e-5)
+    mism = si != idx
+    assert mism.mean() < 1e-3
+    if mism.any():
+        assert np.abs(sk[mism].astype(np.float64) - keys[mism].astype(np.float64)).max() < 1e-5
+    assert_topk_parity(sk[picks], si[picks], ref_keys, ref_idx, ref_scores, "cfg4 fused with split products vs oracle")
+    assert dsx.dsx_fc_topk_flagged(1) == 0
 
 
 def test_cfg5_knn_full_size(pkg, dsx, orc, synth):

@@ -259,6 +259,13 @@ def test_network_api_split_products_hidden_layer_and_new_weights(pkg, dsx, orc, 
         net.close()
 
 
+def test_network_api_split_products_deferred_wide_output(pkg, dsx, orc, synth):
+    """An output layer wide enough to be computed together with its top-K (131,072 units or more): with split products that call is
+    dsx_fc_topk_split; the units asked for afterwards come from the storing kernel of the same mode."""
+    p = synth.autoencoder("split-wide-output", 1004, 140000, [512], 256, 100, 1, 1.1, 50, 1.0, (1, 1000))
+    host_forward_split(orc, p).close()
+
+
 # ---------------------------------------------------------------------------------------------------------------- exact KNN
 
 def knn_split_search(pkg, dsx, cm, rows, pad, dim, queries_m, k):
