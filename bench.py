@@ -25,6 +25,7 @@ import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP32_MFMA_PEAK_TF = 157.3    # MI355X dense fp32 matrix, published
+BF16_MFMA_PEAK_TF = 2500.0       # dense bf16 MFMA, the published figure
 
 # HBM bytes per launch, measured: profiles/pmc_hbm_traffic.json holds, per workload and kernel, what rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE read (KiB per dispatch) and the calibration factors from a plain 256 MiB device-to-device copy in the same runs; the
@@ -288,13 +289,37 @@ def network_bench(args, pkg, lib):
             "algorithmic_flops": flops, "frac": flops / ms / 1e9 / FP32_MFMA_PEAK_TF,
             "note": "what the timed step runs for this layer: first column block stored and scanned, the rest compared in registers"}
 
+    # The output layer's kernel of the split-products mode (off by default, so never the dominant kernel of `roofline`): priced as the
+    # bf16 matrix work it executes, six products per fp32 product, against the bf16 peak.
+    split_name = None
+    info = pkg.DeviceInfo()
+    pkg.check(lib.dsx_get_device_info(info))
+    if ((B + 127) // 128) * ((N + 127) // 128) >= 2 * info.compute_units:
+        kk = p.widths[last]
+        xs = pkg.DeviceArray((lib.dsx_fc_split_bytes(B, kk) // 4,), np.uint32, lib)
+        ws = pkg.DeviceArray((lib.dsx_fc_split_bytes(N, kk) // 4,), np.uint32, lib)
+        pkg.check(lib.dsx_fc_split(ptr(gp.W[last]), N, 1, N, kk, ws.ptr))
+        pkg.check(lib.dsx_fc_split(ptr(gp.units[last - 1]), kk, 0, B, kk, xs.ptr))
+
+        def k_split():
+            pkg.check(lib.dsx_fc_forward_split(xs.ptr, ws.ptr, ptr(gp.b[last]), ptr(gp.units[last]), N, B, kk, N, 0, p.acts[last], params,
+                                               ptr(gp.seg_max), C.byref(gp.seg_width)))
+        flops = 2.0 * B * kk * N
+        ms = time_launches(pkg, lib, k_split, reps)
+        split_name = "fc_gemm_split_kernel[%dx%dx%d]" % (B, kk, N)
+        kernels[split_name] = {"bound": "mfma", "ms": ms, "achieved": 6 * flops / ms / 1e9, "peak": BF16_MFMA_PEAK_TF, "unit": "TFLOP/s",
+                               "frac": 6 * flops / ms / 1e9 / BF16_MFMA_PEAK_TF, "algorithmic_flops": flops,
+                               "fp32_equivalent_tflops": flops / ms / 1e9,
+                               "note": "split-products mode only: six bf16 x bf16 products per fp32 product, priced as executed bf16 work against the bf16 peak"}
+        del xs, ws
+
     for n, t in traffic.items():
         if n in kernels:
             kernels[n]["traffic"] = t["read"] + t["write"]
             kernels[n]["traffic_read"] = t["read"]
             kernels[n]["traffic_write"] = t["write"]
 
-    candidates = [n for n in kernels if "frac" in kernels[n] and not (deferred and n in (gemm_name, "topk_scan_kernel"))]
+    candidates = [n for n in kernels if "frac" in kernels[n] and n != split_name and not (deferred and n in (gemm_name, "topk_scan_kernel"))]
     dominant = max(candidates, key=lambda n: kernels[n]["ms"])
     d = kernels[dominant]
     roofline = {"kernel": dominant, "bound": d["bound"], "achieved": round(d["achieved"], 3), "peak": d["peak"], "unit": d["unit"],
