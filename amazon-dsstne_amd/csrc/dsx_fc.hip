@@ -838,6 +838,9 @@ __global__ __launch_bounds__(kFcThreads, MH == 1 ? 3 : 2) void fc_gemm_split_ker
             woff -= wstep;
         }
         load();
+        // (the loads stay up here: left to itself the scheduler sinks them to the end of the step, right in front of the LDS
+        // stores that wait for them, and every step then pays a round trip to L2)
+        __builtin_amdgcn_sched_barrier(0);
         multiply(buf);
         store(buf ^ 1);
         __syncthreads();
