@@ -397,6 +397,9 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
             __syncthreads();
             auto k_step = [&](uint32_t kt, int buf) __attribute__((always_inline)) {
                 if (kt + 1 < nk) load_lean((kt + 1) * BK);
+                // (with two steps per trip the first step's condition is known to hold and its loads are straight-line code, which
+                // the scheduler sinks to the end of the step, in front of the LDS stores that wait for them: they stay up here)
+                __builtin_amdgcn_sched_barrier(0);
                 multiply(buf);
                 if (kt + 1 < nk) {
                     store_a(buf ^ 1);
