@@ -61,6 +61,7 @@ void NNLayer::Deallocate()
 {
     _pbUnit.reset();
     _pbSegMax.reset();
+    _pbSplitInput.reset();
     _segWidth = 0;
     _deferred = false;
     for (auto& set : _parked) set = LaneSet();
