@@ -75,7 +75,8 @@ def test_split_planes_special_values(pkg, dsx):
     assert abs(total[5] - 1e-40) <= 2.0 ** -134                                         # subnormal: to half a bf16 subnormal step
 
 
-SHAPES = [(300, 100, 1000), (130, 17, 257), (1, 128, 129), (257, 130, 128), (64, 512, 3000), (1024, 128, 5000)]
+SHAPES = [(300, 100, 1000), (130, 17, 257), (1, 128, 129), (257, 130, 128), (64, 512, 3000), (1024, 128, 5000), (1, 1, 1), (257, 1, 5),
+          (40, 4100, 300), (513, 33, 1)]
 
 
 @pytest.fixture(params=[128, 256])
@@ -280,7 +281,8 @@ def knn_split_search(pkg, dsx, cm, rows, pad, dim, queries_m, k):
 
 
 @pytest.mark.parametrize("items,queries,dim,k,blocks", [(1003, 9, 24, 10, 0), (50000, 64, 256, 100, 0), (30011, 70, 64, 100, 1024),
-                                                         (9000, 130, 256, 10, 1024), (26000, 33, 36, 200, 1024)])
+                                                         (9000, 130, 256, 10, 1024), (26000, 33, 36, 200, 1024), (100, 3, 8, 100, 0),
+                                                         (5000, 1, 4, 256, 1024)])
 def test_knn_search_split(pkg, dsx, orc, synth, items, queries, dim, k, blocks):
     """dsx_knn_search_split against the oracle, through the scanned first block alone and (blocks = 1,024: a first block of 1,024
     items) through the candidate ranges."""
