@@ -149,9 +149,11 @@ __device__ __forceinline__ void fc_epilogue(floatx16 (&acc)[MI][NI], const FcArg
 // TRANS: W is stored [n][k].
 // CAND: 0 = the result is stored (epilogue above); 1 = candidate mode, scores compared with score bounds (exact KNN);
 // 2 = candidate mode of a layer: the accumulators start from the bias, pre-activation sums are compared with bounds derived
-// from activated scores, and the survivors are activated (candidate_epilogue, PRE).
+// from activated scores, and the survivors are activated (candidate_epilogue, PRE).  That mode needs a few registers more than
+// 128 (its bounds and the bias beside the two-steps-per-trip loop): it is built for three workgroups per CU instead of spilling
+// at four (config 4, 4,096 x 512 x 1,000,000: 32.2 ms per step against 33.1 with one step per trip and four workgroups).
 template <int MI, int NI, int BK, int XV, int WV, bool TRANS, int ACT, int CAND = 0>
-__global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_kernel(FcArgs a)
+__global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? (CAND == 2 ? 3 : 4) : 2) void fc_gemm_kernel(FcArgs a)
 {
     constexpr int BM = 64 * MI, BN = 64 * NI;
     constexpr int LDA = BM + 4, LDB = BN + 4;
@@ -407,11 +409,10 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? 4 : 2) void fc_gemm_ke
                 }
                 __syncthreads();
             };
-            if constexpr (BK >= 16 && CAND != 2) {
+            if constexpr (BK >= 16) {
                 // Two k-steps per trip: each step's LDS buffer is then a constant and its addresses are immediate offsets, a
                 // dozen vector instructions less per step (1.5-1.8 % at k = 512 and 1,024; with steps of 8 the longer loop body
-                // costs more than that saves, and the layer's candidate mode, which also keeps its bounds and the bias in
-                // registers, would spill).
+                // costs more than that saves).
                 uint32_t kt = 0;
                 for (; kt + 1 < nk; kt += 2) {
                     k_step(kt, 0);
