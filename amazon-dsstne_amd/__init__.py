@@ -83,7 +83,7 @@ SIGNATURES = {
     "dsx_fc_forward": [_vp, _u32, _vp, _int, _vp, _vp, _u32, _u32, _u32, _u32, _int, _u32, C.POINTER(ActParams)],
     "dsx_fc_forward_segmax": [_vp, _u32, _vp, _int, _vp, _vp, _u32, _u32, _u32, _u32, _u32, C.POINTER(ActParams), _vp, C.POINTER(_u32)],
     "dsx_fc_split": [_vp, _u32, _int, _u32, _u32, _vp],
-    "dsx_fc_split_set_tile_rows": [_u32],
+    "dsx_testing_set_split_tile_rows": [_u32],
     "dsx_fc_forward_split": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _int, _u32, C.POINTER(ActParams), _vp, C.POINTER(_u32)],
     "dsx_activation": [_vp, _u32, _u32, _u32, C.POINTER(ActParams)],
     "dsx_add_buffers": [_vp, _vp, _u64],
@@ -98,15 +98,17 @@ SIGNATURES = {
     "dsx_fc_topk_split": [_vp, _u32, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, C.POINTER(ActParams), _u32, _vp, _vp, _u32, _vp, _vp, _vp, _vp],
     "dsx_fc_topk_supported": [_u32, _vp, _u32, C.POINTER(ActParams), _vp],
     "dsx_fc_topk_flagged": [_int],
-    "dsx_fc_topk_set_first_columns": [_u32],
-    "dsx_fc_topk_set_candidate_capacity": [_u32],
+    "dsx_fc_topk_flagged_for": [_vp, _int],
+    "dsx_testing_reset": [],
+    "dsx_testing_set_fc_topk_first_columns": [_u32],
+    "dsx_testing_set_fc_topk_candidate_capacity": [_u32],
     "dsx_knn_search": [_vp, _u32, _u32, _u32, _vp, _u32, _u32, _vp, _vp, _vp, _sz, C.POINTER(_f32)],
-    "dsx_knn_set_block_columns": [_u32],
+    "dsx_testing_set_knn_block_columns": [_u32],
     "dsx_knn_f16_convert_items": [_vp, _u32, _u32, _u32, _vp],
     "dsx_knn_search_f16": [_vp, _u32, _u32, _u32, _vp, _u32, _u32, _vp, _vp, _vp, _sz, C.POINTER(_f32)],
     "dsx_knn_search_split": [_vp, _u32, _u32, _u32, _vp, _u32, _u32, _vp, _vp, _vp, _sz, C.POINTER(_f32)],
     "dsx_knn_last_search_path": [],
-    "dsx_knn_f16_set_sweep": [_int],
+    "dsx_testing_set_knn_f16_sweep": [_int],
 }
 SPECIAL_RESTYPES = {"dsx_last_error": C.c_char_p, "dsx_stream": C.c_void_p, "dsx_knn_workspace_bytes": C.c_size_t,
                     "dsx_knn_workspace_bytes_f16": C.c_size_t, "dsx_knn_f16_table_bytes": C.c_size_t, "dsx_fc_split_bytes": _u64,

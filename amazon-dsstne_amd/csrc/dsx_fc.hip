@@ -864,7 +864,6 @@ __global__ __launch_bounds__(kFcThreads, MH == 1 ? 3 : 2) void fc_gemm_split_ker
     for (int h = 0; h < MH; h++) fc_epilogue<2, 2, ACT>(acc[h], a, row0 + wm * 64 * MH + h * 64, col0 + wn * 64, lane, sT);
 }
 
-static uint32_t g_split_tile_rows = 0;   // dsx_fc_split_set_tile_rows: 0 = by shape
 uint32_t split_rows_padded(uint32_t rows) { return (rows + 255) / 256 * 256; }
 static inline uint32_t split_kblocks(uint32_t k) { return (k + 15) / 16 * 2; }
 uint64_t split_plane_bytes(uint32_t rows, uint32_t k) { return 3ull * split_rows_padded(rows) * split_kblocks(k) * 16; }
@@ -906,7 +905,7 @@ int fc_split_run(const void* Xs, const void* Ws, uint32_t wrows, uint32_t wcol0,
     // 256-row tiles for long sums, when they still give every CU its two workgroups twice over (4,096 x 512 x 262,144: 5,410
     // against 5,730 us; with k = 128 the epilogue dominates and the smaller tiles' third workgroup per CU is worth more)
     int mh = (k >= 512 && (uint64_t)((batch + 255) / 256) * a.tiles_n >= 4ull * ctx().num_cus) ? 2 : 1;
-    if (g_split_tile_rows) mh = g_split_tile_rows == 256 ? 2 : 1;
+    if (ctx().knobs.split_tile_rows) mh = ctx().knobs.split_tile_rows == 256 ? 2 : 1;
     a.tiles_m = (batch + 128 * mh - 1) / (128 * mh);
     if (seg_max && seg_width && !accumulate) {
         a.seg_max = seg_max;
@@ -1042,10 +1041,10 @@ int dsx_fc_split(const float* src, uint32_t ld, int k_major, uint32_t rows, uint
     return k_major ? fc_split_planes_run(src, 1, ld, rows, k, planes) : fc_split_planes_run(src, ld, 1, rows, k, planes);
 }
 
-int dsx_fc_split_set_tile_rows(uint32_t rows)
+int dsx_testing_set_split_tile_rows(uint32_t rows)
 {
-    if (rows != 0 && rows != 128 && rows != 256) return set_error(DSX_EINVAL, "dsx_fc_split_set_tile_rows: %u (0, 128 or 256)", rows);
-    g_split_tile_rows = rows;
+    if (rows != 0 && rows != 128 && rows != 256) return set_error(DSX_EINVAL, "dsx_testing_set_split_tile_rows: %u (0, 128 or 256)", rows);
+    ctx().knobs.split_tile_rows = rows;
     return DSX_OK;
 }
 

@@ -7,7 +7,8 @@
 // scanned: that leaves, per row, a best list and the key of its k-th score.  Every later column range, each several times as
 // wide as everything before it, runs the same GEMM kernel in candidate mode: the tile's pre-activation sums are compared with
 // the rows' bounds in registers and only the few survivors are activated and appended to per-row lists, which a small kernel
-// folds into the best lists after dropping the columns the row's filter names.  Exact for any input: admission is a superset
+// folds into the best lists after dropping the columns the row's filter names (a row whose result a listed column's score * 0
+// could enter - fewer than k scores above 0 - is recomputed with those zeros in place).  Exact for any input: admission is a superset
 // of "score >= current k-th score" (preactivation_bound in dsx_device.h), lists are merged under the total order (score
 // descending, column ascending), and a row whose list fills up is recomputed from scratch on the device.
 #include <algorithm>
@@ -17,10 +18,33 @@
 namespace dsx {
 
 constexpr uint32_t kLayerCandCap = 4096;       // candidate words per row and column range
-static uint32_t g_layer_first_columns = 0;     // 0: default
-static uint32_t g_layer_cap = kLayerCandCap;   // tests lower it to reach the overflow path with small inputs
 static LibScratch g_layer_ws_of[DSX_MAX_LANES];   // per lane
-static uint32_t* g_layer_flagged = nullptr;    // pinned host memory: the device stores 1 there when it flags a row
+// Pinned host memory: the device stores 1 in a word when it flags a row.  One word per weight matrix (the layer a call belongs
+// to), so that one layer's tied scores say nothing about another's; kFlagWords matrices at a time, the oldest gives way.
+constexpr int kFlagWords = 64;
+static uint32_t* g_layer_flagged = nullptr;
+static const void* g_flag_owner[kFlagWords] = {};
+static int g_flag_next = 0;
+
+static void layer_flags_release()
+{
+    if (g_layer_flagged) hipHostFree(g_layer_flagged);
+    g_layer_flagged = nullptr;
+    for (auto& o : g_flag_owner) o = nullptr;
+    g_flag_next = 0;
+}
+
+static int layer_flag_slot(const void* W, bool create)
+{
+    for (int i = 0; i < kFlagWords; i++)
+        if (g_flag_owner[i] == W) return i;
+    if (!create) return -1;
+    const int i = g_flag_next;
+    g_flag_next = (g_flag_next + 1) % kFlagWords;
+    g_flag_owner[i] = W;
+    *(volatile uint32_t*)&g_layer_flagged[i] = 0;
+    return i;
+}
 
 __global__ __launch_bounds__(256) void layer_clear_kernel(uint32_t* p, uint32_t n)
 {
@@ -32,7 +56,7 @@ static inline size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 
 static uint32_t layer_first_columns(uint32_t n, uint32_t k)
 {
-    uint32_t c = g_layer_first_columns ? g_layer_first_columns : 2048;
+    uint32_t c = ctx().knobs.fc_topk_first_columns ? ctx().knobs.fc_topk_first_columns : 2048;
     c = std::max(c, (k + 127) / 128 * 128);   // at least k candidates for the first bound
     c = (c + 127) / 128 * 128;
     // when the first block would be most of the layer anyway, the whole layer goes through the scratch matrix
@@ -88,25 +112,37 @@ using namespace dsx;
 
 extern "C" {
 
-int dsx_fc_topk_set_first_columns(uint32_t columns)
+int dsx_testing_set_fc_topk_first_columns(uint32_t columns)
 {
-    g_layer_first_columns = std::min(columns, 131072u);   // the first block's filter bitmap lives in LDS
+    ctx().knobs.fc_topk_first_columns = std::min(columns, 131072u);   // the first block's filter bitmap lives in LDS
     return DSX_OK;
 }
 
-int dsx_fc_topk_set_candidate_capacity(uint32_t words)
+int dsx_testing_set_fc_topk_candidate_capacity(uint32_t words)
 {
-    if (words == 0) words = kLayerCandCap;
-    DSX_CHECK_ARG(words >= 64 && words <= kLayerCandCap, "dsx_fc_topk_set_candidate_capacity: %u words (64..%u)", words, kLayerCandCap);
-    g_layer_cap = words;
+    DSX_CHECK_ARG(words == 0 || (words >= 64 && words <= kLayerCandCap), "dsx_testing_set_fc_topk_candidate_capacity: %u words (64..%u)", words, kLayerCandCap);
+    ctx().knobs.fc_topk_candidate_capacity = words;
     return DSX_OK;
 }
 
 int dsx_fc_topk_flagged(int reset)
 {
     if (!g_layer_flagged) return 0;
-    const int seen = *(volatile uint32_t*)g_layer_flagged != 0;
-    if (reset) *(volatile uint32_t*)g_layer_flagged = 0;
+    int seen = 0;
+    for (int i = 0; i < kFlagWords; i++) {
+        seen |= *(volatile uint32_t*)&g_layer_flagged[i] != 0;
+        if (reset) *(volatile uint32_t*)&g_layer_flagged[i] = 0;
+    }
+    return seen;
+}
+
+int dsx_fc_topk_flagged_for(const float* W, int reset)
+{
+    if (!g_layer_flagged) return 0;
+    const int i = layer_flag_slot(W, false);
+    if (i < 0) return 0;
+    const int seen = *(volatile uint32_t*)&g_layer_flagged[i] != 0;
+    if (reset) *(volatile uint32_t*)&g_layer_flagged[i] = 0;
     return seen;
 }
 
@@ -135,10 +171,12 @@ static int fc_topk_common(const float* X, uint32_t ldx, const float* W, const fl
                          activation);
     if (batch == 0) return DSX_OK;
     if (!g_layer_flagged) {
-        DSX_HIP(hipHostMalloc((void**)&g_layer_flagged, 256, hipHostMallocMapped));
-        *g_layer_flagged = 0;
+        DSX_HIP(hipHostMalloc((void**)&g_layer_flagged, kFlagWords * sizeof(uint32_t), hipHostMallocMapped));
+        for (int i = 0; i < kFlagWords; i++) g_layer_flagged[i] = 0;
+        at_shutdown(layer_flags_release);
     }
-    const uint32_t cap = g_layer_cap;
+    uint32_t* const flag_word = g_layer_flagged + layer_flag_slot(W, true);
+    const uint32_t cap = ctx().knobs.fc_topk_candidate_capacity ? ctx().knobs.fc_topk_candidate_capacity : kLayerCandCap;   // tests lower it to reach the overflow path with small inputs
     const uint32_t n0 = layer_first_columns(n, k);
     const bool ranges = n0 < n;
     const size_t need = layer_layout(nullptr, batch, n0, k, cap, ranges).bytes;
@@ -187,13 +225,13 @@ static int fc_topk_common(const float* X, uint32_t ldx, const float* W, const fl
         done += ncols;
         LayerRefresh r{};
         r.best = w.best; r.cand = w.cand; r.cand_count = w.cand_count; r.cap = cap; r.k = k;
-        r.row_bound = w.row_bound; r.row_flag = w.row_flag; r.flagged_total = g_layer_flagged;
+        r.row_bound = w.row_bound; r.row_flag = w.row_flag; r.flagged_total = flag_word;
         r.position = position; r.index = index; r.fstart = filter_start; r.fend = filter_end; r.fidx = filter_index;
         if (done == n) {
             r.keys = keys;
             r.values = values;
         }
-        r.X = X; r.W = W; r.bias = bias; r.ldx = ldx; r.ldw = n; r.kdim = kdim; r.n = n;
+        r.X = X; r.W = W; r.bias = bias; r.ldx = ldx; r.ldw = n; r.kdim = kdim; r.n = n; r.first_columns = n0;
         r.act = activation; r.slope = cand.slope; r.alpha = cand.alpha; r.lambda = cand.lambda;
         rc = layer_refresh_run(r, batch);
         if (rc) return rc;

@@ -5,11 +5,23 @@
 #include <cstdint>
 #include <cstdio>
 #include "dsx.h"
+#include "dsx_testing.h"
 
 namespace dsx {
 
+// Switches of include/dsx_testing.h (0 = default unless stated).
+struct TestKnobs {
+    uint32_t split_tile_rows = 0;
+    uint32_t fc_topk_first_columns = 0;
+    uint32_t fc_topk_candidate_capacity = 0;
+    uint32_t knn_block_columns = 0;
+    int knn_f16_sweep = 1;
+};
+
 struct Context {
+    TestKnobs knobs;
     bool initialized = false;
+    bool sync_launches = false;   // DSX_SYNC=1: wait for every kernel right after its launch
     int users = 0;          // dsx_init calls not yet matched by dsx_shutdown
     int device = 0;
     hipStream_t stream = nullptr;
@@ -31,8 +43,11 @@ struct LibScratch {
 // Makes s hold at least `bytes` (contents are not preserved when it grows; the selected lane is waited for before the old
 // block is freed).
 int lib_scratch_reserve(LibScratch& s, size_t bytes, const char* what);
+// fn runs once in the last dsx_shutdown, before the library's memory is released (file-scope state of the other translation units).
+void at_shutdown(void (*fn)());
 int current_lane();   // 0 or 1: which of the two in-order streams ctx().stream is (scratch buffers are kept per lane)
 int set_error(int code, const char* fmt, ...);
+int sync_after_launch(const char* fn, const char* kernel);   // DSX_SYNC=1, see DSX_LAUNCH_CHECK
 
 // engine/NNTypes.h:49
 constexpr float kMaxValue = 999999999999999.0f;
@@ -55,11 +70,17 @@ constexpr float kMaxValue = 999999999999999.0f;
         if (!(cond)) return dsx::set_error(DSX_EINVAL, __VA_ARGS__); \
     } while (0)
 
-// After a kernel launch: pick up launch-configuration errors (the analogue of LAUNCHERROR, engine/GpuTypes.h:215-223).
+// After a kernel launch: pick up launch-configuration errors (the analogue of LAUNCHERROR, engine/GpuTypes.h:215-223).  With
+// DSX_SYNC=1 in the environment when dsx_init runs (the reference's compile-time SYNCHRONOUS, engine/GpuTypes.h:147-176) every
+// launch is also waited for, so that a failure inside a kernel is reported by the call that launched it, with the kernel's name;
+// never while the stream is being captured into a graph.
 #define DSX_LAUNCH_CHECK(name)                                                                                     \
     do {                                                                                                           \
         hipError_t e_ = hipGetLastError();                                                                         \
         if (e_ != hipSuccess) return dsx::set_error(DSX_EHIP, "%s: launch of %s failed: %s", __func__, name, hipGetErrorString(e_)); \
+        if (dsx::ctx().sync_launches) {                                                                            \
+            if (int rc_ = dsx::sync_after_launch(__func__, name)) return rc_;                                      \
+        }                                                                                                          \
     } while (0)
 
 namespace dsx {
@@ -123,6 +144,7 @@ struct LayerRefresh {
     const float* W;
     const float* bias;
     uint32_t ldx, ldw, kdim, n;
+    uint32_t first_columns;   // width of the first block (scanned with the filter applied)
     uint32_t act;
     float slope, alpha, lambda;
 };
@@ -138,7 +160,7 @@ int knn_refresh(uint64_t* best, const uint64_t* cand, uint32_t* cand_count, uint
                 const uint64_t* seg = nullptr, uint32_t* seg_count = nullptr, uint32_t chunks = 0, uint32_t seg_cap = 0);
 // fp16 storage, candidate mode of a column range: one workgroup per tile, or (long ranges) workgroups that sweep a chunk of the
 // range each and keep (row, chunk) lists of their own (seg [queries][chunks][seg_words / chunks], seg_count [queries][64]); full
-// lists spill into cand's shared ones.  mode: see dsx_knn_f16_set_sweep.  *chunks_used is what knn_refresh needs to know.
+// lists spill into cand's shared ones.  mode: see dsx_testing_set_knn_f16_sweep.  *chunks_used is what knn_refresh needs to know.
 int knn_f16_candidates_run(const void* queries16, const void* items16, uint32_t ld, uint32_t batch, uint32_t n, const CandArgs& cand,
                            uint64_t* seg, uint32_t* seg_count, uint32_t seg_words, int mode, uint32_t* chunks_used);
 }  // namespace dsx

@@ -20,15 +20,13 @@ namespace dsx {
 
 static LibScratch g_knn_ws_of[DSX_MAX_LANES];   // per lane
 
-static uint32_t g_knn_block_columns = 0;   // 0: sized by the rule below
 static int g_knn_last_path = 0;            // how the last search ran: DSX_KNN_PATH_*
-static int g_knn_f16_sweep = 1;            // fp16 storage, see dsx_knn_f16_set_sweep
 
 static uint32_t knn_block_columns(uint32_t rows_padded, uint32_t num_queries)
 {
     // about 1 GiB of scores per block, a multiple of 1024 columns
     uint64_t cols = ((uint64_t)1 << 30) / ((uint64_t)std::max(1u, num_queries) * sizeof(float));
-    if (g_knn_block_columns) cols = g_knn_block_columns;
+    if (ctx().knobs.knn_block_columns) cols = ctx().knobs.knn_block_columns;
     cols = std::max<uint64_t>(1024, cols / 1024 * 1024);
     cols = std::min<uint64_t>(cols, ((uint64_t)rows_padded + 1023) / 1024 * 1024);
     return (uint32_t)cols;
@@ -117,7 +115,7 @@ struct KnnOperands {
         *chunks_used = 0;
         if (f16)
             return knn_f16_candidates_run(queries16, items16 + (uint64_t)c0 * ld16 * 2, ld16, num_queries, ncols, cand, seg, seg_count, kCandCap,
-                                          g_knn_f16_sweep, chunks_used);
+                                          ctx().knobs.knn_f16_sweep, chunks_used);
         if (split) return fc_split_candidates_run(query_planes, item_planes, split_rows_padded(rows_padded), c0, num_queries, dim, ncols, cand);
         return fc_candidates_run(queries, dim, items + c0, rows_padded, num_queries, dim, ncols, cand);
     }
@@ -178,7 +176,7 @@ static int knn_search_candidates(const KnnWorkspace& w, const KnnOperands& op, u
     // The first block only has to give every query a usable bound; a quarter of a column block does (measured on 2 M items x 4,096
     // queries: 8 K to 32 K columns are level, the full 64 K cost 0.1 ms more in stores and scan).  A width set by the caller is kept.
     uint32_t done = std::min(cb, M);
-    if (!g_knn_block_columns) done = std::min<uint32_t>(done, std::max<uint32_t>(1024, cb / 4 / 1024 * 1024));
+    if (!ctx().knobs.knn_block_columns) done = std::min<uint32_t>(done, std::max<uint32_t>(1024, cb / 4 / 1024 * 1024));
     t.start(s);
     int rc = op.into_matrix(0, done, num_queries, w.block_scores, cb);
     if (rc) return rc;
@@ -221,18 +219,18 @@ using namespace dsx;
 
 extern "C" {
 
-int dsx_knn_set_block_columns(uint32_t columns)
+int dsx_testing_set_knn_block_columns(uint32_t columns)
 {
-    g_knn_block_columns = columns;
+    ctx().knobs.knn_block_columns = columns;
     return DSX_OK;
 }
 
 int dsx_knn_last_search_path(void) { return g_knn_last_path; }
 
-int dsx_knn_f16_set_sweep(int mode)
+int dsx_testing_set_knn_f16_sweep(int mode)
 {
-    DSX_CHECK_ARG(mode >= 0 && mode <= 3, "dsx_knn_f16_set_sweep: mode %d (0 to 3)", mode);
-    g_knn_f16_sweep = mode;
+    DSX_CHECK_ARG(mode >= 0 && mode <= 3, "dsx_testing_set_knn_f16_sweep: mode %d (0 to 3)", mode);
+    ctx().knobs.knn_f16_sweep = mode;
     return DSX_OK;
 }
 
@@ -290,12 +288,14 @@ static int knn_search_common(KnnOperands& op, uint32_t padding, uint32_t num_que
     if (op.f16) {   // the query batch in the table's format (knn/KnnExactGpu.cu:108-116); counted as GEMM time like the copy it replaces
         t.start(s);
         rc = knn_to_f16(queries_f32, false, op.dim, num_queries, op.dim, w.queries16, (uint32_t)knn_f16_rows(num_queries));
+        if (rc) return rc;
         t.stop(s, t.gemm);
         op.queries16 = w.queries16;
     }
     if (op.split) {   // the query batch as bf16 planes, counted as GEMM time too
         t.start(s);
         rc = fc_split_planes_run(queries_f32, op.dim, 1, num_queries, op.dim, w.queries16);
+        if (rc) return rc;
         t.stop(s, t.gemm);
         op.query_planes = w.queries16;
     }

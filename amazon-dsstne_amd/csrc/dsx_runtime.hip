@@ -1,4 +1,5 @@
 // dsx_runtime.hip — context, memory and timing entry points of libdsx_hip.so.
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -22,6 +23,26 @@ int set_error(int code, const char* fmt, ...)
     vsnprintf(g_error, sizeof(g_error), fmt, ap);
     va_end(ap);
     return code;
+}
+
+}  // namespace dsx
+// How many launches DSX_SYNC=1 has waited for so far (a plain exported counter for the tests; not a function of the ABI).
+extern "C" int dsx_debug_sync_launches;
+int dsx_debug_sync_launches = 0;
+namespace dsx {
+
+int sync_after_launch(const char* fn, const char* kernel)
+{
+    hipStream_t s = ctx().stream;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return DSX_OK;
+    }
+    const hipError_t e = hipStreamSynchronize(s);
+    if (e != hipSuccess) return set_error(DSX_EHIP, "%s: kernel %s failed: %s", fn, kernel, hipGetErrorString(e));
+    ++dsx_debug_sync_launches;
+    return DSX_OK;
 }
 
 static std::mutex g_alloc_mutex;
@@ -53,6 +74,14 @@ int lib_scratch_reserve(LibScratch& s, size_t bytes, const char* what)
         g_lib_scratch.push_back(&s);
     }
     return DSX_OK;
+}
+
+static std::vector<void (*)()> g_shutdown_hooks;
+void at_shutdown(void (*fn)())
+{
+    for (auto f : g_shutdown_hooks)
+        if (f == fn) return;
+    g_shutdown_hooks.push_back(fn);
 }
 
 static void lib_scratch_release()
@@ -218,6 +247,8 @@ int dsx_init(int device)
     c.num_cus = prop.multiProcessorCount;
     c.initialized = true;
     c.users = 1;
+    const char* sync = getenv("DSX_SYNC");
+    c.sync_launches = sync && sync[0] != '\0' && strcmp(sync, "0") != 0;
     return DSX_OK;
 }
 
@@ -230,6 +261,8 @@ int dsx_shutdown(void)
         if (g_lane_stream[l]) hipStreamSynchronize(g_lane_stream[l]);
     if (g_lane_stream[0]) c.stream = g_lane_stream[0];
     hipStreamSynchronize(c.stream);
+    for (auto fn : g_shutdown_hooks) fn();
+    g_shutdown_hooks.clear();
     lanes_release();
     upload_ring_release();
     {
@@ -245,6 +278,12 @@ int dsx_shutdown(void)
     hipEventDestroy(c.ev_stop);
     hipStreamDestroy(c.stream);
     c = Context();
+    return DSX_OK;
+}
+
+int dsx_testing_reset(void)
+{
+    ctx().knobs = TestKnobs();
     return DSX_OK;
 }
 

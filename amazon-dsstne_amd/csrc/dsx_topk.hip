@@ -1230,6 +1230,7 @@ struct LayerRefreshArgs {
     const float* W;
     const float* bias;
     uint32_t ldx, ldw, kdim, n;
+    uint32_t first_columns;    // columns of the first block, whose listed columns the scanning top-K has dealt with
     uint32_t act;
     float slope, alpha, lambda;
 };
@@ -1270,10 +1271,11 @@ __device__ __forceinline__ void layer_recompute_row(WaveTopK<R>& list, const Lay
             }
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const float y = activate_rt(sum[j], a.act, a.slope, a.alpha, a.lambda);
+                float y = activate_rt(sum[j], a.act, a.slope, a.alpha, a.lambda);
                 const uint32_t off = col[j] - C0;
-                const bool ok = col[j] < C1 && y == y && !((sBits[off >> 5] >> (off & 31)) & 1u);
-                list.offer(ok, pack_score(y, col[j]));
+                // a listed column keeps its place with score * 0 (utils/Filters.cpp:62), once however often it is listed
+                if (col[j] < C1 && ((sBits[off >> 5] >> (off & 31)) & 1u)) y *= 0.0f;
+                list.offer(col[j] < C1 && y == y, pack_score(y, col[j]));
             }
         }
         __builtin_amdgcn_wave_barrier();
@@ -1303,7 +1305,7 @@ __global__ __launch_bounds__(kWave) void layer_refresh_kernel(LayerRefreshArgs a
     const bool final_range = a.keys != nullptr;
     if (flagged && !final_range) return;
     uint64_t fs = 0, fe = 0;
-    if (a.fidx && (count > 0 || flagged)) {
+    if (a.fidx && (count > 0 || flagged || final_range)) {
         uint32_t r = a.position + b;
         if (a.index) r = a.index[r];
         fs = a.fstart[r];
@@ -1377,6 +1379,31 @@ __global__ __launch_bounds__(kWave) void layer_refresh_kernel(LayerRefreshArgs a
     }
     list.finish();
     if (final_range) {
+        // The listed columns beyond the first block were struck out above, but a listed column scores 0, not nothing
+        // (utils/Filters.cpp:62 multiplies, kCalculateTopK then sees the zero): when the row's k-th score is not above 0, or the
+        // row has fewer than k scores, such a zero belongs in the result.  Those rows are computed again, column by column.
+        uint64_t kth = 0;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const uint64_t w = shfl_u64(list.q[r], (int)((a.k - 1) & (kWave - 1)));
+            if ((int)((a.k - 1) / kWave) == r) kth = w;
+        }
+        bool zeros_matter = false;
+        if (fe > fs && (kth == 0 || (uint32_t)(kth >> 32) <= score_key(0.0f))) {
+            bool beyond = false;
+            for (uint64_t t = fs + lane; t < fe; t += kWave) {
+                const uint32_t col = a.fidx[t];
+                beyond |= col >= a.first_columns && col < a.n;
+            }
+            zeros_matter = __ballot(beyond) != 0;
+        }
+        if (zeros_matter) {
+            if (lane == 0 && a.flagged_total) *(volatile uint32_t*)a.flagged_total = 1u;
+            __builtin_amdgcn_wave_barrier();
+            list.init(sStage, lane, a.k);
+            layer_recompute_row<R>(list, a, b, lane, fs, fe, sTable);
+            list.finish();
+        }
         write_final<R>(list.q, lane, a.k, 0, a.keys + (uint64_t)b * a.k, a.values + (uint64_t)b * a.k);
         return;
     }
@@ -1397,6 +1424,7 @@ int layer_refresh_run(const LayerRefresh& r, uint32_t batch)
     a.position = r.position; a.index = r.index; a.fstart = r.fstart; a.fend = r.fend; a.fidx = r.fidx;
     a.keys = r.keys; a.values = r.values;
     a.X = r.X; a.W = r.W; a.bias = r.bias; a.ldx = r.ldx; a.ldw = r.ldw; a.kdim = r.kdim; a.n = r.n;
+    a.first_columns = r.first_columns;
     a.act = r.act; a.slope = r.slope; a.alpha = r.alpha; a.lambda = r.lambda;
     hipStream_t s = ctx().stream;
     if (a.k <= 64) hipLaunchKernelGGL((layer_refresh_kernel<1>), dim3(batch), dim3(kWave), 0, s, a);

@@ -169,7 +169,7 @@ void NNLayer::ForwardPropagateFullyConnected(uint32_t position, uint32_t batch, 
             // without the layer's result ever being stored.  The layer is computed when somebody asks for it.
             if (_bDeferOutput && _localStride >= kDeferMinWidth && !w->_bTransposed && _vOutgoingLayer.empty() && _vOutgoingSkip.empty() &&
                 dsx_fc_topk_supported(src->_stride, src->GetUnitBuffer(), (uint32_t)_activation, &params, NULL)) {
-                if (dsx_fc_topk_flagged(0)) {
+                if (dsx_fc_topk_flagged_for(wsrc->_pbWeight->_pDevData, 0)) {
                     // rows whose survivor lists filled up had to be recomputed one by one: this data (thousands of scores tied at the
                     // top of a row) is served better by the stored layer and the scanning top-K
                     printf("NNLayer::ForwardPropagate: scores of layer %s tie in their thousands; its result is stored from now on.\n", _name.c_str());

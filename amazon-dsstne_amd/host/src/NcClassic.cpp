@@ -234,8 +234,19 @@ void Reader::readRaw(const Variable& v, std::vector<uint8_t>& raw) const
     in.seekg(0, std::ios::end);
     const uint64_t fileSize = (uint64_t)in.tellg();
     size_t es = typeSize(v.type);
-    if (v.count > (fileSize + v.inlineData.size() + 8) / es && !(v.hdf5 && (v.chunked || v.begin == ~0ull)))
-        throw Error(_fname + ": variable " + v.name + " claims more data than the file holds");
+    // What a variable may claim: no more than the file can hold where its values are stored in one piece; for a chunked
+    // variable no more than its chunks hold (DSSTNE writes every value, so every chunk exists); a variable that was declared
+    // and never written reads as zeros, up to 256 MiB of them.
+    uint64_t limit = (fileSize + v.inlineData.size() + 8) / es;
+    if (v.hdf5 && v.chunked) {
+        limit = 0;
+        for (const Variable::Extent& e : v.extents) {
+            if (e.count > fileSize) throw Error(_fname + ": variable " + v.name + " has a chunk larger than the file");
+            limit += e.count;
+        }
+    } else if (v.hdf5 && !v.compact && v.begin == ~0ull)
+        limit = (1ull << 28) / es;
+    if (v.count > limit) throw Error(_fname + ": variable " + v.name + " claims more data than the file holds");
     raw.assign((size_t)(v.count * es), 0);
     auto readAt = [&](uint64_t offset, uint8_t* dst, uint64_t bytes) {
         if (offset > fileSize || bytes > fileSize - offset) throw Error(_fname + ": variable " + v.name + " is truncated");
@@ -255,6 +266,7 @@ void Reader::readRaw(const Variable& v, std::vector<uint8_t>& raw) const
         for (const Variable::Extent& e : v.extents) {
             if (e.first >= v.count) continue;
             const uint64_t n = std::min(e.count, v.count - e.first);   // the last chunk may reach beyond the variable
+            if (e.first * es > raw.size() || n * es > raw.size() - e.first * es) throw Error(_fname + ": variable " + v.name + " has a chunk outside its extent");
             readAt(e.offset, raw.data() + e.first * es, n * es);
         }
     } else if (v.begin != ~0ull) {

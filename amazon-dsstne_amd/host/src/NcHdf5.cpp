@@ -87,7 +87,13 @@ struct Cur {
         return ok;
     }
     const uint8_t* here() const { return p + at; }
-    size_t left() const { return n - at; }
+    size_t left() const { return at < n ? n - at : 0; }
+    // Moves to an absolute position taken from fields of the file; a position beyond the block is an error, not a cursor.
+    void seek(size_t to)
+    {
+        if (to > n) f.fail("a structure is shorter than its fields");
+        at = to;
+    }
 };
 
 struct Msg {
@@ -120,6 +126,7 @@ struct Parser {
     explicit Parser(const std::string& fname) : f(fname) {}
 
     uint64_t rootHeader = kUndef;
+    uint64_t chunkEntries_ = 0;   // entries of chunk B-tree nodes visited so far, all variables together
 
     void superblock()
     {
@@ -301,6 +308,12 @@ struct Parser {
         if (rank > 32) f.fail("dataspace of rank " + std::to_string(rank));
         for (unsigned i = 0; i < rank; i++) s.dims.push_back(c.len());
         if (flags & 1) c.skip((size_t)rank * f.L);
+        // the element count must stay a number that sizes and offsets can be computed from (16-byte elements at most)
+        uint64_t product = 1;
+        for (uint64_t d : s.dims) {
+            if (d != 0 && product > (1ull << 58) / d) f.fail("a dataspace of more than 2^58 elements");
+            product *= d;
+        }
         return s;
     }
 
@@ -323,12 +336,10 @@ struct Parser {
         if (version == 1) c.skip((8 - (nameSize & 7)) & 7);
         size_t at = c.at;
         TypeInfo t = datatype(c);
-        c.at = at + typeSize_;
-        if (version == 1) c.at += (8 - (typeSize_ & 7)) & 7;
+        c.seek(at + typeSize_ + (version == 1 ? (8 - (typeSize_ & 7)) & 7 : 0));
         at = c.at;
         SpaceInfo s = dataspace(c);
-        c.at = at + spaceSize;
-        if (version == 1) c.at += (8 - (spaceSize & 7)) & 7;
+        c.seek(at + spaceSize + (version == 1 ? (8 - (spaceSize & 7)) & 7 : 0));
         if (t.nc == 0 || s.dims.size() > 1) return false;
         a.name = name;
         a.type = t.nc;
@@ -595,7 +606,7 @@ struct Parser {
                 if (heapAddr == kUndef || nameTree == kUndef) continue;
                 FractalHeap h = openHeap(heapAddr);
                 btree2(nameTree, 8, [&](const uint8_t* rec, unsigned recSize) {
-                    if (recSize < 8) f.fail("attribute index record too short");
+                    if (recSize < 9) f.fail("attribute index record too short");
                     if (rec[8] & 2) return;   // a shared attribute message
                     std::vector<uint8_t> obj = heapObject(h, rec, 8);
                     Attribute a;
@@ -659,6 +670,10 @@ struct Parser {
         const unsigned type = c.u8(), level = c.u8(), used = c.u16();
         if (type != 1) f.fail("chunk B-tree of the wrong type");
         const uint64_t keyLen = 8 + 8ull * dimensionality;
+        // every entry of a real index occupies its own bytes of the file: more entries than the file has room for means the
+        // tree's pointers run in a circle
+        chunkEntries_ += used;
+        if (chunkEntries_ > f.size / (keyLen + f.O) + 1) f.fail("chunk B-tree with more entries than the file can hold");
         std::vector<uint8_t> body = f.bytes(abs(addr) + 8 + 2 * f.O, used * (keyLen + f.O) + keyLen);
         Cur b(body, f);
         for (unsigned i = 0; i < used; i++) {

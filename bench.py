@@ -104,8 +104,9 @@ def timed_windows(step, sync, steps, windows):
 
 
 def network_bench(args, pkg, lib):
-    from amazon_dsstne_amd import ATTR_BOOLEAN, ATTR_INDEXED, synth
-    from amazon_dsstne_amd.pipeline import DevicePipeline
+    from amazon_dsstne_amd import ATTR_BOOLEAN, ATTR_INDEXED
+    from dsx_support import synth
+    from dsx_support.pipeline import DevicePipeline
 
     from amazon_dsstne_amd.host_api import Network
 
@@ -396,7 +397,7 @@ def network_bench(args, pkg, lib):
 
 
 def knn_bench(args, pkg, lib):
-    from amazon_dsstne_amd import synth
+    from dsx_support import synth
 
     p = synth.knn_config(items=args.knn_items)
     cm, rows, pad = p.column_major_padded()

@@ -221,12 +221,10 @@ int dsx_fc_forward_segmax(const float* X, uint32_t ldx, const float* W, int tran
  * dsx_fc_forward_split then computes Z as dsx_fc_forward (accumulate, bias, activation) and, with seg_max / seg_width non-NULL
  * and accumulate == 0, the segment maxima as dsx_fc_forward_segmax (*seg_width = 64 for every shape).  A plane (2 bytes x rows
  * padded x k padded) must stay below 4 GiB.
- * dsx_fc_split_set_tile_rows(128 | 256) fixes the rows of a workgroup's tile (tests reach both kernels with small shapes);
- * 0, the default, chooses by shape: 256 for k >= 512 when that still leaves four tiles per compute unit.  Results do not
+ * A workgroup's tile has 128 rows, or 256 for k >= 512 when that still leaves four tiles per compute unit; results do not
  * depend on it. */
 uint64_t dsx_fc_split_bytes(uint32_t rows, uint32_t k);
 int dsx_fc_split(const float* src, uint32_t ld, int k_major, uint32_t rows, uint32_t k, void* planes);
-int dsx_fc_split_set_tile_rows(uint32_t rows);
 int dsx_fc_forward_split(const void* x_planes, const void* w_planes, const float* bias, float* Z, uint32_t ldz, uint32_t batch, uint32_t k,
                          uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params, float* seg_max,
                          uint32_t* seg_width);
@@ -292,13 +290,15 @@ int dsx_topk_guided(const float* in, float* keys, uint32_t* values, uint32_t bat
 /* Output layer and recommendations in one call: the forward GEMM of NNLayer::ForwardPropagateFullyConnected (bias, product,
  * activation; engine/NNLayer.cpp:994-1167) on the output layer, followed by NNRecsGenerator::generateRecs' filtered
  * kCalculateTopK (utils/NNRecsGenerator.cpp:83-150) over its result, without ever storing the [batch x n] result:
- *   keys/values[b] = top-k over columns j of act(bias[j] + sum_i X[b][i] * W[i][j]), the columns listed in row b's filter dropped
- * (filter arguments as dsx_topk_filtered with filter_mul == NULL; filter_index == NULL: no filter).  W is [k_dim x n]
+ *   keys/values[b] = top-k over columns j of act(bias[j] + sum_i X[b][i] * W[i][j]), the scores of the columns listed in row b's
+ * filter multiplied by 0 (filter arguments and semantics as dsx_topk_filtered with filter_mul == NULL: a listed column keeps
+ * its place with a score of 0 and comes back when fewer than k scores lie above 0; filter_index == NULL: no filter).  W is [k_dim x n]
  * row-major.  Only the first few thousand columns are produced as a matrix (library scratch) and scanned; every later column
  * range is compared with the rows' running k-th scores inside the GEMM kernel's registers and only the survivors are kept.
  * Results are exact under the same total order as dsx_topk (score descending, column ascending); a score here and the same
  * score from dsx_fc_forward may differ in the last place (the bias enters the sum first instead of last).  A row whose
- * survivor list fills up (thousands of scores tied at the top) is recomputed on the device, slowly; dsx_fc_topk_flagged tells
+ * survivor list fills up (thousands of scores tied at the top), or whose k-th score is not above 0 while its filter lists columns
+ * beyond the first block, is recomputed on the device, slowly; dsx_fc_topk_flagged tells
  * a caller that this has happened, so that it can go back to dsx_fc_forward + dsx_topk_filtered for such data.
  * Returns DSX_EUNSUPPORTED (dsx_fc_topk_supported() == 0) unless the activation is non-decreasing (sigmoid, tanh, ReLU, leaky
  * ReLU with a positive slope, linear) and X is 16-byte aligned with ldx a multiple of 4. */
@@ -312,12 +312,10 @@ int dsx_fc_topk_split(const float* X, uint32_t ldx, const float* W, const void* 
                       uint32_t* values, uint32_t position, const uint32_t* index, const uint64_t* filter_start, const uint64_t* filter_end,
                       const uint32_t* filter_index);
 int dsx_fc_topk_supported(uint32_t ldx, const float* X, uint32_t activation, const dsx_act_params* params, const float* filter_mul);
-/* 1 if any row of any dsx_fc_topk call so far had to be recomputed (reset != 0 clears the mark). */
+/* 1 if any row of any dsx_fc_topk call so far had to be recomputed (reset != 0 clears the mark); dsx_fc_topk_flagged_for: the
+ * same for the calls with this weight matrix only (the mark is kept per W pointer, for the 64 matrices used last). */
 int dsx_fc_topk_flagged(int reset);
-/* Tuning knobs, used by the tests to reach every path with small inputs: width of the first column block (0: default 2,048) and
- * survivor words per row and column range (0: default 4,096, the maximum). */
-int dsx_fc_topk_set_first_columns(uint32_t columns);
-int dsx_fc_topk_set_candidate_capacity(uint32_t words);
+int dsx_fc_topk_flagged_for(const float* W, int reset);
 
 /* ---- KNN ------------------------------------------------------------------------------------------------------------- */
 /* Device part of KnnExactGpu::search (knn/KnnExactGpu.cu:99-148): scores = queries . items^T (cublasSgemmEx) followed by
@@ -355,21 +353,15 @@ int dsx_knn_search_split(const void* item_planes, uint32_t rows_padded, uint32_t
                          uint32_t num_queries, uint32_t k, float* scores, uint32_t* indexes, void* workspace, size_t workspace_bytes,
                          float* elapsed_ms);
 size_t dsx_knn_workspace_bytes_split(uint32_t rows_padded, uint32_t dim, uint32_t num_queries, uint32_t k);
-/* No counterpart in the reference: width of the first column block (rounded down to a multiple of 1024, at least 1024;
- * 0 restores the default of about 1 GiB of scores).  Workspace sizes depend on it: set it before asking for them. */
-int dsx_knn_set_block_columns(uint32_t columns);
 /* No counterpart in the reference: how the last dsx_knn_search of this process ran. */
 #define DSX_KNN_PATH_BLOCKS 0             /* every column block through the scratch score matrix and the scanning top-K */
 #define DSX_KNN_PATH_CANDIDATES 1         /* first block as above, then candidate lists */
 #define DSX_KNN_PATH_CANDIDATES_REDONE 2  /* a candidate list filled up: repeated block by block */
 int dsx_knn_last_search_path(void);
-/* No counterpart in the reference: how dsx_knn_search_f16 scores the column ranges after the first block.  1 (default): a
- * range with enough item tiles is swept by workgroups that keep their queries and walk a chunk of the range each (private
- * candidate lists, no atomics on device memory) — with the queries held in registers when the vectors have at most 256
- * components, 128 queries per workgroup staged through LDS otherwise; 0: always one workgroup per tile; 2 and 3: the LDS sweep
- * and the register sweep for every range that has at least one tile per chunk (for tests at small sizes).  The results are
- * the same in every mode. */
-int dsx_knn_f16_set_sweep(int mode);
+/* dsx_knn_search_f16 scores the column ranges after the first block one workgroup per tile, or, when a range has enough item
+ * tiles, with workgroups that keep their queries and walk a chunk of the range each (private candidate lists, no atomics on
+ * device memory): the queries in registers when the vectors have at most 256 components, 128 queries per workgroup staged
+ * through LDS otherwise.  The results are the same either way. */
 
 #ifdef __cplusplus
 }

@@ -29,7 +29,7 @@ def orc():
 
 @pytest.fixture(scope="session")
 def synth(pkg):
-    from amazon_dsstne_amd import synth as s
+    from dsx_support import synth as s
     return s
 
 

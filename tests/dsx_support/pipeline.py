@@ -8,7 +8,7 @@ import ctypes as C
 
 import numpy as np
 
-from . import ACT_SOFTMAX, ActParams, DeviceArray, check, load_library, ptr
+from amazon_dsstne_amd import ACT_SOFTMAX, ActParams, DeviceArray, check, load_library, ptr
 
 
 class DevicePipeline:

@@ -12,7 +12,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 import numpy as np
 
-from . import (ACT_RELU, ACT_SIGMOID, ATTR_BOOLEAN, ATTR_INDEXED, ATTR_SPARSE, T_FLOAT)
+from amazon_dsstne_amd import (ACT_RELU, ACT_SIGMOID, ATTR_BOOLEAN, ATTR_INDEXED, ATTR_SPARSE, T_FLOAT)
 
 WEIGHT_STD = 0.1
 

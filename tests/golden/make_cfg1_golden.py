@@ -14,7 +14,7 @@ sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 
 entry.load_package()
-from amazon_dsstne_amd import synth  # noqa: E402
+from dsx_support import synth  # noqa: E402
 
 p = synth.config(1)
 X = np.zeros((p.batch, p.widths[0]), dtype=np.float64)

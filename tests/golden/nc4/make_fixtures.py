@@ -64,12 +64,12 @@ def write_cdf5(path, dims, atts, variables):
 
 
 def small_network():
-    """The network of the `small` fixtures: 256 sparse inputs -> 32 ReLU -> 256 sigmoid, weights from amazon_dsstne_amd/synth.py
+    """The network of the `small` fixtures: 256 sparse inputs -> 32 ReLU -> 256 sigmoid, weights from tests/dsx_support/synth.py
     (seed 4242), so that a test can rebuild the same problem and ask the oracle what the network must predict."""
     sys.path.insert(0, ROOT)
     import __graft_entry__ as entry
     entry.load_package()
-    from amazon_dsstne_amd import synth
+    from dsx_support import synth
     return synth.autoencoder("small-nc4", 4242, 256, [32], 16, 5, 1, 1.0, 12, 0.5, (1, 40), bias_std=0.3)
 
 

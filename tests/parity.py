@@ -79,22 +79,36 @@ def forward_f64(p, rows):
     return np.asarray(out)
 
 
-def assert_units_close(got, ref, p, position=0, what="activations", rel=REL_TOL, abs_floor=1e-3, positions=None):
-    """Layer outputs against the fp32 oracle: within `rel` of it, or — where deep sums cancel and two fp32 summation orders part
-    by more than that — at least as close to the float64 ground truth as the oracle itself is (row by row: the largest deviation
-    from the truth at most twice the oracle's, plus one part in 10^6 of the row's largest value).  Row i of got / ref is batch position `position + i`, or positions[i]."""
+FALLBACK_LOG = []  # one (what, rows compared, rows judged against float64, worst relative error vs the oracle) per call
+
+
+def assert_units_close(got, ref, p, position=0, what="activations", rel=REL_TOL, abs_floor=1e-3, positions=None, max_fallback_rows=0):
+    """Layer outputs against the fp32 oracle: every row within `rel` of it (relative to max(|ref|, abs_floor)).
+
+    `max_fallback_rows` (0 unless the caller states a ceiling) is how many rows may miss that and be judged against the float64
+    ground truth instead: where deep sums cancel, two fp32 summation orders part by more than `rel`, and such a row passes if
+    its largest deviation from the truth is at most twice the oracle's own, plus one part in 10^6 of the row's largest value.
+    Every call prints one `[parity]` line with the number of rows that took this second rule and the worst error against the
+    oracle, and appends the same to FALLBACK_LOG.  Row i of got / ref is batch position `position + i`, or positions[i]."""
     got64, ref64 = np.asarray(got, dtype=np.float64), np.asarray(ref, dtype=np.float64)
     err = np.abs(got64 - ref64) / np.maximum(np.abs(ref64), abs_floor)
+    worst = float(err.max()) if err.size else 0.0
     bad_rows = np.nonzero((err > rel).any(axis=1))[0]
+    FALLBACK_LOG.append((what, int(got64.shape[0]), int(bad_rows.size), worst))
+    print("[parity] %s: %d rows, %d beyond %.0e of the oracle (ceiling %d), worst relative error %.3g" % (
+        what, got64.shape[0], bad_rows.size, rel, max_fallback_rows, worst), flush=True)
     if bad_rows.size == 0:
-        return float(err.max()) if err.size else 0.0
-    assert bad_rows.size <= max(4, got.shape[0] // 20), "%s: %d rows differ from the oracle by more than %.0e" % (what, bad_rows.size, rel)
+        return worst
+    assert bad_rows.size <= max_fallback_rows, "%s: %d rows differ from the oracle by more than %.0e (ceiling %d), worst %.3g" % (
+        what, bad_rows.size, rel, max_fallback_rows, worst)
     truth = forward_f64(p, (position + bad_rows) if positions is None else np.asarray(positions)[bad_rows])
     e_got = np.abs(got64[bad_rows] - truth)
     e_ref = np.abs(ref64[bad_rows] - truth)
     # rounding errors fall on different elements in the two computations: compare their levels row by row
     level_got, level_ref = e_got.max(axis=1), e_ref.max(axis=1)
     worse = level_got > 2.0 * level_ref + 1e-6 * np.abs(truth).max(axis=1) + 1e-9
+    print("[parity] %s: the %d rows against float64: largest deviation %.3g, the oracle's %.3g" % (
+        what, bad_rows.size, float(level_got.max()), float(level_ref.max())), flush=True)
     assert not worse.any(), "%s: %d rows are further from the float64 result than the fp32 oracle is (worst %.3g vs oracle %.3g)" % (
         what, int(worse.sum()), float(level_got.max()), float(level_ref.max()))
-    return float(err.max())
+    return worst

@@ -1,4 +1,5 @@
-"""The C-ABI library loads and exports exactly what include/dsx.h declares (no GPU, no compute calls)."""
+"""The C-ABI library loads and exports exactly what include/dsx.h and include/dsx_testing.h (the tests' switches) declare (no
+GPU, no compute calls)."""
 import ctypes as C
 import os
 import re
@@ -9,7 +10,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def declared_functions():
-    text = open(os.path.join(ROOT, "include", "dsx.h")).read()
+    text = open(os.path.join(ROOT, "include", "dsx.h")).read() + open(os.path.join(ROOT, "include", "dsx_testing.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(dsx_[a-z0-9_]+)\s*\(", text)))
 
@@ -37,7 +38,7 @@ def test_header_compiles_as_c():
     import tempfile
     with tempfile.TemporaryDirectory() as d:
         src = os.path.join(d, "t.c")
-        open(src, "w").write('#include "dsx.h"\nint main(void) { return DSX_OK; }\n')
+        open(src, "w").write('#include "dsx.h"\n#include "dsx_testing.h"\nint main(void) { return DSX_OK; }\n')
         subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), "-c", src, "-o",
                                os.path.join(d, "t.o")])
 

@@ -32,8 +32,8 @@ def knobs(request, dsx):
     dsx.dsx_fc_topk_flagged(1)
     yield dsx
     MODE["split"] = False
-    dsx.dsx_fc_topk_set_first_columns(0)
-    dsx.dsx_fc_topk_set_candidate_capacity(0)
+    dsx.dsx_testing_set_fc_topk_first_columns(0)
+    dsx.dsx_testing_set_fc_topk_candidate_capacity(0)
     dsx.dsx_fc_topk_flagged(1)
 
 
@@ -106,7 +106,7 @@ def test_fc_topk_catalogue_shape(pkg, dsx, orc, rng, knobs, n):
 @pytest.mark.parametrize("k", [1, 33, 100, 256])
 def test_fc_topk_ranges_activations_and_k(pkg, dsx, orc, rng, knobs, act, k):
     # a first block of 256 columns, so that 6,001 columns run several candidate ranges
-    dsx.dsx_fc_topk_set_first_columns(256)
+    dsx.dsx_testing_set_fc_topk_first_columns(256)
     batch, kdim, n = 150, 64, 6001
     say("fc_topk act=%d k=%d" % (act, k))
     X, W, bias = layer(rng, batch, kdim, n)
@@ -143,8 +143,8 @@ def test_fc_topk_ties_and_full_lists_are_recomputed_exactly(pkg, dsx, orc, rng, 
     """Scores tied in their thousands: integer operands give exactly representable sums whatever the order, a ReLU turns half of
     them into the same 0, and a saturated sigmoid into the same 1.  Lists fill up, the rows are recomputed on the device, and
     the result must be the two-call path's bit for bit (score descending, then the lower column)."""
-    dsx.dsx_fc_topk_set_first_columns(256)
-    dsx.dsx_fc_topk_set_candidate_capacity(512)          # a third of row 5's columns tie at the top: more than a list holds
+    dsx.dsx_testing_set_fc_topk_first_columns(256)
+    dsx.dsx_testing_set_fc_topk_candidate_capacity(512)          # a third of row 5's columns tie at the top: more than a list holds
     batch, kdim, n, k = 70, 32, 9000, 50
     X = rng.integers(-2, 3, size=(batch, kdim)).astype(np.float32)
     W = rng.integers(-2, 3, size=(kdim, n)).astype(np.float32)
@@ -157,7 +157,7 @@ def test_fc_topk_ties_and_full_lists_are_recomputed_exactly(pkg, dsx, orc, rng, 
         assert np.array_equal(gi, ti) and np.array_equal(gk.view(np.uint32), tk.view(np.uint32))
     assert dsx.dsx_fc_topk_flagged(1) == 1               # row 5 at least filled its list
     # saturated sigmoids: 1.0f in every column, more than even a full-size list holds
-    dsx.dsx_fc_topk_set_candidate_capacity(0)
+    dsx.dsx_testing_set_fc_topk_candidate_capacity(0)
     Xs = np.abs(X) + 1.0
     Ws = np.abs(W) * 3.0 + 1.0
     gk, gi, _, tk, ti = run_both(pkg, dsx, orc, Xs.astype(np.float32), Ws.astype(np.float32), bias, ACT_SIGMOID, k, 0, None, start, end, fidx,
@@ -166,10 +166,32 @@ def test_fc_topk_ties_and_full_lists_are_recomputed_exactly(pkg, dsx, orc, rng, 
     assert dsx.dsx_fc_topk_flagged(1) == 1
 
 
+@pytest.mark.parametrize("act", [ACT_RELU, ACT_LINEAR, ACT_TANH, ACT_LRELU])
+def test_fc_topk_listed_columns_score_zero_not_nothing(pkg, dsx, orc, rng, knobs, act):
+    """utils/Filters.cpp:62 multiplies a listed column's score by 0 and kCalculateTopK then sees that zero: in a row with fewer
+    than k scores above 0 the listed columns come back, lower column first.  Most scores here are negative (or a ReLU's 0), every
+    row has listed columns on both sides of the first block, and the fused call must give the two-call path's result bit for bit."""
+    dsx.dsx_testing_set_fc_topk_first_columns(256)
+    batch, kdim, n, k = 48, 32, 5000, 40
+    X = rng.integers(1, 3, size=(batch, kdim)).astype(np.float32)
+    W = -rng.integers(0, 3, size=(kdim, n)).astype(np.float32)           # exact sums whatever the order
+    bias = np.zeros(n, dtype=np.float32)
+    W[:, rng.choice(n, 12, replace=False)] *= -1.0                        # a dozen columns score above 0: fewer than k
+    start, end, fidx = random_csr(rng, batch, n, 120, empty_rows=(3,))
+    say("fc_topk listed zeros act=%d" % act)
+    dsx.dsx_fc_topk_flagged(1)
+    gk, gi, unit, tk, ti = run_both(pkg, dsx, orc, X, W, bias, act, k, 0, None, start, end, fidx, "listed zeros act=%d" % act)
+    assert np.array_equal(gi, ti) and np.array_equal(gk.view(np.uint32), tk.view(np.uint32))
+    listed_back = sum(len(set(gi[b].tolist()) & set(fidx[int(start[b]):int(end[b])].tolist())) for b in range(batch))
+    assert listed_back > 0, "the case does not reach a listed column"
+    rk, ri = orc.topk_filtered(unit, k, 0, None, start, end, fidx, None)
+    assert np.array_equal(gi, ri) and np.array_equal(gk, rk)              # (-0.0 == 0.0: the oracle keeps the product's sign)
+
+
 def test_fc_topk_tiny_lists_overflow_on_ordinary_data(pkg, dsx, orc, rng, knobs):
     # 64 words per row and range: ordinary rows overflow, most rows are recomputed; results still under the parity rules
-    dsx.dsx_fc_topk_set_first_columns(128)
-    dsx.dsx_fc_topk_set_candidate_capacity(64)
+    dsx.dsx_testing_set_fc_topk_first_columns(128)
+    dsx.dsx_testing_set_fc_topk_candidate_capacity(64)
     batch, kdim, n, k = 90, 128, 8000, 30
     X, W, bias = layer(rng, batch, kdim, n)
     start, end, fidx = random_csr(rng, batch, n, 500)

@@ -77,8 +77,8 @@ def check_batch_properties(p, keys, idx, filtered_rows=True):
             assert not np.isin(idx[b], own).any(), "row %d: an item of the sample's own input came back" % b
 
 
-def run_network_config(pkg, dsx, orc, p, guided):
-    from amazon_dsstne_amd.pipeline import DevicePipeline
+def run_network_config(pkg, dsx, orc, p, guided, fallback_rows=0):
+    from dsx_support.pipeline import DevicePipeline
     B, N, k = p.batch, p.widths[-1], p.k
     pipe = DevicePipeline(p, dsx, guided=guided)
     pipe.step()
@@ -89,7 +89,8 @@ def run_network_config(pkg, dsx, orc, p, guided):
     check_batch_properties(p, keys, idx)
     ref_unit, ref_scores, ref_keys, ref_idx = oracle_rows(orc, p, picks, k)
     unit = download_rows(pkg, dsx, pipe.units[-1], N, picks)
-    assert_units_close(unit, ref_unit, p, what="%s output activations of the sampled rows" % p.name, positions=picks)
+    assert_units_close(unit, ref_unit, p, what="%s output activations of the sampled rows" % p.name, positions=picks,
+                       max_fallback_rows=fallback_rows)
     assert np.array_equal(unit[np.arange(len(picks))[:, None], idx[picks]], keys[picks]), "score is not the activation at the reported index"
     n = assert_topk_parity(keys[picks], idx[picks], ref_keys, ref_idx, ref_scores, p.name)
     say("%s: sampled rows agree with the oracle (%d tie-equivalent index differences)" % (p.name, n))
@@ -98,8 +99,10 @@ def run_network_config(pkg, dsx, orc, p, guided):
 
 def test_cfg3_full_size(pkg, dsx, orc, synth):
     p = synth.config(3)
-    _, k_scan, i_scan = run_network_config(pkg, dsx, orc, p, guided=False)
-    _, k_gd, i_gd = run_network_config(pkg, dsx, orc, p, guided=True)
+    # Of the 19 sampled rows one holds an output that differs from the fp32 oracle's by 2.2e-4 (a small sigmoid behind sums over
+    # 1,024 ReLU units: the two summation orders part); it is judged against float64.  Configurations 1, 2 and 4 have no such row.
+    _, k_scan, i_scan = run_network_config(pkg, dsx, orc, p, guided=False, fallback_rows=1)
+    _, k_gd, i_gd = run_network_config(pkg, dsx, orc, p, guided=True, fallback_rows=1)
     assert np.array_equal(i_gd, i_scan) and np.array_equal(k_gd.view(np.uint32), k_scan.view(np.uint32)), "guided and scanning top-K differ"
 
 

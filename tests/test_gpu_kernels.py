@@ -624,9 +624,9 @@ def knn_case(pkg, dsx, orc, items_m, queries_m, k, pad_value=50.0):
 def small_knn_blocks(dsx):
     """First column block of 1,024 items, so that searches of a few ten thousand items run the candidate ranges
     (1,024 scanned, then 4,096, 20,480, ... compared with the queries' bounds)."""
-    dsx.dsx_knn_set_block_columns(1024)
+    dsx.dsx_testing_set_knn_block_columns(1024)
     yield
-    dsx.dsx_knn_set_block_columns(0)
+    dsx.dsx_testing_set_knn_block_columns(0)
 
 
 @pytest.mark.parametrize("items,queries,dim,k", [(30011, 70, 64, 100), (9000, 130, 256, 10), (26000, 33, 32, 200), (1500, 5, 16, 64)])
@@ -692,12 +692,12 @@ def test_knn_search_nan_scores_never_returned_on_either_path(pkg, dsx, orc, synt
     p = synth.knn_config(seed=11, items=20000, queries=24, dim=32, k=50)
     bad = np.arange(7, 20000, 13)
     p.items[bad, 5] = np.nan
-    dsx.dsx_knn_set_block_columns(1024)
+    dsx.dsx_testing_set_knn_block_columns(1024)
     try:
         cs, ci, _, _, _ = knn_case(pkg, dsx, orc, p.items, p.queries, 50)
         assert dsx.dsx_knn_last_search_path() == 1
     finally:
-        dsx.dsx_knn_set_block_columns(0)
+        dsx.dsx_testing_set_knn_block_columns(0)
     bs, bi, _, _, _ = knn_case(pkg, dsx, orc, p.items, p.queries, 50)
     assert dsx.dsx_knn_last_search_path() == 0
     assert np.array_equal(ci, bi) and np.array_equal(cs.view(np.uint32), bs.view(np.uint32))
@@ -767,14 +767,14 @@ def knn_case_f16(pkg, dsx, orc, items_m, queries_m, k):
 def test_knn_search_f16(pkg, dsx, orc, synth, items, queries, dim, k, blocks, sweep):
     say("knn fp16 items=%d queries=%d dim=%d k=%d first block=%d sweep=%d" % (items, queries, dim, k, blocks, sweep))
     p = synth.knn_config(seed=21, items=items, queries=queries, dim=dim, k=k)
-    dsx.dsx_knn_set_block_columns(blocks)
-    pkg.check(dsx.dsx_knn_f16_set_sweep(sweep))
+    dsx.dsx_testing_set_knn_block_columns(blocks)
+    pkg.check(dsx.dsx_testing_set_knn_f16_sweep(sweep))
     try:
         got_s, got_i, ref_s, ref_i, it16, q16, _ = knn_case_f16(pkg, dsx, orc, p.items, p.queries, k)
         assert dsx.dsx_knn_last_search_path() == (1 if blocks else 0)
     finally:
-        dsx.dsx_knn_set_block_columns(0)
-        pkg.check(dsx.dsx_knn_f16_set_sweep(1))
+        dsx.dsx_testing_set_knn_block_columns(0)
+        pkg.check(dsx.dsx_testing_set_knn_f16_sweep(1))
     full = q16.astype(np.float64) @ it16.astype(np.float64).T
     assert got_i.max() < items
     mism = got_i != ref_i
@@ -796,14 +796,14 @@ def test_knn_search_f16_sweep_spills_clustered_items(pkg, dsx, orc, rng, dim, sw
     u = q[5] / np.linalg.norm(q[5])
     for j in range(300):
         it[21000 + j] = u * (40.0 + 0.25 * j)   # far above anything else for query 5, all different
-    dsx.dsx_knn_set_block_columns(1024)
-    pkg.check(dsx.dsx_knn_f16_set_sweep(sweep))
+    dsx.dsx_testing_set_knn_block_columns(1024)
+    pkg.check(dsx.dsx_testing_set_knn_f16_sweep(sweep))
     try:
         got_s, got_i, ref_s, ref_i, it16, q16, _ = knn_case_f16(pkg, dsx, orc, it, q, k)
         assert dsx.dsx_knn_last_search_path() == 1
     finally:
-        dsx.dsx_knn_set_block_columns(0)
-        pkg.check(dsx.dsx_knn_f16_set_sweep(1))
+        dsx.dsx_testing_set_knn_block_columns(0)
+        pkg.check(dsx.dsx_testing_set_knn_f16_sweep(1))
     assert set(got_i[5]) <= set(range(21000, 21300))
     full = q16.astype(np.float64) @ it16.astype(np.float64).T
     mism = got_i != ref_i
@@ -837,8 +837,8 @@ def test_knn_search_f16_exact_ties_and_full_lists(pkg, dsx, orc, rng, sweep, dim
     items, queries, k = 21000, 40, 100
     it = rng.integers(-2, 3, size=(items, dim)).astype(np.float32)
     q = rng.integers(-2, 3, size=(queries, dim)).astype(np.float32)
-    dsx.dsx_knn_set_block_columns(1024)
-    pkg.check(dsx.dsx_knn_f16_set_sweep(sweep))
+    dsx.dsx_testing_set_knn_block_columns(1024)
+    pkg.check(dsx.dsx_testing_set_knn_f16_sweep(sweep))
     try:
         got_s, got_i, ref_s, ref_i, _, _, _ = knn_case_f16(pkg, dsx, orc, it, q, k)
         assert dsx.dsx_knn_last_search_path() == 1
@@ -848,5 +848,5 @@ def test_knn_search_f16_exact_ties_and_full_lists(pkg, dsx, orc, rng, sweep, dim
         assert dsx.dsx_knn_last_search_path() == 2
         assert np.array_equal(got_s, ref_s) and np.array_equal(got_i, ref_i)
     finally:
-        dsx.dsx_knn_set_block_columns(0)
-        pkg.check(dsx.dsx_knn_f16_set_sweep(1))
+        dsx.dsx_testing_set_knn_block_columns(0)
+        pkg.check(dsx.dsx_testing_set_knn_f16_sweep(1))

@@ -82,14 +82,14 @@ SHAPES = [(300, 100, 1000), (130, 17, 257), (1, 128, 129), (257, 130, 128), (64,
 @pytest.fixture(params=[128, 256])
 def tile_rows(request, pkg, dsx):
     """Both tile heights of the kernel on every shape (by itself it takes 256 rows only for long sums over many tiles)."""
-    pkg.check(dsx.dsx_fc_split_set_tile_rows(request.param))
+    pkg.check(dsx.dsx_testing_set_split_tile_rows(request.param))
     yield request.param
-    pkg.check(dsx.dsx_fc_split_set_tile_rows(0))
+    pkg.check(dsx.dsx_testing_set_split_tile_rows(0))
 
 
 def test_fc_split_tile_rows_argument(pkg, dsx):
-    assert dsx.dsx_fc_split_set_tile_rows(64) != 0
-    pkg.check(dsx.dsx_fc_split_set_tile_rows(0))
+    assert dsx.dsx_testing_set_split_tile_rows(64) != 0
+    pkg.check(dsx.dsx_testing_set_split_tile_rows(0))
 
 
 @pytest.mark.parametrize("B,k,n", SHAPES)
@@ -181,7 +181,7 @@ def test_fc_split_segment_maxima_and_arguments(pkg, dsx, rng, tile_rows):
 def test_cfg2_with_split_products_matches_the_oracle(pkg, dsx, orc, synth):
     """Config 2 end to end with the output layer in this mode, scanning and guided top-K: activations within 1e-4 of the oracle's,
     indexes the oracle's except where its scores are closer than 1e-5."""
-    from amazon_dsstne_amd.pipeline import DevicePipeline
+    from dsx_support.pipeline import DevicePipeline
     p = synth.config(2)
     _, ref_unit, _, _ = orc.forward(p, 0, None, filtered=False, want_unit=True, want_topk=False)
     _, _, ref_keys, ref_idx = orc.forward(p, 0, None, filtered=True)
@@ -290,12 +290,12 @@ def test_knn_search_split(pkg, dsx, orc, synth, items, queries, dim, k, blocks):
     p = synth.knn_config(seed=11, items=items, queries=queries, dim=dim, k=k)
     cm, rows, pad = p.column_major_padded()
     cm[:, rows - pad:] = 50.0     # pad rows must never be returned (knn/KnnData.cpp:336-340 leaves them uninitialised)
-    dsx.dsx_knn_set_block_columns(blocks)
+    dsx.dsx_testing_set_knn_block_columns(blocks)
     try:
         got_s, got_i, el = knn_split_search(pkg, dsx, cm, rows, pad, dim, p.queries, k)
         path = dsx.dsx_knn_last_search_path()
     finally:
-        dsx.dsx_knn_set_block_columns(0)
+        dsx.dsx_testing_set_knn_block_columns(0)
     assert path == (1 if blocks else 0), path          # DSX_KNN_PATH_CANDIDATES where there are ranges after the first block
     ref_s, ref_i = orc.knn_search(cm, rows, pad, dim, p.queries, k)
     full = p.queries.astype(np.float64) @ p.items.astype(np.float64).T

@@ -24,6 +24,18 @@ def test_cpp_host_unit_tests(tmp_path):
     assert "0 failed" in r.stdout
 
 
+def test_cpp_host_unit_tests_under_the_sanitizers(tmp_path):
+    """The same program with the whole host layer compiled with -fsanitize=address,undefined (tests/cpp: make asan)."""
+    exe = EXE + "_asan"
+    if not os.path.exists(exe):
+        pytest.fail("%s is missing: run __graft_entry__.build()" % exe)
+    env = dict(os.environ, ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=0", UBSAN_OPTIONS="halt_on_error=1")
+    r = subprocess.run([exe, str(tmp_path), os.path.join(ROOT, "tests", "golden", "ldl")], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True,
+                       timeout=600, env=env)
+    assert r.returncode == 0, r.stdout[-4000:]
+    assert "0 failed" in r.stdout and "runtime error" not in r.stdout and "AddressSanitizer" not in r.stdout
+
+
 def test_network_reader_against_scipy_writer(tmp_path):
     """A network file written by an independent NetCDF implementation (classic CDF-2, signed attribute types) with the
     reference's attribute and variable names (engine/NNNetwork.cpp:1933-1971, NNLayer.cpp:3447-3500, NNWeight.cpp:853-900)."""

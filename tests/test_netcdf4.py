@@ -15,6 +15,8 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 NC4 = os.path.join(ROOT, "tests", "golden", "nc4")
 DUMP = os.path.join(ROOT, "tests", "cpp", "nc_dump")
+DUMP_ASAN = os.path.join(ROOT, "tests", "cpp", "nc_dump_asan")   # the readers built with -fsanitize=address,undefined (make asan)
+ASAN_ENV = dict(os.environ, ASAN_OPTIONS="verify_asan_link_order=0:detect_leaks=0:abort_on_error=0", UBSAN_OPTIONS="halt_on_error=1")
 HOST = os.path.join(ROOT, "tests", "cpp", "test_host_cpu")
 FIXTURES = sorted(f for f in glob.glob(os.path.join(NC4, "*.nc")) if not f.endswith(".classic.nc"))
 
@@ -114,3 +116,62 @@ def test_damaged_files_are_refused_not_crashed_on(tmp_path):
             p.write_bytes(blob)
             r = subprocess.run([DUMP, str(p)], stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=60)
             assert r.returncode in (0, 1), "%s case %d: exit %d %s" % (name, i, r.returncode, r.stderr[-300:])
+
+
+def run_asan(args, timeout=300):
+    assert os.path.exists(DUMP_ASAN), "tests/cpp/nc_dump_asan is missing: run __graft_entry__.build()"
+    return subprocess.run([DUMP_ASAN] + args, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=timeout, env=ASAN_ENV)
+
+
+@pytest.mark.parametrize("fixture", FIXTURES, ids=[os.path.basename(f) for f in FIXTURES])
+def test_fixtures_read_cleanly_under_the_sanitizers(fixture):
+    r = run_asan([fixture])
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert "runtime error" not in r.stderr and "AddressSanitizer" not in r.stderr
+    assert r.stdout == dump(fixture)[0]
+
+
+def test_single_byte_damage_under_the_sanitizers(tmp_path):
+    """Every byte of the first 1,500 of four fixtures (superblock, root header, the first heaps and indexes) set to four other
+    values, one at a time, read by the sanitizer build in one process per fixture: a read or write outside a buffer, a signed
+    overflow or a misaligned access ends that process with a report; damage that is merely wrong data or a refused file does not."""
+    procs = []
+    for name in ("net.earliest.nc", "tied.v18.nc", "tied.plain.nc", "big.earliest.c7.nc"):
+        assert os.path.exists(DUMP_ASAN), "tests/cpp/nc_dump_asan is missing: run __graft_entry__.build()"
+        procs.append((name, subprocess.Popen([DUMP_ASAN, "--sweep", os.path.join(NC4, name), "0", "1500", str(tmp_path / (name + ".tmp"))],
+                                             stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, env=ASAN_ENV)))
+    for name, p in procs:
+        out, err = p.communicate(timeout=600)
+        assert p.returncode == 0, "%s: exit %d\n%s" % (name, p.returncode, err[-3000:])
+        assert "copies still read" in out and "runtime error" not in err
+
+
+def patched(data, at, value_le16):
+    b = bytearray(data)
+    b[at:at + 2] = int(value_le16).to_bytes(2, "little")
+    return bytes(b)
+
+
+def test_attribute_sizes_beyond_the_message_are_refused(tmp_path):
+    """An attribute message whose datatype or dataspace size field points past the end of the message (the cursor used to be
+    moved there unchecked and the value copied from outside the block).  Version 1 messages (old-style file): version, reserved,
+    name size, datatype size, dataspace size (2 bytes each), name; version 3 (new-style): ... one byte of character set, name."""
+    cases = []
+    old = open(os.path.join(NC4, "tied.plain.nc"), "rb").read()
+    name = b"version\x00"
+    pos = old.index(name)
+    assert old[pos - 8] == 1 and int.from_bytes(old[pos - 6:pos - 4], "little") == len(name)      # a version 1 attribute message
+    for field in (pos - 4, pos - 2):
+        for value in (0xFFF8, 0x7FF0, 0x0400):
+            cases.append(patched(old, field, value))
+    new = open(os.path.join(NC4, "net.v18.nc"), "rb").read()
+    pos = new.index(name)
+    assert new[pos - 9] == 3 and int.from_bytes(new[pos - 7:pos - 5], "little") == len(name)       # a version 3 attribute message
+    for field in (pos - 5, pos - 3):
+        for value in (0xFFFF, 0x7FF0, 0x0400):
+            cases.append(patched(new, field, value))
+    for i, blob in enumerate(cases):
+        p = tmp_path / ("attr_%d.nc" % i)
+        p.write_bytes(blob)
+        r = run_asan([str(p)])
+        assert r.returncode == 1 and r.stdout.startswith("error:"), (i, r.returncode, r.stdout[:300], r.stderr[-1500:])
