@@ -100,6 +100,7 @@ SIGNATURES = {
     "dsx_fc_topk_flagged": [_int],
     "dsx_fc_topk_flagged_for": [_vp, _int],
     "dsx_testing_reset": [],
+    "dsx_testing_occupy": [_u32, _u32, _u32],
     "dsx_testing_set_fc_topk_first_columns": [_u32],
     "dsx_testing_set_fc_topk_candidate_capacity": [_u32],
     "dsx_knn_search": [_vp, _u32, _u32, _u32, _vp, _u32, _u32, _vp, _vp, _vp, _sz, C.POINTER(_f32)],

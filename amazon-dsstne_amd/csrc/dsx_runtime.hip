@@ -214,6 +214,16 @@ static void lanes_release()
     g_lane = 0;
 }
 
+// Holds a workgroup's place (registers, a slot of every SIMD) without issuing vector or memory instructions.
+template <int REGS>
+__global__ __launch_bounds__(256) void occupy_kernel(uint32_t cycles)
+{
+    if (REGS == 128) asm volatile("v_mov_b32 v127, 0" ::: "v127");   // the highest register named fixes the allocation
+    if (REGS == 64) asm volatile("v_mov_b32 v63, 0" ::: "v63");
+    const uint64_t t0 = __builtin_readcyclecounter();
+    for (uint32_t spins = 0; spins < 100000 && __builtin_readcyclecounter() - t0 < cycles; spins++) __builtin_amdgcn_s_sleep(8);
+}
+
 extern "C" {
 
 const char* dsx_last_error(void) { return g_error; }
@@ -278,6 +288,18 @@ int dsx_shutdown(void)
     hipEventDestroy(c.ev_stop);
     hipStreamDestroy(c.stream);
     c = Context();
+    return DSX_OK;
+}
+
+int dsx_testing_occupy(uint32_t workgroups, uint32_t cycles, uint32_t vgprs)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(workgroups >= 1 && workgroups <= 65536 && cycles <= 10000000u, "dsx_testing_occupy: %u workgroups, %u cycles", workgroups, cycles);
+    hipStream_t s = ctx().stream;
+    if (vgprs == 128) hipLaunchKernelGGL((occupy_kernel<128>), dim3(workgroups), dim3(256), 0, s, cycles);
+    else if (vgprs == 64) hipLaunchKernelGGL((occupy_kernel<64>), dim3(workgroups), dim3(256), 0, s, cycles);
+    else hipLaunchKernelGGL((occupy_kernel<0>), dim3(workgroups), dim3(256), 0, s, cycles);
+    DSX_LAUNCH_CHECK("occupy_kernel");
     return DSX_OK;
 }
 

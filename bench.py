@@ -103,6 +103,74 @@ def timed_windows(step, sync, steps, windows):
     return out
 
 
+def interference_block(pkg, lib, p, steps):
+    """What each kernel of a batch costs the output layer's GEMM when it runs beside it: the GEMMs back to back on lane 0, the
+    other kernel back to back on lane 1, nothing ordering the two (no step can do better than that with these kernels), and the
+    same with a probe that only holds its workgroups' places (dsx_testing_occupy).  Microseconds per GEMM."""
+    from dsx_support.pipeline import DevicePipeline
+    ptr = pkg.ptr
+    pipes = [DevicePipeline(p, lib, guided=True) for _ in range(2)]
+    for q in pipes:
+        q.step()
+    pkg.check(lib.dsx_sync())
+    B, last = p.batch, len(p.weights) - 1
+
+    def gemm(q):
+        kk, n = p.widths[last], p.widths[last + 1]
+        pkg.check(lib.dsx_fc_forward_segmax(ptr(q.units[last - 1]), kk, ptr(q.W[last]), 0, ptr(q.b[last]), ptr(q.units[last]), n, B, kk, n,
+                                            p.acts[last], C.byref(q.params), ptr(q.seg_max), C.byref(q.seg_width)))
+
+    def sparse(q):
+        pkg.check(lib.dsx_sparse_layer_forward(p.attributes, p.data_type, 0, B, p.widths[1], ptr(q.W[0]), ptr(q.index), ptr(q.start), ptr(q.end),
+                                               ptr(q.sidx), ptr(q.dw), ptr(q.sdata), ptr(q.b[0]), p.acts[0], C.byref(q.params), ptr(q.units[0])))
+
+    def hidden(q):
+        for l in range(1, last):
+            kk, n = p.widths[l], p.widths[l + 1]
+            pkg.check(lib.dsx_fc_forward(ptr(q.units[l - 1]), kk, ptr(q.W[l]), 0, ptr(q.b[l]), ptr(q.units[l]), n, B, kk, n, 0, p.acts[l],
+                                         C.byref(q.params)))
+
+    def us(step):
+        def run(i):
+            step(i)
+        settle(pkg, lib, lambda: run(0))
+        w = timed_windows(run, lambda: pkg.check(lib.dsx_sync()), steps, 3)
+        pkg.check(lib.dsx_set_lane(0))
+        return round(float(np.median(w)) * 1e3, 2)
+
+    def beside(other):
+        def step(i):
+            pkg.check(lib.dsx_set_lane(0))
+            gemm(pipes[0])
+            pkg.check(lib.dsx_set_lane(1))
+            other(pipes[1])
+        return step
+
+    def two_lanes(i):
+        pkg.check(lib.dsx_set_lane(i % 2))
+        gemm(pipes[i % 2])
+
+    def everything(q):
+        q.topk()
+        sparse(q)
+        hidden(q)
+    out = {"unit": "us per output-layer GEMM",
+           "gemm_alone": us(lambda i: gemm(pipes[0])),
+           "gemm_two_lanes": us(two_lanes),
+           "beside_sparse_layer": us(beside(sparse)),
+           "beside_hidden_layers": us(beside(hidden)),
+           "beside_guided_topk": us(beside(lambda q: q.topk())),
+           "beside_all_of_them": us(beside(everything)),
+           "beside_probe": {}}
+    for wgs, cycles, regs in ((1024, 20000, 128), (1024, 20000, 64), (1024, 20000, 0), (2048, 20000, 64), (256, 80000, 64), (256, 80000, 128),
+                              (1024, 10, 0)):
+        out["beside_probe"]["%d workgroups x %d cycles, %d registers" % (wgs, cycles, regs)] = us(
+            beside(lambda q, wgs=wgs, cycles=cycles, regs=regs: pkg.check(lib.dsx_testing_occupy(wgs, cycles, regs))))
+    out["note"] = ("lane 0: the GEMMs back to back; lane 1: the named kernel(s) back to back, unordered against lane 0.  The probe issues no "
+                   "vector or memory instruction: what it costs is the place its workgroups take (20,000 cycles are about 8 us)")
+    return out
+
+
 def network_bench(args, pkg, lib):
     from amazon_dsstne_amd import ATTR_BOOLEAN, ATTR_INDEXED
     from dsx_support import synth
@@ -352,6 +420,11 @@ def network_bench(args, pkg, lib):
         cpu = {"value": round(rows * nb / secs, 1), "unit": "samples/s", "cores": cores, "kind": "port",
                "sample": "%d passes over the first %d rows of one batch of %d of the same workload (%s), %.1f s" % (nb, rows, B, p.name, secs)}
 
+    interference = None
+    if args.interference and gp.seg_width.value and not deferred:
+        del pipe, gp
+        interference = interference_block(pkg, lib, p, max(50, min(300, args.steps)))
+
     def rate(ms):
         return round(B / (ms / 1e3), 1)
     out = {
@@ -393,6 +466,8 @@ def network_bench(args, pkg, lib):
         "request_round_trip": {"ms": round(ms_request, 5), "value": rate(ms_request), "unit": "samples/s",
                                "note": "median over requests served one at a time: upload, predict, filtered top-K, results read back"},
     }
+    if interference:
+        out["interference"] = interference
     return out
 
 
@@ -492,6 +567,7 @@ def main():
     ap.add_argument("--lanes", type=int, default=2, help="NNNetwork::SetLanes for the timed step: batches in flight (1..4, the library's default is 2)")
     ap.add_argument("--knn-items", type=int, default=2000000)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget; 0 skips it")
+    ap.add_argument("--interference", action="store_true", help="also measure what each kernel of a batch costs the output GEMM beside it")
     ap.add_argument("--calibrate-copy", type=int, default=0, help="also run a plain d2d copy of this many MiB (counter calibration)")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -22,6 +22,11 @@ int dsx_testing_set_knn_block_columns(uint32_t columns);
  * range is long enough; 0: always one workgroup per tile; 2 and 3: the LDS sweep and the register sweep for every range that
  * has at least one tile per chunk. */
 int dsx_testing_set_knn_f16_sweep(int mode);
+/* Occupancy probe: launches `workgroups` workgroups of 256 lanes on the selected lane that do nothing but hold their place for
+ * about `cycles` shader clocks (bounded; every wavefront exits), with 128, 64 or (any other value) next to no vector
+ * registers per lane.  bench.py --interference uses it to separate what a kernel beside a dense layer costs that layer by
+ * merely being resident from what its instructions and memory traffic cost. */
+int dsx_testing_occupy(uint32_t workgroups, uint32_t cycles, uint32_t vgprs);
 /* Every switch back to its default. */
 int dsx_testing_reset(void);
 
