@@ -108,7 +108,8 @@ constexpr int kUploadSlots = 8;
 constexpr size_t kUploadSlotBytes = (size_t)4 << 20;
 static char* g_upload_host[kUploadSlots] = {};
 static hipEvent_t g_upload_done[kUploadSlots][DSX_MAX_LANES] = {};   // [slot][lane]: after the slot's last copy on that lane
-static bool g_upload_busy[kUploadSlots][DSX_MAX_LANES] = {};
+static bool g_upload_busy[kUploadSlots][DSX_MAX_LANES] = {};    // an event has been recorded and not yet waited for
+static bool g_upload_dirty[kUploadSlots][DSX_MAX_LANES] = {};   // copies queued since the slot was opened, no event recorded yet
 static int g_upload_slot = 0;       // slot being filled
 static size_t g_upload_fill = 0;    // bytes of it handed out
 
@@ -135,6 +136,7 @@ static void upload_ring_release()
             if (g_upload_done[i][l]) hipEventDestroy(g_upload_done[i][l]);
             g_upload_done[i][l] = nullptr;
             g_upload_busy[i][l] = false;
+            g_upload_dirty[i][l] = false;
         }
     }
     g_upload_slot = 0;
@@ -463,6 +465,14 @@ static int upload_on_selected_lane(void* dst, const void* src, size_t bytes)
     }
     std::lock_guard<std::mutex> lock(g_alloc_mutex);
     if (g_upload_fill + bytes > kUploadSlotBytes) {   // on to the next slot, once nothing is being copied out of it any more
+        // The slot that is full: one event per lane that copied out of it, recorded now — behind its last copy on that lane's
+        // in-order stream, if later than strictly needed — instead of one behind every upload.
+        for (int l = 0; l < DSX_MAX_LANES; l++)
+            if (g_upload_dirty[g_upload_slot][l]) {
+                DSX_HIP(hipEventRecord(g_upload_done[g_upload_slot][l], g_lane_stream[l] ? g_lane_stream[l] : ctx().stream));
+                g_upload_dirty[g_upload_slot][l] = false;
+                g_upload_busy[g_upload_slot][l] = true;
+            }
         g_upload_slot = (g_upload_slot + 1) % kUploadSlots;
         g_upload_fill = 0;
         for (int l = 0; l < DSX_MAX_LANES; l++)
@@ -480,8 +490,7 @@ static int upload_on_selected_lane(void* dst, const void* src, size_t bytes)
     g_upload_fill += (bytes + 255) / 256 * 256;
     memcpy(staged, src, bytes);
     DSX_HIP(hipMemcpyAsync(dst, staged, bytes, hipMemcpyHostToDevice, ctx().stream));
-    DSX_HIP(hipEventRecord(g_upload_done[slot][g_lane], ctx().stream));
-    g_upload_busy[slot][g_lane] = true;
+    g_upload_dirty[slot][g_lane] = true;
     return DSX_OK;
 }
 

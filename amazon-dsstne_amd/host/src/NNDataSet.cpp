@@ -5,6 +5,7 @@
 #include <sstream>
 #include <stdexcept>
 
+#include <cstring>
 #include "NcClassic.h"
 #include "amazon/dsstne/engine/NNTypes.h"
 
@@ -201,10 +202,10 @@ void NNDataSet<T>::CopySparseData(const uint64_t* srcSparseStart, const uint64_t
     checkSparseLoad(srcSparseStart[0], srcSparseEnd[_uniqueExamples - 1]);
     const uint64_t dataLength = srcSparseEnd[_uniqueExamples - 1];
     const T* src = static_cast<const T*>(srcSparseData);
-    copy(srcSparseStart, srcSparseStart + _uniqueExamples, _vSparseStart.data());
-    copy(srcSparseEnd, srcSparseEnd + _uniqueExamples, _vSparseEnd.data());
-    copy(src, src + dataLength, _vSparseData.data());
-    copy(srcSparseIndex, srcSparseIndex + dataLength, _vSparseIndex.data());
+    memcpy(_vSparseStart.data(), srcSparseStart, _uniqueExamples * sizeof(uint64_t));
+    memcpy(_vSparseEnd.data(), srcSparseEnd, _uniqueExamples * sizeof(uint64_t));
+    if (src) memcpy(_vSparseData.data(), src, dataLength * sizeof(T));   // (no values: a Boolean set, whose kernels never read them)
+    memcpy(_vSparseIndex.data(), srcSparseIndex, dataLength * sizeof(uint32_t));
 }
 
 template <typename T>
@@ -213,6 +214,7 @@ void NNDataSet<T>::LoadSparseData(const uint64_t* srcSparseStart, const uint64_t
 {
     if (!(_attributes & NNDataSetEnums::Attributes::Sparse)) throw std::runtime_error("Cannot set sparse data on a non sparse NNDataSet");
     checkSparseLoad(srcSparseStart[0], srcSparseEnd[_uniqueExamples - 1]);
+    if (!srcSparseData && !(_attributes & NNDataSetEnums::Attributes::Boolean)) throw std::runtime_error("NNDataSet::LoadSparseData: no values for a data set that is not Boolean");
     // The device copies are queued first, straight from the caller's arrays and only as long as this batch's data (the
     // buffers may be larger): the device starts on them while the host shadows below are still being filled.  They go to the
     // set of device arrays that the kernels in flight do not read, on the lane the next PredictBatch will use, and are
@@ -281,7 +283,7 @@ void NNDataSet<T>::CopySparseData(const long* srcSparseStart, const long* srcSpa
         _vSparseEnd[i] = (uint64_t)srcSparseEnd[i];
     }
     for (uint64_t i = 0; i < dataLength; ++i) {
-        _vSparseData[i] = src[i];
+        if (src) _vSparseData[i] = src[i];
         _vSparseIndex[i] = (uint32_t)srcSparseIndex[i];
     }
 }

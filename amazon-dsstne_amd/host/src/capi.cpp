@@ -1,4 +1,5 @@
 // capi.cpp — C ABI over the C++ inference classes (include/dsstne_capi.h).
+#include <cstring>
 #include <cstdarg>
 #include <stdexcept>
 
@@ -57,8 +58,10 @@ static void makeResultBuffers(dsstne_context* c)
     vector<const NNLayer*> outs;
     for (auto it = c->network->GetLayers(NNLayer::Kind::Output, outs); it != outs.end(); ++it) {
         for (int lane = 0; lane < DSX_MAX_LANES; lane++) {
-            c->scores[lane][(*it)->GetName()] = new GpuBuffer<NNFloat>((size_t)c->maxK * c->batch);
-            c->indexes[lane][(*it)->GetName()] = new GpuBuffer<uint32_t>((size_t)c->maxK * c->batch);
+            // (pinned host memory that the device writes straight into: a batch's results are batch x k pairs, and reading them
+            // back is then a wait for the lane and a host copy, no transfer of its own)
+            c->scores[lane][(*it)->GetName()] = new GpuBuffer<NNFloat>((size_t)c->maxK * c->batch, false, true);
+            c->indexes[lane][(*it)->GetName()] = new GpuBuffer<uint32_t>((size_t)c->maxK * c->batch, false, true);
         }
     }
 }
@@ -290,9 +293,10 @@ int dsstne_load_sparse_data(dsstne_context* c, const char* name, const uint64_t*
 {
     CAPI_TRY
     NNDataSetBase* d = findDataSet(c, name);
-    // a Boolean dataset has no value array; hand the loader a harmless stand-in of the right length
+    // a Boolean dataset has no value array and its kernels read none: nothing is copied or uploaded for it.  Any other set
+    // without values gets zeros of the right length.
     vector<uint8_t> zeros;
-    if (!sparse_data) {
+    if (!sparse_data && !(d->_attributes & NNDataSetEnums::Boolean)) {
         zeros.assign((size_t)sparse_end[d->_uniqueExamples - 1] * 8, 0);
         sparse_data = zeros.data();
     }
@@ -353,8 +357,16 @@ int dsstne_topk(dsstne_context* c, const char* layer, uint32_t k, const char* fi
 int dsstne_get_topk(dsstne_context* c, const char* layer, uint32_t rows, uint32_t k, float* scores, uint32_t* indexes)
 {
     CAPI_TRY
-    dsxFatal(dsx_memcpy_d2h_pair(scores, c->scoreBuf(layer)->_pDevData, (size_t)rows * k * sizeof(float), indexes,
-                                 c->indexBuf(layer)->_pDevData, (size_t)rows * k * sizeof(uint32_t)),
+    GpuBuffer<NNFloat>* s = c->scoreBuf(layer);
+    GpuBuffer<uint32_t>* i = c->indexBuf(layer);
+    if (s->_bManaged && i->_bManaged) {   // the kernels wrote into host memory: wait for the batch's lane, then it is all there
+        dsxFatal(dsx_sync_lane(c->net()->GetLane()), "dsstne_get_topk");
+        memcpy(scores, s->_pSysData, (size_t)rows * k * sizeof(float));
+        memcpy(indexes, i->_pSysData, (size_t)rows * k * sizeof(uint32_t));
+        return 0;
+    }
+    dsxFatal(dsx_memcpy_d2h_pair(scores, s->_pDevData, (size_t)rows * k * sizeof(float), indexes, i->_pDevData,
+                                 (size_t)rows * k * sizeof(uint32_t)),
              "dsstne_get_topk");
     return 0;
     CAPI_CATCH(-1)
@@ -368,6 +380,12 @@ int dsstne_get_topk_previous(dsstne_context* c, const char* layer, uint32_t rows
     const int lane = (int)((n->GetLane() + n->GetLanes() - 1) % n->GetLanes());
     GpuBuffer<NNFloat>* s = c->dc ? c->dc->getOutputScoresBuffer(layer, lane) : c->scores[lane].at(layer);
     GpuBuffer<uint32_t>* i = c->dc ? c->dc->getOutputIndexesBuffer(layer, lane) : c->indexes[lane].at(layer);
+    if (s->_bManaged && i->_bManaged) {
+        dsxFatal(dsx_sync_lane(lane), "dsstne_get_topk_previous");
+        memcpy(scores, s->_pSysData, (size_t)rows * k * sizeof(float));
+        memcpy(indexes, i->_pSysData, (size_t)rows * k * sizeof(uint32_t));
+        return 0;
+    }
     dsxFatal(dsx_memcpy_d2h_lane(lane, scores, s->_pDevData, (size_t)rows * k * sizeof(float)), "dsstne_get_topk_previous");
     dsxFatal(dsx_memcpy_d2h_lane(lane, indexes, i->_pDevData, (size_t)rows * k * sizeof(uint32_t)), "dsstne_get_topk_previous");
     return 0;
