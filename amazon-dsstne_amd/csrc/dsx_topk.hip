@@ -238,6 +238,21 @@ template <int R> struct WaveTopK {
         }
     }
 
+    // The same with a column: at least k real words are >= w (w need not be a real word itself).  Scores equal to w's then only
+    // pass with a column at or before w's, which admission_score turns into "strictly above" for everything that lies behind it.
+    __device__ __forceinline__ void prime_word(uint64_t w)
+    {
+        if (w - 1 > thr) {
+            thr = w - 1;
+            float key;
+            uint32_t col;
+            unpack_score(w, key, col);
+            thr_key = key;
+            thr_above = key_score((uint32_t)(w >> 32) + 1u);
+            thr_col = col;
+        }
+    }
+
     // Stage the lanes' words that beat the threshold.  All 64 lanes must call this together.  Nothing is merged here: after
     // at most five calls the caller runs drain(), which keeps count < L between bursts.
     __device__ __forceinline__ void stage_only(bool valid, uint64_t word)
@@ -502,7 +517,7 @@ __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kern
     // Vector loads complete in the order they were issued, so the column numbers are requested between the first and the
     // second span: waiting for them then costs no more than waiting for the first span, which priming needs anyway, and the
     // listed scores (requested last) are not waited for until the scan is over.
-    constexpr int kFU = 4;
+    constexpr int kFU = (R >= 2) ? 2 : 4;   // (the longer lists of k > 64 need the registers: fewer listed columns are held at once)
     __shared__ uint32_t sTaint[kTopkThreads / 2];   // 16 bits per lane: bit u = group u of the first two spans holds a listed column
     uint32_t fcol[kFU];
     float fm[kFU], fv[kFU];
@@ -601,7 +616,41 @@ __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kern
         else if (a.k <= 32) t = wave_kth_key<2>(reinterpret_cast<const uint32_t(&)[2]>(all), a.k);
         else if (a.k <= 64) t = wave_kth_key<4>(reinterpret_cast<const uint32_t(&)[4]>(all), a.k);
         else t = wave_kth_key<4 * PV>(all, a.k);
-        if (t > score_key(-__builtin_inff())) list.prime(t);
+        if (t > score_key(-__builtin_inff())) {
+            list.prime(t);
+            // Rows whose best scores tie in their hundreds (saturated sigmoids: exactly 1.0f in every eighth column) would
+            // otherwise stage every group that holds one of them until a list fills up and is sorted.  Among equal scores the
+            // lower column wins, so the bound gets a column: a wavefront's first group is 256 consecutive columns, the lowest it
+            // will see; if k of them reach the bound, the k-th such column X closes the bound — a score equal to it passes at or
+            // before X only, and every later group fails the one compare of the scan.
+            const float S = key_score(t);
+            const float4& g = cur[0];
+            const float e[4] = {g.x, g.y, g.z, g.w};
+            const uint32_t col = head + 4 * (span + threadIdx.x);
+            bool ok[4];
+            uint32_t before = 0, mine = 0, total = 0;
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                ok[c] = e[c] >= S;
+                if constexpr (FILTERED) {
+                    if (ok[c]) ok[c] = !filtered_out(col + c);
+                }
+                const uint64_t q = __ballot(ok[c]);
+                before += __builtin_amdgcn_mbcnt_hi((uint32_t)(q >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)q, 0u));
+                mine += ok[c] ? 1u : 0u;
+                total += (uint32_t)__popcll(q);
+            }
+            if (total >= a.k) {   // wave-uniform
+                const bool has = before < a.k && a.k <= before + mine;   // exactly one lane
+                uint32_t need = has ? a.k - before : 0u, colX = 0;
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    if (ok[c] && need != 0 && --need == 0) colX = col + c;
+                const uint64_t hm = __ballot(has);
+                const uint32_t X = (uint32_t)__builtin_amdgcn_readlane((int)colX, __builtin_ctzll(hm));
+                list.prime_word(pack_score(S, X));
+            }
+        }
     };
     if (R <= 2 && g0 < g1) prime_from_first_spans();   // (k <= 128)
 
@@ -630,10 +679,11 @@ __global__ __launch_bounds__(kTopkThreads, (R <= 2) ? 4 : 2) void topk_scan_kern
         uint32_t hot = 0;
         {
             const float t = list.admission_score(head + 4 * span);   // every column of this span and after is at or beyond that
+            const float t1 = list.admission_score(head + 4 * (span + step));   // ... and every column of its groups 1 to 7 at or beyond this
 #pragma unroll
             for (int u = 0; u < CH; u++) {
                 const float m = fmaxf(fmaxf(cur[u].x, cur[u].y), fmaxf(cur[u].z, cur[u].w));
-                if (__ballot(m >= t) != 0) hot |= 1u << u;
+                if (__ballot(m >= (u == 0 ? t : t1)) != 0) hot |= 1u << u;
             }
         }
         while (hot != 0) {

@@ -43,7 +43,12 @@ def measured_traffic(workload):
         return {}
     w = t.get("workloads", {}).get(workload, {})
     ff, wf = t.get("fetch_factor", 1.0), t.get("write_factor", 1.0)
-    return {k: {"read": int(v["fetch_kib"] * 1024 * ff), "write": int(v["write_kib"] * 1024 * wf)} for k, v in w.items()}
+    out = {}
+    for k, v in w.items():
+        out[k] = {"read": int(v["fetch_kib"] * 1024 * ff), "write": int(v["write_kib"] * 1024 * wf)}
+        if "l2_hit" in v and "l2_miss" in v and v["l2_hit"] + v["l2_miss"] > 0:
+            out[k]["l2_hit_rate"] = round(v["l2_hit"] / (v["l2_hit"] + v["l2_miss"]), 4)
+    return out
 
 
 class StdoutToStderr:
@@ -101,6 +106,18 @@ def timed_windows(step, sync, steps, windows):
         sync()
         out.append((time.perf_counter() - t0) * 1e3 / steps)
     return out
+
+
+def calibration_copy(args, pkg, lib):
+    """--calibrate-copy N: a plain device-to-device copy of N MiB; what FETCH_SIZE / WRITE_SIZE read for it calibrates the counters."""
+    if not args.calibrate_copy:
+        return
+    nbytes = args.calibrate_copy << 20
+    src = pkg.DeviceArray((nbytes // 4,), np.float32)
+    dst = pkg.DeviceArray((nbytes // 4,), np.float32)
+    for _ in range(3):
+        pkg.check(lib.dsx_memcpy_d2d(dst.ptr, src.ptr, nbytes))
+    pkg.check(lib.dsx_sync())
 
 
 def interference_block(pkg, lib, p, steps):
@@ -293,10 +310,20 @@ def network_bench(args, pkg, lib):
     touched = np.unique(np.concatenate([p.sparse_index[int(p.start[r]):int(p.end[r])] for r in rows0])).size
     compulsory = touched * 4 * H + nnzB * (4 + val_bytes) + fixed     # every distinct weight row once
     ms = time_launches(pkg, lib, k_sparse, reps)
-    kernels["sparse_z_kernel"] = {"bound": "hbm", "ms": ms, "achieved": spmm_bytes / ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                  "algorithmic_bytes": spmm_bytes, "compulsory_bytes": compulsory,
-                                  "compulsory_gbs": compulsory / ms / 1e6,
-                                  "note": "algorithmic = every non-zero gathers its weight row (no reuse); compulsory = every distinct weight row of the batch once"}
+    # The sparse layer gathers weight rows that other rows of the batch (and the L2 / last-level cache) mostly already hold: the
+    # bytes it moves to and from HBM are the counters' (profiles/pmc_hbm_traffic.json), and its roofline fraction is those over the
+    # launch time.  The rate at which it consumes gathered bytes (every non-zero's weight row, no reuse) is reported beside it
+    # with the L2 hit rate: a figure of the gather machinery, not of HBM.
+    sp_traffic = traffic.get("sparse_z_kernel")
+    sp = {"bound": "hbm", "ms": ms, "peak": HBM_PEAK_GBS, "unit": "GB/s", "compulsory_bytes": compulsory,
+          "gather": {"bytes": spmm_bytes, "rate_gbs": round(spmm_bytes / ms / 1e6, 1),
+                     "note": "every non-zero gathers its weight row (no reuse): served by L2 and the last-level cache, not a bandwidth of HBM"},
+          "note": "achieved = HBM bytes per launch as FETCH_SIZE / WRITE_SIZE count them over the launch time; compulsory_bytes = every distinct weight row of the batch once"}
+    if sp_traffic:
+        sp["achieved"] = (sp_traffic["read"] + sp_traffic["write"]) / ms / 1e6
+        if sp_traffic.get("l2_hit_rate") is not None:
+            sp["gather"]["l2_hit_rate"] = sp_traffic["l2_hit_rate"]
+    kernels["sparse_z_kernel"] = sp
 
     # the dense layers as the stored-output step runs them: the last one also leaves segment maxima for the guided top-K
     gp = DevicePipeline(p, lib, guided=True)
@@ -330,7 +357,8 @@ def network_bench(args, pkg, lib):
     kernels["topk_scan_kernel"] = {"bound": "hbm", "ms": ms, "achieved": topk_bytes / ms / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                    "algorithmic_bytes": topk_bytes}
     for v in kernels.values():
-        v["frac"] = v["achieved"] / v["peak"]
+        if "achieved" in v:
+            v["frac"] = v["achieved"] / v["peak"]
     if gp.seg_width.value:
         # what the step runs when the output layer left segment maxima: it reads the maxima and the few segments that can hold a
         # result, so it is a chain of dependent loads, not a stream.  Its figure is the bandwidth of what it really moves.
@@ -387,6 +415,8 @@ def network_bench(args, pkg, lib):
             kernels[n]["traffic"] = t["read"] + t["write"]
             kernels[n]["traffic_read"] = t["read"]
             kernels[n]["traffic_write"] = t["write"]
+            if "l2_hit_rate" in t:
+                kernels[n]["l2_hit_rate"] = t["l2_hit_rate"]
 
     candidates = [n for n in kernels if "frac" in kernels[n] and n != split_name and not (deferred and n in (gemm_name, "topk_scan_kernel"))]
     dominant = max(candidates, key=lambda n: kernels[n]["ms"])
@@ -394,14 +424,7 @@ def network_bench(args, pkg, lib):
     roofline = {"kernel": dominant, "bound": d["bound"], "achieved": round(d["achieved"], 3), "peak": d["peak"], "unit": d["unit"],
                 "frac": round(d["frac"], 4), "traffic": d.get("traffic"), "avg_launch_ms": round(d["ms"], 5),
                 "note": "isolated back-to-back launches, clocks settled; `pipeline` below prices the whole timed step"}
-    if args.calibrate_copy:
-        # plain device-to-device copy of known size: what FETCH_SIZE / WRITE_SIZE read for it calibrates the counters
-        nbytes = args.calibrate_copy << 20
-        src = pkg.DeviceArray((nbytes // 4,), np.float32)
-        dst = pkg.DeviceArray((nbytes // 4,), np.float32)
-        for _ in range(3):
-            pkg.check(lib.dsx_memcpy_d2d(dst.ptr, src.ptr, nbytes))
-        pkg.check(lib.dsx_sync())
+    calibration_copy(args, pkg, lib)
 
     # CPU baseline: the oracle (scalar C++ restatement of the reference kernels, OpenMP over rows) on whole batches of the
     # same workload, bounded to about 10-20 s.
@@ -441,7 +464,11 @@ def network_bench(args, pkg, lib):
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": p.name, "batch": B, "input_width": p.widths[0], "layers": p.widths[1:], "top_k": K, "filtered": True,
-                   "resident_batches": batches, "batch_nnz": nnzB, "mean_batch_nnz": round(nnz_mean, 1), "lanes": args.lanes},
+                   "resident_batches": batches, "batch_nnz": nnzB, "mean_batch_nnz": round(nnz_mean, 1), "lanes": args.lanes,
+                   "weights": "N(0, std %g) (the definition's N(0, 0.01) read as a variance), biases %s" % (
+                       p.law["weight_std"], "0" if not p.law["bias_std"] else "N(0, std %g)" % p.law["bias_std"]),
+                   "index_law": p.law["index_law"], "nnz_per_row": p.law["nnz_per_row"], "values": p.law["values"],
+                   "indexed_rows": p.law["indexed_rows"], "seed": p.law["seed"]},
         "windows": {"count": WINDOWS, "steps_each": args.steps, "ms_per_step": [round(w, 5) for w in windows],
                     "min": round(min(windows), 5), "median": round(ms_step, 5), "max": round(max(windows), 5),
                     "note": "value is the median window; the timed steps cycle over the resident batches"},
@@ -496,7 +523,8 @@ def knn_bench(args, pkg, lib):
     step(el)
     flops = 2.0 * Q * D * (rows - pad)
     roofline = {"kernel": "fc_gemm_kernel (knn scores)", "bound": "mfma", "achieved": round(flops / el[0] / 1e9, 3), "peak": FP32_MFMA_PEAK_TF,
-                "unit": "TFLOP/s", "frac": round(flops / el[0] / 1e9 / FP32_MFMA_PEAK_TF, 4), "traffic": None, "avg_launch_ms": round(el[0], 4),
+                "unit": "TFLOP/s", "frac": round(flops / el[0] / 1e9 / FP32_MFMA_PEAK_TF, 4), "traffic": (lambda t: (t["read"] + t["write"]) if t else None)(
+                    measured_traffic(p.name).get("fc_gemm_kernel (knn scores)")), "avg_launch_ms": round(el[0], 4),
                 "topk_ms": round(el[1], 4),
                 "path": {0: "blocks", 1: "candidate lists", 2: "candidate lists, redone block by block"}[lib.dsx_knn_last_search_path()]}
     # the same search with fp16 storage of items and queries (the reference's DataType::FP16): reported beside the fp32 figure
@@ -540,6 +568,7 @@ def knn_bench(args, pkg, lib):
              "scores_ms": round(el[0], 4), "topk_ms": round(el[1], 4),
              "path": {0: "blocks", 1: "candidate lists", 2: "candidate lists, redone block by block"}[lib.dsx_knn_last_search_path()]}
     del planes
+    calibration_copy(args, pkg, lib)
     cpu = None
     if args.cpu_seconds > 0:
         orc = entry.load_oracle()
@@ -554,7 +583,8 @@ def knn_bench(args, pkg, lib):
     return {"metric": "KNN queries/sec (exact top-%d over %d items)" % (K, rows - pad), "value": round(Q / (ms_step / 1e3), 1),
             "unit": "queries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-            "config": {"workload": p.name, "queries": Q, "dim": D, "items": rows - pad, "top_k": K}, "roofline": roofline,
+            "config": {"workload": p.name, "queries": Q, "dim": D, "items": rows - pad, "top_k": K,
+                       "vectors": "N(0, 1) components, rows L2-normalised, seed 1005"}, "roofline": roofline,
             "cpu_baseline": cpu, "f16_storage": f16, "split_products": split}
 
 

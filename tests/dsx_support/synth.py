@@ -38,6 +38,7 @@ class Problem:
         self.sparse_data = None   # values (None for Boolean data)
         self.index = None         # uint32 [examples] (Indexed datasets)
         self.data_weight = None
+        self.law = {}             # how the workload was drawn (for reports): weight spread, index law, non-zeros per row
 
     @property
     def nnz(self):
@@ -178,6 +179,10 @@ def autoencoder(name, seed, n_items, hidden, batch, k, batches=1, zipf_s=None, n
     if indexed:
         p.attributes |= ATTR_INDEXED
         p.index = rng.permutation(rows).astype(np.uint32)
+    p.law = {"seed": seed, "weight_std": WEIGHT_STD, "bias_std": bias_std,
+             "index_law": ("uniform without replacement" if zipf_s is None else "Zipf(s=%g) over a random permutation of the items, without replacement within a row" % zipf_s),
+             "nnz_per_row": ("%d" % nnz_mean if nnz_sigma <= 0 else "lognormal(mean %g, sigma %g) clipped to [%d, %d]" % (nnz_mean, nnz_sigma, nnz_clip[0], nnz_clip[1])),
+             "values": ("0.5 .. 5.0 in steps of 0.5, uniform" if analog else "1 (Boolean)"), "indexed_rows": bool(indexed)}
     return p
 
 
