@@ -216,8 +216,11 @@ int dsx_fc_forward_segmax(const float* X, uint32_t ldx, const float* W, int tran
  *   k_major == 0: vector r is src[r * ld + 0 .. k)        (X, a [batch x k] unit buffer; W stored [n x k], i.e. transposed)
  *   k_major != 0: vector r is src[0 .. k) * ld + r         (W stored [k x n])
  * into `planes`, dsx_fc_split_bytes(rows, k) bytes of 16-byte aligned device memory (3 x 2 bytes per value, rows padded to
- * 256 and k to 16).  Weights are split once, a layer's input once per batch.  Inf and NaN inputs stay Inf / NaN; finite values
- * from 3.0e38 up are kept to bf16 precision only.
+ * 256 and k to 16).  Weights are split once, a layer's input once per batch.  Non-finite operands: an Inf or NaN stays in the
+ * first plane, the other planes hold 0, and the six-term sum then contains Inf x 0 and infinities of either sign: a sum with an
+ * Inf operand comes out NaN (sometimes +/-Inf) where dsx_fc_forward gives +/-Inf (the candidate modes drop NaN scores), one with a
+ * NaN operand NaN as there.  Sums without such
+ * an operand are not affected.  Finite values from 3.0e38 up are kept to bf16 precision only.
  * dsx_fc_forward_split then computes Z as dsx_fc_forward (accumulate, bias, activation) and, with seg_max / seg_width non-NULL
  * and accumulate == 0, the segment maxima as dsx_fc_forward_segmax (*seg_width = 64 for every shape).  A plane (2 bytes x rows
  * padded x k padded) must stay below 4 GiB.

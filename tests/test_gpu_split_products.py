@@ -119,6 +119,34 @@ def test_fc_split_vs_oracle_fp64_and_fp32_kernel(pkg, dsx, orc, rng, tile_rows, 
     assert err_split < 2e-6
 
 
+def test_fc_split_infinite_operand_gives_nan_only_where_it_takes_part(pkg, dsx, rng):
+    """The stated limit of the mode: an Inf operand sits in the first plane with zeros behind it, so the six-term sum holds
+    Inf x 0 (or +Inf and -Inf from planes of opposite sign) and the sums it takes part in come out NaN or +/-Inf, where the fp32
+    kernel gives +/-Inf.  Every other sum is unaffected."""
+    B, k, n = 130, 48, 200
+    X = rng.standard_normal((B, k)).astype(np.float32)
+    W = rng.standard_normal((k, n)).astype(np.float32)
+    X[7, 5] = np.inf
+    W[9, 33] = -np.inf
+    dX, dW = dev(pkg, X), dev(pkg, W)
+    xp = planes_of(pkg, dsx, dX, k, 0, B, k)
+    wp = planes_of(pkg, dsx, dW, n, 1, n, k)
+    Z = pkg.DeviceArray((B, n), np.float32)
+    pkg.check(dsx.dsx_fc_forward_split(xp.ptr, wp.ptr, None, Z.ptr, n, B, k, n, 0, 3, None, None, None))
+    Zf = pkg.DeviceArray((B, n), np.float32)
+    pkg.check(dsx.dsx_fc_forward(dX.ptr, k, dW.ptr, 0, None, Zf.ptr, n, B, k, n, 0, 3, None))
+    got, plain = Z.numpy(), Zf.numpy()
+    touched = np.zeros((B, n), dtype=bool)
+    touched[7, :] = True
+    touched[:, 33] = True
+    assert np.all(~np.isfinite(got[touched])) and np.all(~np.isfinite(plain[touched]))
+    assert np.isnan(got[touched]).any()                                  # Inf x 0, or Inf - Inf between the planes' terms
+    assert np.isinf(plain[7, 0]) and np.isinf(plain[0, 33])              # the fp32 kernel keeps the infinity
+    clean = ~touched
+    assert np.all(np.isfinite(got[clean]))
+    assert_close(got[clean], plain[clean], "sums without a non-finite operand", rel=1e-4, abs_floor=1.0)
+
+
 @pytest.mark.parametrize("act", [0, 1, 2, 10, 11, 12])
 @pytest.mark.parametrize("accumulate", [0, 1])
 def test_fc_split_epilogue(pkg, dsx, orc, rng, tile_rows, act, accumulate):
