@@ -83,6 +83,7 @@ SIGNATURES = {
     "dsx_fc_forward": [_vp, _u32, _vp, _int, _vp, _vp, _u32, _u32, _u32, _u32, _int, _u32, C.POINTER(ActParams)],
     "dsx_fc_forward_segmax": [_vp, _u32, _vp, _int, _vp, _vp, _u32, _u32, _u32, _u32, _u32, C.POINTER(ActParams), _vp, C.POINTER(_u32)],
     "dsx_fc_split": [_vp, _u32, _int, _u32, _u32, _vp],
+    "dsx_fc_forward_planes": [_vp, _u32, _vp, _int, _vp, _vp, _u32, _u32, _u32, _u32, _u32, C.POINTER(ActParams), _vp],
     "dsx_testing_set_split_tile_rows": [_u32],
     "dsx_fc_forward_split": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _int, _u32, C.POINTER(ActParams), _vp, C.POINTER(_u32)],
     "dsx_activation": [_vp, _u32, _u32, _u32, C.POINTER(ActParams)],

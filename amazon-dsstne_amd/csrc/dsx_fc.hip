@@ -30,6 +30,9 @@ struct FcArgs {
     uint32_t nseg;
     float slope, alpha, lambda;
     CandArgs cand;       // candidate mode (template flag CAND): Z is not written, see candidate_epilogue
+    // fc_small_kernel only: also write Z as bf16 planes (the next layer's operand in the split-products mode), as fc_split_kernel would
+    uint4* out_planes;
+    uint32_t out_rows_padded, out_kblocks;
 };
 
 // Epilogue shared by the GEMM kernels: bias, accumulate, activation, store, and on request the maxima of 64-column segments.
@@ -468,6 +471,35 @@ __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? (CAND == 2 ? 3 : 4) : 
 // four ways: every lane requests all its operands at once, straight from global memory into registers (the X row segment as
 // 128-bit loads, the W column as dwords that coalesce across the 32 lanes of a half wave), one round trip instead of one
 // per k-step; the four partial tiles meet in LDS.  S = k / 4 (32 or 64).
+// Three bf16 planes of eight fp32 values (see fc_split_kernel below): hi = RN(x), mid = RN(x - hi), lo = RN(x - hi - mid), packed two
+// to a word; infinities, NaN and what would round up to infinity stay in the first plane alone.  One 16-byte unit per plane.
+__device__ __forceinline__ uint32_t bf16_rn_bits(float x)
+{
+    const uint32_t u = __float_as_uint(x);
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+
+__device__ __forceinline__ void split_unit_store(const float (&x)[8], uint4* __restrict__ planes, uint64_t unit, uint64_t plane)
+{
+    uint32_t h[8], m[8], l[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        if (!(fabsf(x[e]) < 3.0e38f)) {
+            h[e] = __float_as_uint(x[e]) >> 16; m[e] = 0; l[e] = 0;
+            if (x[e] != x[e]) h[e] |= 0x40;
+            continue;
+        }
+        h[e] = bf16_rn_bits(x[e]);
+        const float r1 = x[e] - __uint_as_float(h[e] << 16);   // exact
+        m[e] = bf16_rn_bits(r1);
+        const float r2 = r1 - __uint_as_float(m[e] << 16);     // exact
+        l[e] = bf16_rn_bits(r2);
+    }
+    planes[unit] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+    planes[plane + unit] = make_uint4(m[0] | (m[1] << 16), m[2] | (m[3] << 16), m[4] | (m[5] << 16), m[6] | (m[7] << 16));
+    planes[2 * plane + unit] = make_uint4(l[0] | (l[1] << 16), l[2] | (l[3] << 16), l[4] | (l[5] << 16), l[6] | (l[7] << 16));
+}
+
 template <int S, int ACT>
 __global__ __launch_bounds__(kFcThreads) void fc_small_kernel(FcArgs a)
 {
@@ -502,13 +534,33 @@ __global__ __launch_bounds__(kFcThreads) void fc_small_kernel(FcArgs a)
 #pragma unroll
     for (int v = 0; v < 16; v++) sPart[wave][v][lane] = acc[v];
     __syncthreads();
-    if (col0 + l32 >= a.n) return;
+    const bool col_ok = col0 + l32 < a.n;
+    float y[4];
 #pragma unroll
     for (int q = 0; q < 4; q++) {
         const int v = wave * 4 + q;
         const float x = ((sPart[0][v][lane] + sPart[1][v][lane]) + (sPart[2][v][lane] + sPart[3][v][lane])) + bias;
         const uint32_t r = row0 + 8 * (v / 4) + 4 * lhi + (v % 4);   // v / 4 == wave, v % 4 == q
-        if (r < a.batch) a.Z[(uint64_t)r * a.ldz + col0 + l32] = activate<ACT>(x, a.slope, a.alpha, a.lambda);
+        y[q] = activate<ACT>(x, a.slope, a.alpha, a.lambda);
+        if (col_ok && r < a.batch) a.Z[(uint64_t)r * a.ldz + col0 + l32] = y[q];
+    }
+    if (a.out_planes == nullptr) return;   // (the same for the whole workgroup)
+    // The tile once more as planes: a unit is eight consecutive columns of one row.  The tile goes through LDS (the partial
+    // tiles are done with after the barrier), 128 lanes then pack one unit each.
+    __syncthreads();
+    float (*sOut)[33] = reinterpret_cast<float (*)[33]>(&sPart[0][0][0]);
+#pragma unroll
+    for (int q = 0; q < 4; q++) sOut[8 * wave + 4 * lhi + q][l32] = col_ok ? y[q] : 0.0f;   // zeros beyond the last column: k padding
+    __syncthreads();
+    if (tid < 128) {
+        const uint32_t rl = tid >> 2, kbl = tid & 3;
+        const uint32_t r = row0 + rl, kb = col0 / 8 + kbl;
+        if (r < a.batch && kb < a.out_kblocks) {
+            float x[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) x[e] = sOut[rl][8 * kbl + e];
+            split_unit_store(x, a.out_planes, (uint64_t)kb * a.out_rows_padded + r, (uint64_t)a.out_kblocks * a.out_rows_padded);
+        }
     }
 }
 
@@ -572,7 +624,7 @@ template <int MI, int NI, int BK> static void launch_fc_shape(FcArgs& a, int xv,
 
 int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int transposed, const float* bias, float* Z, uint32_t ldz,
            uint32_t batch, uint32_t k, uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params, float* seg_max,
-           uint32_t* seg_width)
+           uint32_t* seg_width, void* out_planes)
 {
     if (seg_width) *seg_width = 0;
     FcArgs a{};
@@ -603,11 +655,18 @@ int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int trans
         if (k <= 256) launch_fc_shape<2, 2, 8>(a, xv, wv, transposed != 0);
         else launch_fc_shape<2, 2, 16>(a, xv, wv, transposed != 0);
     } else if (!transposed && !accumulate && xv == 4 && (k == 128 || k == 256) && (uint64_t)batch * n <= (1u << 20)) {
+        if (out_planes) {   // the result also as the next layer's planes, written by the same workgroups
+            a.out_planes = reinterpret_cast<uint4*>(out_planes);
+            a.out_rows_padded = split_rows_padded(batch);
+            a.out_kblocks = (n + 15) / 16 * 2;
+            out_planes = nullptr;
+        }
         if (k == 128) launch_fc_small<32>(a);   // latency bound: all operands in one round trip
         else launch_fc_small<64>(a);
     } else
         launch_fc_shape<1, 1, 32>(a, xv, wv, transposed != 0);   // few workgroups: deep k-steps, fewer barrier round trips
     DSX_LAUNCH_CHECK("fc_gemm_kernel");
+    if (out_planes) return fc_split_planes_run(Z, ldz, 1, batch, n, out_planes);   // every other kernel: a launch of its own
     return DSX_OK;
 }
 
@@ -673,12 +732,6 @@ int fc_layer_candidates_run(const float* X, uint32_t ldx, const float* W, uint32
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // (a native vector: arrays of it stay in registers)
 
-__device__ __forceinline__ uint32_t bf16_rn_bits(float x)
-{
-    const uint32_t u = __float_as_uint(x);
-    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
-}
-
 // src element (r, kk) is src[r * stride_r + kk * stride_k].  One lane per (block of eight k, row); consecutive lanes take
 // consecutive rows (a [k][n] weight matrix is read along n, the planes are written 16 bytes per lane, consecutively).
 __global__ __launch_bounds__(256) void fc_split_kernel(const float* __restrict__ src, uint64_t stride_r, uint64_t stride_k, uint32_t rows,
@@ -687,27 +740,13 @@ __global__ __launch_bounds__(256) void fc_split_kernel(const float* __restrict__
     const uint64_t id = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (id >= (uint64_t)rows_padded * kblocks) return;
     const uint32_t r = (uint32_t)(id % rows_padded), kb = (uint32_t)(id / rows_padded);
-    uint32_t h[8], m[8], l[8];
+    float x[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) {
         const uint32_t kk = kb * 8 + e;
-        float x = 0.0f;
-        if (r < rows && kk < k) x = src[r * stride_r + kk * stride_k];
-        if (!(fabsf(x) < 3.0e38f)) {   // infinities, NaN and what would round up to infinity stay in the first plane alone
-            h[e] = __float_as_uint(x) >> 16; m[e] = 0; l[e] = 0;
-            if (x != x) h[e] |= 0x40;
-            continue;
-        }
-        h[e] = bf16_rn_bits(x);
-        const float r1 = x - __uint_as_float(h[e] << 16);   // exact
-        m[e] = bf16_rn_bits(r1);
-        const float r2 = r1 - __uint_as_float(m[e] << 16);  // exact
-        l[e] = bf16_rn_bits(r2);
+        x[e] = (r < rows && kk < k) ? src[r * stride_r + kk * stride_k] : 0.0f;
     }
-    const uint64_t unit = (uint64_t)kb * rows_padded + r, plane = (uint64_t)kblocks * rows_padded;
-    planes[unit] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
-    planes[plane + unit] = make_uint4(m[0] | (m[1] << 16), m[2] | (m[3] << 16), m[4] | (m[5] << 16), m[6] | (m[7] << 16));
-    planes[2 * plane + unit] = make_uint4(l[0] | (l[1] << 16), l[2] | (l[3] << 16), l[4] | (l[5] << 16), l[6] | (l[7] << 16));
+    split_unit_store(x, planes, (uint64_t)kb * rows_padded + r, (uint64_t)kblocks * rows_padded);
 }
 
 struct FcSplitArgs {
@@ -1011,6 +1050,19 @@ int dsx_fc_forward(const float* X, uint32_t ldx, const float* W, int transposed,
     DSX_CHECK_ARG(is_elementwise_activation(activation), "dsx_fc_forward: activation %u is a row operation; pass DSX_ACT_LINEAR and call dsx_activation", activation);
     if (batch == 0) return DSX_OK;
     return fc_run(X, ldx, W, transposed ? k : n, transposed, bias, Z, ldz, batch, k, n, accumulate, activation, params);
+}
+
+int dsx_fc_forward_planes(const float* X, uint32_t ldx, const float* W, int transposed, const float* bias, float* Z, uint32_t ldz,
+                          uint32_t batch, uint32_t k, uint32_t n, uint32_t activation, const dsx_act_params* params, void* z_planes)
+{
+    DSX_REQUIRE_INIT();
+    DSX_CHECK_ARG(X && W && Z && z_planes, "dsx_fc_forward_planes: null device pointer");
+    DSX_CHECK_ARG(((uintptr_t)z_planes % 16) == 0, "dsx_fc_forward_planes: planes must be 16-byte aligned");
+    DSX_CHECK_ARG(k > 0 && n > 0, "dsx_fc_forward_planes: k = %u, n = %u", k, n);
+    DSX_CHECK_ARG(ldx >= k && ldz >= n, "dsx_fc_forward_planes: row pitch smaller than the row (ldx %u < k %u or ldz %u < n %u)", ldx, k, ldz, n);
+    DSX_CHECK_ARG(is_elementwise_activation(activation), "dsx_fc_forward_planes: activation %u is a row operation", activation);
+    if (batch == 0) return DSX_OK;
+    return fc_run(X, ldx, W, transposed ? k : n, transposed, bias, Z, ldz, batch, k, n, 0, activation, params, nullptr, nullptr, z_planes);
 }
 
 int dsx_fc_forward_segmax(const float* X, uint32_t ldx, const float* W, int transposed, const float* bias, float* Z, uint32_t ldz,

@@ -101,7 +101,7 @@ int topk_merge(const uint64_t* partial, uint32_t slots, uint32_t k, float* keys,
 // GEMM building block shared with the KNN search (dsx_fc.hip): Z = X.W (+bias, activation), see dsx_fc_forward.
 int fc_run(const float* X, uint32_t ldx, const float* W, uint32_t ldw, int transposed, const float* bias, float* Z, uint32_t ldz,
            uint32_t batch, uint32_t k, uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params,
-           float* seg_max = nullptr, uint32_t* seg_width = nullptr);
+           float* seg_max = nullptr, uint32_t* seg_width = nullptr, void* out_planes = nullptr);
 // Candidate mode of the same kernel (exact KNN): scores are compared with the rows' bounds and the survivors appended to
 // per-row lists as packed words (CandArgs); nothing else is written.  knn_refresh folds a row's candidates into its best
 // list.  The caller guarantees 16-byte aligned operands with pitches that are multiples of four floats.

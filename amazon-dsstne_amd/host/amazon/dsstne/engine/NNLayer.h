@@ -72,6 +72,7 @@ private:
         unique_ptr<GpuBuffer<NNFloat>> unit;
         unique_ptr<GpuBuffer<NNFloat>> segMax;
         unique_ptr<GpuBuffer<uint32_t>> splitInput;
+        bool splitInputFresh = false;
         uint32_t segWidth = 0;
         bool deferred = false;
         uint32_t deferredBatch = 0;
@@ -89,6 +90,8 @@ private:
     bool _bSplitProducts = false;
     uint32_t _splitMinTiles = 0;
     unique_ptr<GpuBuffer<uint32_t>> _pbSplitInput;
+    bool _bSplitInputFresh = false;   // the layer before this one wrote the planes of the current batch itself (dsx_fc_forward_planes)
+    void* SplitInputBuffer();         // this lane's buffer for them, allocated on first use
     bool UseSplitProducts(uint32_t batch) const
     {
         if (!_bSplitProducts || _vIncomingLayer.empty()) return false;
@@ -109,6 +112,7 @@ private:
         mine.unit.swap(_pbUnit);
         mine.segMax.swap(_pbSegMax);
         mine.splitInput.swap(_pbSplitInput);
+        mine.splitInputFresh = _bSplitInputFresh;
         mine.segWidth = _segWidth;
         mine.deferred = _deferred;
         mine.deferredBatch = _deferredBatch;
@@ -116,6 +120,7 @@ private:
         _pbUnit.swap(next.unit);
         _pbSegMax.swap(next.segMax);
         _pbSplitInput.swap(next.splitInput);
+        _bSplitInputFresh = next.splitInputFresh;
         _segWidth = next.segWidth;
         _deferred = next.deferred;
         _deferredBatch = next.deferredBatch;

@@ -185,9 +185,19 @@ void NNLayer::ForwardPropagateFullyConnected(uint32_t position, uint32_t batch, 
         } else if (UseSplitProducts(batch)) {
             ForwardSplit(batch, NULL, NULL);
         } else {
-            dsxFatal(dsx_fc_forward(src->GetUnitBuffer(), src->_stride, wsrc->_pbWeight->_pDevData, w->_bTransposed ? 1 : 0,
-                                    w->_pbBias->_pDevData, pUnit, _stride, batch, src->_stride, _localStride, 0, (uint32_t)_activation, &params),
-                     "NNLayer::ForwardPropagate: GEMM failure");
+            // The only consumer of this layer forms its products from bf16 planes of its input: this layer's kernel writes them
+            // along with its result (one launch less per batch than splitting the result afterwards).
+            NNLayer* next = (_vOutgoingLayer.size() == 1 && _vOutgoingSkip.empty()) ? _vOutgoingLayer[0] : NULL;
+            if (next && next->_vIncomingLayer.size() == 1 && next->_vIncomingLayer[0] == this && next->UseSplitProducts(batch)) {
+                dsxFatal(dsx_fc_forward_planes(src->GetUnitBuffer(), src->_stride, wsrc->_pbWeight->_pDevData, w->_bTransposed ? 1 : 0,
+                                               w->_pbBias->_pDevData, pUnit, _stride, batch, src->_stride, _localStride, (uint32_t)_activation,
+                                               &params, next->SplitInputBuffer()),
+                         "NNLayer::ForwardPropagate: GEMM failure");
+                next->_bSplitInputFresh = true;
+            } else
+                dsxFatal(dsx_fc_forward(src->GetUnitBuffer(), src->_stride, wsrc->_pbWeight->_pDevData, w->_bTransposed ? 1 : 0,
+                                        w->_pbBias->_pDevData, pUnit, _stride, batch, src->_stride, _localStride, 0, (uint32_t)_activation, &params),
+                         "NNLayer::ForwardPropagate: GEMM failure");
         }
         return;
     }
@@ -245,14 +255,23 @@ void NNLayer::ForwardSplit(uint32_t batch, NNFloat* pSegMax, uint32_t* pSegWidth
              "NNLayer::ForwardPropagate: GEMM failure");
 }
 
+void* NNLayer::SplitInputBuffer()
+{
+    const size_t words = (size_t)(dsx_fc_split_bytes(_batch, _vIncomingLayer[0]->_stride) / sizeof(uint32_t));
+    if (!_pbSplitInput || _pbSplitInput->_length < words) _pbSplitInput.reset(new GpuBuffer<uint32_t>(words));
+    return _pbSplitInput->_pDevData;
+}
+
 const void* NNLayer::SplitInput(uint32_t batch)
 {
     NNLayer* src = _vIncomingLayer[0];
-    const uint32_t k = src->_stride;
-    const size_t words = (size_t)(dsx_fc_split_bytes(_batch, k) / sizeof(uint32_t));
-    if (!_pbSplitInput || _pbSplitInput->_length < words) _pbSplitInput.reset(new GpuBuffer<uint32_t>(words));
-    dsxFatal(dsx_fc_split(src->GetUnitBuffer(), src->_stride, 0, batch, k, _pbSplitInput->_pDevData), "NNLayer::ForwardPropagate: input planes");
-    return _pbSplitInput->_pDevData;
+    void* planes = SplitInputBuffer();
+    if (_bSplitInputFresh) {   // written by the source layer's own kernel, for this batch
+        _bSplitInputFresh = false;
+        return planes;
+    }
+    dsxFatal(dsx_fc_split(src->GetUnitBuffer(), src->_stride, 0, batch, src->_stride, planes), "NNLayer::ForwardPropagate: input planes");
+    return planes;
 }
 
 void NNLayer::CalculateActivation(uint32_t batch)

@@ -285,6 +285,7 @@ void NNNetwork::PredictBatch(uint32_t layers)
     if (_position + batch > _examples) batch = _examples - _position;
     ClearUpdates();
     LoadBatch();
+    for (auto l : _vLayer) l->_bSplitInputFresh = false;   // planes a layer wrote for its consumer belong to the batch they were written in
     for (auto l : _vFPOrder) l->ForwardPropagate(_position, batch, false);
 }
 

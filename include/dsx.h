@@ -227,6 +227,11 @@ int dsx_fc_forward_segmax(const float* X, uint32_t ldx, const float* W, int tran
  * A workgroup's tile has 128 rows, or 256 for k >= 512 when that still leaves four tiles per compute unit; results do not
  * depend on it. */
 uint64_t dsx_fc_split_bytes(uint32_t rows, uint32_t k);
+/* dsx_fc_forward (accumulate == 0) that leaves its result a second time as planes: z_planes as dsx_fc_split(Z, ldz, 0, batch, n,
+ * z_planes) would write them (dsx_fc_split_bytes(batch, n) bytes), for the layer that takes Z as its input in this mode.  The
+ * small-layer kernel (k = 128 or 256, batch x n <= 2^20) writes them itself; every other shape runs the splitter behind the layer. */
+int dsx_fc_forward_planes(const float* X, uint32_t ldx, const float* W, int transposed, const float* bias, float* Z, uint32_t ldz,
+                          uint32_t batch, uint32_t k, uint32_t n, uint32_t activation, const dsx_act_params* params, void* z_planes);
 int dsx_fc_split(const float* src, uint32_t ld, int k_major, uint32_t rows, uint32_t k, void* planes);
 int dsx_fc_forward_split(const void* x_planes, const void* w_planes, const float* bias, float* Z, uint32_t ldz, uint32_t batch, uint32_t k,
                          uint32_t n, int accumulate, uint32_t activation, const dsx_act_params* params, float* seg_max,

@@ -335,3 +335,27 @@ def test_knn_search_split(pkg, dsx, orc, synth, items, queries, dim, k, blocks):
     assert_close(got_s, np.take_along_axis(full, got_i.astype(np.int64), axis=1), "knn scores, split products", rel=1e-4, abs_floor=0.05)
     assert np.all(np.diff(got_s, axis=1) <= 0)
     assert el[0] > 0 and el[1] > 0
+
+
+@pytest.mark.parametrize("B,k,n,act", [(1024, 128, 128, 2), (200, 256, 96, 0), (33, 128, 50, 3), (700, 512, 300, 2)])
+def test_fc_forward_planes_matches_forward_then_split(pkg, dsx, rng, B, k, n, act):
+    """dsx_fc_forward_planes = dsx_fc_forward + dsx_fc_split of its result, bit for bit (result and planes; the small-layer kernel
+    writes the planes itself, other shapes run the splitter behind the layer), also over stale contents of the planes buffer."""
+    say("fc_forward_planes B=%d k=%d n=%d act=%d" % (B, k, n, act))
+    X = rng.standard_normal((B, k)).astype(np.float32)
+    W = (rng.standard_normal((k, n)) * 0.2).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    dX, dW, db = dev(pkg, X), dev(pkg, W), dev(pkg, bias)
+    words = dsx.dsx_fc_split_bytes(B, n) // 4
+    Z1 = pkg.DeviceArray((B, n), np.float32)
+    P1 = pkg.DeviceArray.from_numpy(np.zeros(words, dtype=np.uint32))
+    pkg.check(dsx.dsx_fc_forward(dX.ptr, k, dW.ptr, 0, db.ptr, Z1.ptr, n, B, k, n, 0, act, None))
+    pkg.check(dsx.dsx_fc_split(Z1.ptr, n, 0, B, n, P1.ptr))
+    Z2 = pkg.DeviceArray((B, n), np.float32)
+    P2 = pkg.DeviceArray.from_numpy(np.zeros(words, dtype=np.uint32))
+    pkg.check(dsx.dsx_fc_forward_planes(dX.ptr, k, dW.ptr, 0, db.ptr, Z2.ptr, n, B, k, n, act, None, P2.ptr))
+    assert np.array_equal(Z1.numpy().view(np.uint32), Z2.numpy().view(np.uint32))
+    f1, rp, kp = bf16_planes_to_float(P1.numpy(), B, n)
+    f2, _, _ = bf16_planes_to_float(P2.numpy(), B, n)
+    assert np.array_equal(f1[:, :B, :], f2[:, :B, :])                       # every valid row, k padding included
+    assert not f2[:, B:, :].any()                                           # rows beyond the batch stay as they were (zero)
