@@ -780,6 +780,7 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
     __shared__ uint64_t sStage[kTopkWaves][List::kStageWords];
     __shared__ uint32_t sPrime[kTopkWaves][kGuidedMaxK];
     __shared__ uint32_t sListCount, sBound;
+    __shared__ uint32_t sChunk[8 * kTopkWaves];   // listed segments per group of 64 maxima
     extern __shared__ uint32_t sDyn[];   // segments to read [nseg] | their maxima [nseg] | best listed score per segment [nseg] | bitmap of listed columns
     uint32_t* sList = sDyn;
     uint32_t* sListKey = sDyn + a.nseg;
@@ -924,11 +925,13 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
     }
 
     // Segments whose maximum (listed or not) reaches the bound.
+    uint64_t listed[E];
 #pragma unroll
     for (int e = 0; e < E; e++) {
         const uint32_t idx = e * kTopkThreads + threadIdx.x;
         const bool flagged = idx < a.nseg && mk[e] >= bound;
         const uint64_t m = __ballot(flagged);
+        listed[e] = m;
         if (m == 0) continue;
         uint32_t base = 0;
         if (lane == 0) base = atomicAdd(&sListCount, (uint32_t)__popcll(m));
@@ -940,12 +943,43 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
         }
     }
     __syncthreads();
+    const uint32_t count = sListCount;
+    constexpr int kSegsInFlight = 8;
+    // More segments than one round of reads takes (rows of tied scores, mostly): the list is written again in ascending
+    // order, so that the first round reads the lowest columns and what only ties behind them can be left out.  Lane j holds
+    // the count of the j-th group of 64 maxima; a scan over the first lanes gives every group its place.
+    const bool heavy = bound != 0 && count > kTopkWaves * kSegsInFlight;   // the same for the whole workgroup
+    if (heavy) {
+        if (lane == 0) {
+#pragma unroll
+            for (int e = 0; e < E; e++) sChunk[e * kTopkWaves + wave] = (uint32_t)__popcll(listed[e]);
+        }
+        __syncthreads();   // (everyone has read the count and is done with the unordered list)
+        const uint32_t mine = (lane < (uint32_t)(E * kTopkWaves)) ? sChunk[lane] : 0u;
+        uint32_t incl = mine;
+#pragma unroll
+        for (int d = 1; d < E * kTopkWaves; d *= 2) {
+            const uint32_t up = (uint32_t)__shfl_up((int)incl, d);
+            if (lane >= (uint32_t)d) incl += up;
+        }
+        const uint32_t excl = incl - mine;
+#pragma unroll
+        for (int e = 0; e < E; e++) {
+            const uint32_t base = (uint32_t)__shfl((int)excl, e * kTopkWaves + (int)wave);
+            const uint64_t m = listed[e];
+            if ((m >> lane) & 1ull) {
+                const uint32_t pos = base + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+                sList[pos] = e * kTopkThreads + threadIdx.x;
+                sListKey[pos] = mk[e];
+            }
+        }
+        __syncthreads();
+    }
 
     // One lane per column of a segment, eight segments in flight per wave: the usual dozen or two of segments are one round
     // trip.  A segment whose maximum no longer reaches what its columns need is not read: in a row of saturated scores every
     // segment reaches the bound, but once a wavefront holds k of them, later segments that only tie are out.
-    const uint32_t count = sListCount;
-    constexpr int kSegsInFlight = 8;
+    bool first_round = heavy;
     // (the listed segments are dealt out one at a time: the usual dozen or two then keep all four wavefronts busy)
     for (uint32_t i0 = wave; i0 < count; i0 += kTopkWaves * kSegsInFlight) {
         float v[kSegsInFlight];
@@ -962,6 +996,52 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
                     if (col[u] < a.width) v[u] = row[col[u]];
                 }
             }
+        }
+        // Rows of tied scores (saturated activations): when the wavefront's first segments already hold k columns that reach
+        // the bound, the largest column among the first k of them goes into the bound, and what only ties behind it is
+        // neither staged here nor read later.
+        if (first_round) {   // wave-uniform
+            first_round = false;
+            uint64_t qm[kSegsInFlight];   // lanes whose score reaches the bound and whose column is not listed
+            uint32_t reach = 0;
+#pragma unroll
+            for (int u = 0; u < kSegsInFlight; u++) {
+                bool q = v[u] >= list.thr_key;
+                qm[u] = 0;
+                if (__ballot(q) == 0) continue;
+                if (q) q = !filtered_out(col[u]);
+                qm[u] = __ballot(q);
+                reach += (uint32_t)__popcll(qm[u]);
+            }
+            if (reach >= a.k) {
+                const float S = list.thr_key;
+                uint32_t need = a.k, X = 0;
+                bool found = false;
+#pragma unroll
+                for (int u = 0; u < kSegsInFlight; u++) {
+                    const uint32_t c = (uint32_t)__popcll(qm[u]);
+                    if (found || c == 0) continue;
+                    int at;
+                    if (need > c) {
+                        need -= c;
+                        at = 63 - __builtin_clzll(qm[u]);
+                    } else {
+                        const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(qm[u] >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)qm[u], 0u));
+                        at = __builtin_ctzll(__ballot(((qm[u] >> lane) & 1ull) && rank + 1 == need));
+                        found = true;
+                    }
+                    const uint32_t x = (uint32_t)__builtin_amdgcn_readlane((int)col[u], at);
+                    X = x > X ? x : X;
+                }
+                list.prime_word(pack_score(S, X));
+            }
+#pragma unroll
+            for (int u = 0; u < kSegsInFlight; u++) {
+                if (qm[u] != 0) list.stage_only((qm[u] >> lane) & 1ull, pack_score(v[u], col[u]));
+                if ((u & 3) == 3) list.drain();
+            }
+            list.drain();
+            continue;
         }
 #pragma unroll
         for (int u = 0; u < kSegsInFlight; u++) {

@@ -541,6 +541,22 @@ def test_topk_saturated_rows_scan_and_guided(pkg, dsx, orc, rng, batch, width, k
     assert_topk_exact(gk, gi, rk, ri)
 
 
+@pytest.mark.parametrize("batch,width,k,share", [(48, 27278, 10, 0.13), (8, 27278, 50, 0.4), (4, 120000, 32, 0.02)])
+def test_topk_saturated_rows_with_multipliers(pkg, dsx, orc, rng, batch, width, k, share):
+    """Tied rows whose listed columns carry multipliers: x1 keeps a listed column in the tie at its own place, x2 puts it on
+    top, x0.5 and x0 take it out.  The guided form reads such rows in ascending order of columns and gives its bound a column."""
+    say("topk saturated with multipliers batch=%d width=%d k=%d share=%g" % (batch, width, k, share))
+    scores = (rng.random((batch, width), dtype=np.float32) * np.float32(0.999)).astype(np.float32)
+    scores[rng.random((batch, width)) < share] = 1.0
+    start, end, fidx = random_csr(rng, batch, width, 600, empty_rows=(1,))
+    fmul = rng.choice(np.array([0.0, 0.5, 1.0, 2.0], dtype=np.float32), size=fidx.size).astype(np.float32)
+    keys, idx = run_filtered(pkg, dsx, scores, k, 0, None, start, end, fidx, fmul)
+    rk, ri = orc.topk_filtered(scores, k, 0, None, start, end, fidx, fmul)
+    assert_topk_exact(keys, idx, rk, ri)
+    gk, gi = run_guided(pkg, dsx, scores, k, segment_maxima(scores), 0, None, start, end, fidx, fmul)
+    assert_topk_exact(gk, gi, rk, ri)
+
+
 def test_topk_guided_indexed_filter_and_position(pkg, dsx, orc, rng):
     rows, batch, width, k, position = 40, 17, 3000, 20, 9
     scores = rng.random((batch, width), dtype=np.float32)
