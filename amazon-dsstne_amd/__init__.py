@@ -67,6 +67,7 @@ SIGNATURES = {
     "dsx_memcpy_d2h_lane": [_int, _vp, _vp, _sz],
     "dsx_memcpy_d2h_pair": [_vp, _vp, _sz, _vp, _vp, _sz],
     "dsx_memcpy_h2d_unordered": [_vp, _vp, _sz],
+    "dsx_memcpy_h2d_unordered_many": [C.c_int, _vp, _vp, _vp],
     "dsx_lane_wait_other": [],
     "dsx_marker_create": [C.POINTER(C.c_void_p)],
     "dsx_marker_record": [_vp],

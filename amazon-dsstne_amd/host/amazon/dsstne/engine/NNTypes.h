@@ -100,6 +100,11 @@ struct NNDataSetBase {
     void NoteSparseRead();
     // The lane the next PredictBatch will run on (kept by NNNetwork); a wrong value costs a wait between the lanes, no more.
     static int s_nextLane;
+    // No counterpart in the reference (which fills the host vectors first and uploads them): a LoadSparseData that goes
+    // straight to the device arrays leaves _vSparseStart / End / Index / Data behind, and the accessors below, Shard and
+    // SaveNetCDF fetch them back before they read them.  Code that reads the vectors itself calls SyncSparseHostCopy() first.
+    bool _bSparseHostStale = false;
+    virtual void SyncSparseHostCopy() = 0;
 
     NNDataSetBase();
     virtual ~NNDataSetBase() = 0;
@@ -175,6 +180,7 @@ public:
     void CopySparseData(const long* srcSparseStart, const long* srcSparseEnd, const void* srcSparseData, const long* srcSparseIndex) override;
     void LoadIndexedData(const uint32_t* srcIndexedData) override;
     void LoadDataWeight(const NNFloat* srcWeightData) override;
+    void SyncSparseHostCopy() override;
 
     void RefreshState(uint32_t batch) override {}
     bool Shard(NNDataSetEnums::Sharding sharding) override;

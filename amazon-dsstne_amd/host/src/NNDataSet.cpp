@@ -192,6 +192,7 @@ template <typename T> void NNDataSet<T>::uploadSparse()
     _pbSparseEnd->Upload(_vSparseEnd.data());
     _pbSparseIndex->Upload(_vSparseIndex.data());
     if (_pbSparseData) _pbSparseData->Upload(_vSparseData.data());
+    _bSparseHostStale = false;
 }
 
 template <typename T>
@@ -206,6 +207,24 @@ void NNDataSet<T>::CopySparseData(const uint64_t* srcSparseStart, const uint64_t
     memcpy(_vSparseEnd.data(), srcSparseEnd, _uniqueExamples * sizeof(uint64_t));
     if (src) memcpy(_vSparseData.data(), src, dataLength * sizeof(T));   // (no values: a Boolean set, whose kernels never read them)
     memcpy(_vSparseIndex.data(), srcSparseIndex, dataLength * sizeof(uint32_t));
+    _bSparseHostStale = false;
+}
+
+// The device arrays hold the latest load; the host vectors are brought up to date from them (everything queued is waited for).
+template <typename T> void NNDataSet<T>::SyncSparseHostCopy()
+{
+    if (!_bSparseHostStale) return;
+    _bSparseHostStale = false;
+    dsxFatal(dsx_sync(), "NNDataSet::SyncSparseHostCopy");
+    auto fetch = [](auto& vec, auto& buf) {
+        if (!buf || vec.empty()) return;
+        const size_t n = std::min<size_t>(vec.size(), buf->_length);
+        dsxFatal(dsx_memcpy_d2h(vec.data(), buf->_pDevData, n * sizeof(vec[0])), "NNDataSet::SyncSparseHostCopy");
+    };
+    fetch(_vSparseStart, _pbSparseStart);
+    fetch(_vSparseEnd, _pbSparseEnd);
+    fetch(_vSparseIndex, _pbSparseIndex);
+    if (!(_attributes & NNDataSetEnums::Attributes::Boolean)) fetch(_vSparseData, _pbSparseData);
 }
 
 template <typename T>
@@ -215,10 +234,10 @@ void NNDataSet<T>::LoadSparseData(const uint64_t* srcSparseStart, const uint64_t
     if (!(_attributes & NNDataSetEnums::Attributes::Sparse)) throw std::runtime_error("Cannot set sparse data on a non sparse NNDataSet");
     checkSparseLoad(srcSparseStart[0], srcSparseEnd[_uniqueExamples - 1]);
     if (!srcSparseData && !(_attributes & NNDataSetEnums::Attributes::Boolean)) throw std::runtime_error("NNDataSet::LoadSparseData: no values for a data set that is not Boolean");
-    // The device copies are queued first, straight from the caller's arrays and only as long as this batch's data (the
-    // buffers may be larger): the device starts on them while the host shadows below are still being filled.  They go to the
-    // set of device arrays that the kernels in flight do not read, on the lane the next PredictBatch will use, and are
-    // ordered against that lane only.
+    // The device copies are queued straight from the caller's arrays and only as long as this batch's data (the buffers may
+    // be larger).  They go to the set of device arrays that the kernels in flight do not read, on the lane the next
+    // PredictBatch will use, and are ordered against that lane only.  The host vectors are not filled here (that copy is a
+    // tenth of a request's round trip, and the forward pass never reads them): they are marked stale instead.
     const uint64_t dataLength = srcSparseEnd[_uniqueExamples - 1];
     const bool direct = _pbSparseStart && _pbSparseEnd && _pbSparseIndex && _pbSparseStart->_length >= _uniqueExamples &&
                         _pbSparseIndex->_length >= dataLength && (!_pbSparseData || _pbSparseData->_length >= dataLength);
@@ -256,19 +275,23 @@ void NNDataSet<T>::LoadSparseData(const uint64_t* srcSparseStart, const uint64_t
         // batch of 1024 instead of 102.)
         if (!_sparseSet._uploaded) dsxFatal(dsx_marker_create(&_sparseSet._uploaded), "NNDataSet::LoadSparseData");
         else dsxFatal(dsx_marker_wait(_sparseSet._uploaded), "NNDataSet::LoadSparseData");
-        dsxFatal(dsx_memcpy_h2d_unordered(_pbSparseStart->_pDevData, srcSparseStart, _uniqueExamples * sizeof(uint64_t)), "NNDataSet::LoadSparseData");
-        dsxFatal(dsx_memcpy_h2d_unordered(_pbSparseEnd->_pDevData, srcSparseEnd, _uniqueExamples * sizeof(uint64_t)), "NNDataSet::LoadSparseData");
-        dsxFatal(dsx_memcpy_h2d_unordered(_pbSparseIndex->_pDevData, srcSparseIndex, dataLength * sizeof(uint32_t)), "NNDataSet::LoadSparseData");
-        if (_pbSparseData && srcSparseData)
-            dsxFatal(dsx_memcpy_h2d_unordered(_pbSparseData->_pDevData, srcSparseData, dataLength * sizeof(T)), "NNDataSet::LoadSparseData");
+        {
+            const bool values = _pbSparseData && srcSparseData;
+            void* const dst[4] = {_pbSparseStart->_pDevData, _pbSparseEnd->_pDevData, _pbSparseIndex->_pDevData, values ? _pbSparseData->_pDevData : NULL};
+            const void* const src[4] = {srcSparseStart, srcSparseEnd, srcSparseIndex, srcSparseData};
+            const size_t bytes[4] = {_uniqueExamples * sizeof(uint64_t), _uniqueExamples * sizeof(uint64_t), dataLength * sizeof(uint32_t), dataLength * sizeof(T)};
+            dsxFatal(dsx_memcpy_h2d_unordered_many(values ? 4 : 3, dst, src, bytes), "NNDataSet::LoadSparseData");
+        }
         _sparseSet._uploadLane = target;
         _sparseSet._readLanes = 0;
         _sparseSet._orderedLanes = 1u << target;
         dsxFatal(dsx_marker_record(_sparseSet._uploaded), "NNDataSet::LoadSparseData");
         if (target != selected) dsxFatal(dsx_set_lane(selected), "NNDataSet::LoadSparseData");
+        _bSparseHostStale = true;   // (the host vectors are fetched back when something reads them: SyncSparseHostCopy)
+        return;
     }
     CopySparseData(srcSparseStart, srcSparseEnd, srcSparseData, srcSparseIndex);
-    if (!direct) uploadSparse();
+    uploadSparse();
 }
 
 template <typename T>
@@ -341,6 +364,7 @@ template <typename T> uint64_t NNDataSet<T>::GetSparseDataPoints(uint32_t n)
 {
     if (!(_attributes & NNDataSetEnums::Sparse)) fatalAccess("NNDataSet::GetSparseDataPoints: attempt to read sparse data from non-sparse data set.");
     if (n >= _examples) fatalAccess("NNDataSet::GetSparseDataPoints: illegal example index.");
+    SyncSparseHostCopy();
     if (_bIndexed) n = _vIndex[n];
     return _vSparseEnd[n] - _vSparseStart[n];
 }
@@ -349,6 +373,7 @@ template <typename T> uint32_t NNDataSet<T>::GetSparseIndex(uint32_t n, uint32_t
 {
     if (!(_attributes & NNDataSetEnums::Sparse)) fatalAccess("NNDataSet::GetSparseIndex: attempt to read sparse data from non-sparse data set.");
     if (n >= _examples) fatalAccess("NNDataSet::GetSparseIndex: illegal example index.");
+    SyncSparseHostCopy();
     if (_bIndexed) n = _vIndex[n];
     if (i >= _vSparseEnd[n] - _vSparseStart[n]) fatalAccess("NNDataSet::GetSparseIndex: Sparse index out of range.");
     return _vSparseIndex[_vSparseStart[n] + i];
@@ -358,6 +383,7 @@ template <typename T> bool NNDataSet<T>::SetSparseIndex(uint32_t n, uint32_t i, 
 {
     if (!(_attributes & NNDataSetEnums::Sparse)) fatalAccess("NNDataSet::SetSparseIndex: attempt to read sparse data from non-sparse data set.");
     if (n >= _examples) fatalAccess("NNDataSet::SetSparseIndex: illegal example index.");
+    SyncSparseHostCopy();
     if (_bIndexed) n = _vIndex[n];
     if (i >= _vSparseEnd[n] - _vSparseStart[n]) fatalAccess("NNDataSet::SetSparseIndex: Sparse index out of range.");
     _vSparseIndex[_vSparseStart[n] + i] = v;
@@ -369,6 +395,7 @@ template <typename T> T NNDataSet<T>::GetSparseDataPoint(uint32_t n, uint32_t i)
 {
     if (!(_attributes & NNDataSetEnums::Sparse)) fatalAccess("NNDataSet::GetSparseDataPoint: attempt to read sparse data from non-sparse data set.");
     if (n >= _examples) fatalAccess("NNDataSet::GetSparseDataPoint: illegal example index.");
+    SyncSparseHostCopy();
     if (_bIndexed) n = _vIndex[n];
     if (i >= _vSparseEnd[n] - _vSparseStart[n]) fatalAccess("NNDataSet::GetSparseDataPoint: Sparse index out of range.");
     return _vSparseData[_vSparseStart[n] + i];
@@ -378,6 +405,7 @@ template <typename T> bool NNDataSet<T>::SetSparseDataPoint(uint32_t n, uint32_t
 {
     if (!(_attributes & NNDataSetEnums::Sparse)) fatalAccess("NNDataSet::SetSparseDataPoint: attempt to read sparse data from non-sparse data set.");
     if (n >= _examples) fatalAccess("NNDataSet::SetSparseDataPoint: illegal example index.");
+    SyncSparseHostCopy();
     if (_bIndexed) n = _vIndex[n];
     if (i >= _vSparseEnd[n] - _vSparseStart[n]) fatalAccess("NNDataSet::SetSparseDataPoint: Sparse index out of range.");
     _vSparseData[_vSparseStart[n] + i] = v;
@@ -391,6 +419,7 @@ template <typename T> bool NNDataSet<T>::SetSparseDataPoint(uint32_t n, uint32_t
 template <typename T> bool NNDataSet<T>::Shard(NNDataSetEnums::Sharding sharding)
 {
     if (sharding == _sharding) return true;
+    SyncSparseHostCopy();
     UnShard();
     _sharding = sharding;
     _minX = 0;
@@ -515,6 +544,7 @@ struct DataSetWriterHook {
 template <typename T> static void writeDataSet(ncc::Writer& nc, NNDataSet<T>& d, uint32_t n)
 {
     const string s = std::to_string(n);
+    d.SyncSparseHostCopy();
     nc.putAttString("name" + s, d._name);
     nc.putAttUInt("attributes" + s, d._attributes);
     nc.putAttUInt("kind" + s, 0);

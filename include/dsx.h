@@ -136,6 +136,9 @@ int dsx_memcpy_d2h_lane(int lane, void* host_dst, const void* device_src, size_t
  * dsx_lane_wait_other (the selected lane waits for everything queued so far on the other ones) before work on one lane
  * depends on what another lane wrote. */
 int dsx_memcpy_h2d_unordered(void* device_dst, const void* host_src, size_t bytes);
+/* Several arrays in one call (a batch's CSR arrays): what dsx_memcpy_h2d_unordered would do for each, with the small ones
+ * sharing a launch and the host staging one piece while the device copies the one before. */
+int dsx_memcpy_h2d_unordered_many(int count, void* const* device_dst, const void* const* host_src, const size_t* bytes);
 int dsx_lane_wait_other(void);
 /* A marker is a point in the selected lane's queue (no counterpart in the reference): dsx_marker_record places it after
  * everything queued so far on that lane, dsx_marker_wait blocks the calling host thread until the device has passed it (at

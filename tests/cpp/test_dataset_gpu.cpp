@@ -113,6 +113,8 @@ static void testLoadSparse()
     std::vector<long> ls(sparseStart.begin(), sparseStart.end()), le(sparseEnd.begin(), sparseEnd.end()), li(sparseIndex.begin(), sparseIndex.end());
     NNDataSet<NNFloat> viaLong(examples, sparseDensity, datasetDim, false);
     viaLong.LoadSparseData(ls.data(), le.data(), sparseData.data(), li.data());
+    dataset.SyncSparseHostCopy();   // (loaded straight to the device: the host vectors follow on request)
+    viaLong.SyncSparseHostCopy();
     CHECK(viaLong._vSparseIndex == dataset._vSparseIndex && viaLong._vSparseEnd == dataset._vSparseEnd);
 
     checkThrows<std::length_error>("sparse overflow", [&] {

@@ -80,6 +80,45 @@ def test_lanes_unordered_upload_and_explicit_wait(pkg, dsx, rng):
         pkg.check(dsx.dsx_sync())
 
 
+def test_uploads_of_every_size_and_alignment_arrive_byte_for_byte(pkg, dsx, rng):
+    """Uploads go through pinned staging memory and a copy kernel in pieces of 128 KiB (16 bytes per lane, a byte tail), through
+    the copy engine when the destination is not 16-byte aligned or the array exceeds a staging slot (4 MiB).  Sizes on both
+    sides of every such boundary, destinations at odd offsets, and the several-arrays form: each byte must arrive, and the
+    bytes around a destination must stay as they were."""
+    room = (5 << 20) + 4096
+    dev = pkg.DeviceArray((room,), np.uint8)
+    sizes = [1, 3, 15, 16, 17, 255, 4096, (128 << 10) - 16, (128 << 10) - 1, 128 << 10, (128 << 10) + 1, (128 << 10) + 17,
+             (256 << 10) + 5, (1 << 20) + 123, 4 << 20, (4 << 20) + 1, (5 << 20) + 7]
+    for size in sizes:
+        for off in (0, 16, 4, 1):
+            say("upload size=%d offset=%d" % (size, off))
+            pkg.check(dsx.dsx_memset(dev.ptr, 0xA5, room))
+            x = rng.integers(0, 256, size=size, dtype=np.uint8)
+            pkg.check(dsx.dsx_memcpy_h2d(dev.ptr + 256 + off, x.ctypes.data, size))
+            got = dev.numpy()
+            assert np.array_equal(got[256 + off:256 + off + size], x), (size, off)
+            assert (got[:256 + off] == 0xA5).all() and (got[256 + off + size:] == 0xA5).all(), (size, off)
+    # several arrays in one call: sizes that share launches, cross piece boundaries, are empty, or are not multiples of 16
+    for lens in [(8192, 8192, 400000), (8, 0, 131072 - 8, 40), (100, 131000, 131072, 7), (300000, 4, 4, 300001)]:
+        say("upload many %s" % (lens,))
+        pkg.check(dsx.dsx_memset(dev.ptr, 0x5A, room))
+        xs = [rng.integers(0, 256, size=n, dtype=np.uint8) for n in lens]
+        at, offs = 512, []
+        for n in lens:
+            offs.append(at)
+            at += (n + 255) // 256 * 256 + 256
+        dst = (C.c_void_p * len(lens))(*[dev.ptr + o for o in offs])
+        src = (C.c_void_p * len(lens))(*[x.ctypes.data if x.size else None for x in xs])
+        nb = (C.c_size_t * len(lens))(*lens)
+        pkg.check(dsx.dsx_memcpy_h2d_unordered_many(len(lens), dst, src, nb))
+        got = dev.numpy()
+        want = np.full(room, 0x5A, np.uint8)
+        for o, x in zip(offs, xs):
+            want[o:o + x.size] = x
+        assert np.array_equal(got, want), lens
+    assert dsx.dsx_memcpy_h2d_unordered_many(2, dst, None, nb) == -1
+
+
 def test_bad_arguments_are_rejected(pkg, dsx):
     a = pkg.DeviceArray((4, 8), np.float32)
     k = pkg.DeviceArray((4, 8), np.float32)
