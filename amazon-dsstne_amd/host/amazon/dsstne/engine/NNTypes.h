@@ -204,6 +204,8 @@ public:
 private:
     void checkSparseLoad(const uint64_t start0, const uint64_t dataLength) const;
     void uploadSparse();
+    bool uploadSparseDirect(const uint64_t* srcSparseStart, const uint64_t* srcSparseEnd, const void* srcSparseData,
+                            const uint32_t* srcSparseIndex);
 };
 
 // Dataset files (same attribute and variable names as the reference writes, engine/NNTypes.cpp:1081-1358).

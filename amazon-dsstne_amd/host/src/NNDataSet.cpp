@@ -227,21 +227,18 @@ template <typename T> void NNDataSet<T>::SyncSparseHostCopy()
     if (!(_attributes & NNDataSetEnums::Attributes::Boolean)) fetch(_vSparseData, _pbSparseData);
 }
 
+// Queues the copies of one batch's arrays to the device, only as long as the batch's data (the buffers may be larger).  They go
+// to the set of device arrays that the kernels in flight do not read, on the lane the next PredictBatch will use, and are
+// ordered against that lane only.  False (and nothing done) when the device arrays are missing or too small.
 template <typename T>
-void NNDataSet<T>::LoadSparseData(const uint64_t* srcSparseStart, const uint64_t* srcSparseEnd, const void* srcSparseData,
-                                  const uint32_t* srcSparseIndex)
+bool NNDataSet<T>::uploadSparseDirect(const uint64_t* srcSparseStart, const uint64_t* srcSparseEnd, const void* srcSparseData,
+                                      const uint32_t* srcSparseIndex)
 {
-    if (!(_attributes & NNDataSetEnums::Attributes::Sparse)) throw std::runtime_error("Cannot set sparse data on a non sparse NNDataSet");
-    checkSparseLoad(srcSparseStart[0], srcSparseEnd[_uniqueExamples - 1]);
-    if (!srcSparseData && !(_attributes & NNDataSetEnums::Attributes::Boolean)) throw std::runtime_error("NNDataSet::LoadSparseData: no values for a data set that is not Boolean");
-    // The device copies are queued straight from the caller's arrays and only as long as this batch's data (the buffers may
-    // be larger).  They go to the set of device arrays that the kernels in flight do not read, on the lane the next
-    // PredictBatch will use, and are ordered against that lane only.  The host vectors are not filled here (that copy is a
-    // tenth of a request's round trip, and the forward pass never reads them): they are marked stale instead.
     const uint64_t dataLength = srcSparseEnd[_uniqueExamples - 1];
     const bool direct = _pbSparseStart && _pbSparseEnd && _pbSparseIndex && _pbSparseStart->_length >= _uniqueExamples &&
                         _pbSparseIndex->_length >= dataLength && (!_pbSparseData || _pbSparseData->_length >= dataLength);
-    if (direct) {
+    if (!direct) return false;
+    {
         const int selected = dsx_get_lane();
         const int target = (s_nextLane >= 0 && s_nextLane < DSX_MAX_LANES) ? s_nextLane : 0;
         if (target != _sparseLane) {   // park the arrays of the lane that loaded last, take out the target lane's
@@ -287,7 +284,21 @@ void NNDataSet<T>::LoadSparseData(const uint64_t* srcSparseStart, const uint64_t
         _sparseSet._orderedLanes = 1u << target;
         dsxFatal(dsx_marker_record(_sparseSet._uploaded), "NNDataSet::LoadSparseData");
         if (target != selected) dsxFatal(dsx_set_lane(selected), "NNDataSet::LoadSparseData");
-        _bSparseHostStale = true;   // (the host vectors are fetched back when something reads them: SyncSparseHostCopy)
+    }
+    return true;
+}
+
+template <typename T>
+void NNDataSet<T>::LoadSparseData(const uint64_t* srcSparseStart, const uint64_t* srcSparseEnd, const void* srcSparseData,
+                                  const uint32_t* srcSparseIndex)
+{
+    if (!(_attributes & NNDataSetEnums::Attributes::Sparse)) throw std::runtime_error("Cannot set sparse data on a non sparse NNDataSet");
+    checkSparseLoad(srcSparseStart[0], srcSparseEnd[_uniqueExamples - 1]);
+    if (!srcSparseData && !(_attributes & NNDataSetEnums::Attributes::Boolean)) throw std::runtime_error("NNDataSet::LoadSparseData: no values for a data set that is not Boolean");
+    // Straight from the caller's arrays.  The host vectors are not filled here (that copy is a tenth of a request's round trip,
+    // and the forward pass never reads them): they are marked stale and fetched back when something reads them.
+    if (uploadSparseDirect(srcSparseStart, srcSparseEnd, srcSparseData, srcSparseIndex)) {
+        _bSparseHostStale = true;
         return;
     }
     CopySparseData(srcSparseStart, srcSparseEnd, srcSparseData, srcSparseIndex);
@@ -311,11 +322,13 @@ void NNDataSet<T>::CopySparseData(const long* srcSparseStart, const long* srcSpa
     }
 }
 
+// (the arrays of a language without unsigned types are converted into the host vectors, which then are the source)
 template <typename T>
 void NNDataSet<T>::LoadSparseData(const long* srcSparseStart, const long* srcSparseEnd, const void* srcSparseData, const long* srcSparseIndex)
 {
+    if (!srcSparseData && !(_attributes & NNDataSetEnums::Attributes::Boolean)) throw std::runtime_error("NNDataSet::LoadSparseData: no values for a data set that is not Boolean");
     CopySparseData(srcSparseStart, srcSparseEnd, srcSparseData, srcSparseIndex);
-    uploadSparse();
+    if (!uploadSparseDirect(_vSparseStart.data(), _vSparseEnd.data(), srcSparseData ? _vSparseData.data() : NULL, _vSparseIndex.data())) uploadSparse();
 }
 
 template <typename T> void NNDataSet<T>::LoadIndexedData(const uint32_t* srcIndexedData)
