@@ -890,31 +890,49 @@ __global__ __launch_bounds__(kTopkThreads, 4) void topk_guided_kernel(TopKArgs a
                 if (idx < a.nseg && (light ? sFiltMax[idx] != 0 : sFiltMax[idx] == mk[e])) tk[e] = 0;
             }
         }
-        const uint32_t tw = wave_kth_key<E>(tk, a.k);
-        uint32_t published = 0;   // wave-uniform
+        if (a.k <= 16) {   // the same for the whole workgroup
+            // Small k: the maxima go to LDS, one wavefront takes the largest of each lane's share (every 64th) and searches
+            // those 64.  The k-th largest of them is reached by k real items as well; it is the exact k-th maximum unless two of
+            // the k best share a lane (then it is the next one down, and a segment more is read) — one short search instead of
+            // a search per wavefront and a second one over what they publish.
 #pragma unroll
-        for (int e = 0; e < E; e++) {
-            const bool pub = tk[e] != 0 && tk[e] >= tw;
-            const uint64_t pm = __ballot(pub);
-            const uint32_t pos = published + __builtin_amdgcn_mbcnt_hi((uint32_t)(pm >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)pm, 0u));
-            if (pub && pos < a.k) sPrime[wave][pos] = tk[e];
-            published += (uint32_t)__popcll(pm);
-        }
-        __syncthreads();
-        // (one wavefront searches, the others wait: four workgroups share a CU, and what the searches of sixteen wavefronts
-        // cost is instruction issue, not latency)
-        if (wave == 0) {
-            uint32_t all[4];
-#pragma unroll
-            for (int n = 0; n < 4; n++) {
-                const uint32_t i = n * kWave + lane;
-                all[n] = (i < kTopkWaves * a.k) ? sPrime[i / a.k][i % a.k] : 0u;
+            for (int e = 0; e < E; e++) {
+                const uint32_t idx = e * kTopkThreads + threadIdx.x;
+                if (idx < a.nseg) sListKey[idx] = tk[e];   // (the list of segments is built later)
             }
-            uint32_t t;
-            if (a.k <= 16) t = wave_kth_key<1>(reinterpret_cast<const uint32_t(&)[1]>(all), a.k);
-            else if (a.k <= 32) t = wave_kth_key<2>(reinterpret_cast<const uint32_t(&)[2]>(all), a.k);
-            else t = wave_kth_key<4>(all, a.k);
-            if (lane == 0) sBound = t;
+            __syncthreads();
+            if (wave == 0) {
+                uint32_t best[1] = {0u};
+                for (uint32_t i = lane; i < a.nseg; i += kWave) best[0] = max(best[0], sListKey[i]);
+                const uint32_t t = wave_kth_key<1>(best, a.k);
+                if (lane == 0) sBound = t;
+            }
+        } else {
+            const uint32_t tw = wave_kth_key<E>(tk, a.k);
+            uint32_t published = 0;   // wave-uniform
+#pragma unroll
+            for (int e = 0; e < E; e++) {
+                const bool pub = tk[e] != 0 && tk[e] >= tw;
+                const uint64_t pm = __ballot(pub);
+                const uint32_t pos = published + __builtin_amdgcn_mbcnt_hi((uint32_t)(pm >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)pm, 0u));
+                if (pub && pos < a.k) sPrime[wave][pos] = tk[e];
+                published += (uint32_t)__popcll(pm);
+            }
+            __syncthreads();
+            // (one wavefront searches, the others wait: four workgroups share a CU, and what the searches of sixteen wavefronts
+            // cost is instruction issue, not latency)
+            if (wave == 0) {
+                uint32_t all[4];
+#pragma unroll
+                for (int n = 0; n < 4; n++) {
+                    const uint32_t i = n * kWave + lane;
+                    all[n] = (i < kTopkWaves * a.k) ? sPrime[i / a.k][i % a.k] : 0u;
+                }
+                uint32_t t;
+                if (a.k <= 32) t = wave_kth_key<2>(reinterpret_cast<const uint32_t(&)[2]>(all), a.k);
+                else t = wave_kth_key<4>(all, a.k);
+                if (lane == 0) sBound = t;
+            }
         }
         __syncthreads();
         const uint32_t t = sBound;
