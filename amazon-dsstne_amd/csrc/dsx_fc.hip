@@ -159,7 +159,10 @@ template <int MI, int NI, int BK, int XV, int WV, bool TRANS, int ACT, int CAND 
 __global__ __launch_bounds__(kFcThreads, (MI * NI >= 4) ? (CAND == 2 ? 3 : 4) : 2) void fc_gemm_kernel(FcArgs a)
 {
     constexpr int BM = 64 * MI, BN = 64 * NI;
-    constexpr int LDA = BM + 4, LDB = BN + 4;
+    // (X tiles 32 deep: the eight lanes that hold one row's 16-byte pieces store rows of sA that are 4 * LDA floats apart; with
+    // LDA = BM + 4 they fall on two LDS banks — a third of the LDS cycles of a 4,096 x 1,024 x 1,024 layer were bank conflicts —,
+    // with an odd LDA on eight)
+    constexpr int LDA = BM + ((BK == 32 && XV == 4) ? 1 : 4), LDB = BN + 4;
     constexpr int A_ELEMS = BM * BK / kFcThreads;   // floats of the X tile per lane
     constexpr int B_ELEMS = BN * BK / kFcThreads;
     __shared__ float sA[2][BK][LDA];
