@@ -554,7 +554,8 @@ def test_topk_guided_filtered(pkg, dsx, orc, rng, batch, width, k, maxnnz, with_
 
 
 @pytest.mark.parametrize("batch,width,k,share", [(64, 27278, 10, 0.13), (64, 27278, 10, 0.004), (16, 27278, 50, 0.4), (3, 300000, 10, 0.13),
-                                                  (9, 27278, 100, 0.13), (5, 70000, 200, 0.05)])
+                                                  (9, 27278, 100, 0.13), (5, 70000, 200, 0.05), (6, 120000, 10, 0.05), (6, 60000, 16, 0.3),
+                                                  (7, 3000, 5, 0.5)])
 @pytest.mark.parametrize("filtered", [False, True])
 def test_topk_saturated_rows_scan_and_guided(pkg, dsx, orc, rng, batch, width, k, share, filtered):
     """Saturated sigmoids: a share of every row is exactly 1.0, the top of the list is ties all the way down and the lowest
