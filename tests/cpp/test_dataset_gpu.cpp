@@ -1,6 +1,9 @@
 // Dataset and buffer behaviour on the device, following the assertions of the reference's own unit tests
 // tst/amazon/dsstne/engine/TestNNDataSet.cpp:58-349 and TestGpuBuffer.cpp:31-68.
+#include <cstdio>
+#include <cstdlib>
 #include <stdexcept>
+#include <string>
 
 #include "amazon/dsstne/engine/NNTypes.h"
 #include "check.h"
@@ -116,6 +119,39 @@ static void testLoadSparse()
     dataset.SyncSparseHostCopy();   // (loaded straight to the device: the host vectors follow on request)
     viaLong.SyncSparseHostCopy();
     CHECK(viaLong._vSparseIndex == dataset._vSparseIndex && viaLong._vSparseEnd == dataset._vSparseEnd);
+
+    // A load that went straight to the device leaves the host vectors stale until something reads them: a second load with
+    // other numbers, then SaveNetCDF (which reads them) and LoadNetCDF must give back the second load, not the first.
+    {
+        NNDataSet<NNFloat> second(examples, sparseDensity, datasetDim, false);
+        second._name = "second";
+        second.LoadSparseData(sparseStart.data(), sparseEnd.data(), sparseData.data(), sparseIndex.data());
+        std::vector<NNFloat> data2(sparseData);
+        std::vector<uint32_t> index2(sparseIndex);
+        for (size_t i = 0; i < data2.size(); i++) {
+            data2[i] = (NNFloat)(1000 + i);
+            index2[i] = (uint32_t)((i * 7) % 128);
+        }
+        second.LoadSparseData(sparseStart.data(), sparseEnd.data(), data2.data(), index2.data());
+        CHECK(second._bSparseHostStale);
+        const char* tmp = getenv("TMPDIR");
+        const std::string file = std::string(tmp && tmp[0] ? tmp : "/tmp") + "/dsx_stale_host_copy.nc";
+        CHECK(second.SaveNetCDF(file));
+        CHECK(!second._bSparseHostStale);
+        std::vector<NNDataSetBase*> back2 = LoadNetCDF(file);
+        CHECK(back2.size() == 1);
+        if (back2.size() == 1) {
+            NNDataSet<NNFloat>* r = dynamic_cast<NNDataSet<NNFloat>*>(back2[0]);
+            CHECK(r != NULL);
+            if (r) {
+                CHECK(std::equal(index2.begin(), index2.end(), r->_vSparseIndex.begin()));
+                CHECK(std::equal(data2.begin(), data2.end(), r->_vSparseData.begin()));
+                CHECK(r->_vSparseEnd == std::vector<uint64_t>(sparseEnd.begin(), sparseEnd.end()));
+            }
+        }
+        for (auto* d : back2) delete d;
+        remove(file.c_str());
+    }
 
     checkThrows<std::length_error>("sparse overflow", [&] {
         NNDataSet<NNFloat> d(examples, sparseDensity, datasetDim, false);
